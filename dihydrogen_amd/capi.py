@@ -1,0 +1,128 @@
+"""ctypes binding of ``libh2x.so`` (the C ABI declared in ``include/h2x.h``).
+
+The library is loaded from this package directory.  There is no fallback: if
+the shared object is missing or a call fails, an exception is raised.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import POINTER, c_double, c_int, c_int32, c_int64, c_size_t, c_void_p
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libh2x.so")
+
+H2X_MAX_DIMS = 6
+F32, F64 = 0, 1
+LHS, RHS = 0, 1
+HALO_ID, HALO_SUM, HALO_MAX, HALO_MIN = 0, 1, 2, 3
+
+ABI_VERSION = 1
+
+
+class H2XError(RuntimeError):
+    pass
+
+
+class HaloFace(ctypes.Structure):
+    """struct h2x_halo_face"""
+    _fields_ = [
+        ("tensor", c_void_p),
+        ("buffer", c_void_p),
+        ("real_shape", c_int64 * H2X_MAX_DIMS),
+        ("num_dims", c_int32),
+        ("dim", c_int32),
+        ("side", c_int32),
+        ("width", c_int32),
+        ("inner", c_int32),
+        ("is_pack", c_int32),
+        ("op", c_int32),
+        ("reserved", c_int32),
+    ]
+
+
+class ShuffleGeometry(ctypes.Structure):
+    """struct h2x_shuffle_geometry"""
+    _fields_ = [
+        ("num_dims", c_int32),
+        ("elem_size", c_int32),
+        ("local_shape", c_int64 * H2X_MAX_DIMS),
+        ("strides", c_int64 * H2X_MAX_DIMS),
+        ("peer_locale_shape", c_int64 * H2X_MAX_DIMS),
+        ("rank_limits", POINTER(c_int32)),
+        ("displs", POINTER(c_int32)),
+    ]
+
+
+# name -> (restype, argtypes); every symbol include/h2x.h declares.
+SIGNATURES = {
+    "h2x_abi_version": (c_int, []),
+    "h2x_status_string": (ctypes.c_char_p, [c_int]),
+    "h2x_bn_workspace_bytes": (c_size_t, [c_int]),
+    "h2x_bn_workspace_init": (c_int, [c_void_p, c_int, c_void_p]),
+    "h2x_bn_channel_sums_and_sqsums": (c_int, [c_int, c_int, c_int, c_size_t, c_size_t, c_void_p,
+                                               c_void_p, c_void_p, c_void_p, c_void_p]),
+    "h2x_bn_sums_to_statistics": (c_int, [c_int, c_int, c_size_t, c_double, c_void_p, c_void_p,
+                                          c_void_p, c_void_p, c_void_p]),
+    "h2x_bn_batch_normalization": (c_int, [c_int, c_int, c_int, c_size_t, c_size_t, c_size_t,
+                                           c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                           c_void_p, c_double, c_void_p]),
+    "h2x_bn_backprop1": (c_int, [c_int, c_int, c_int, c_size_t, c_size_t, c_size_t, c_void_p,
+                                 c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                 c_void_p, c_void_p, c_double, c_void_p, c_void_p]),
+    "h2x_bn_backprop2": (c_int, [c_int, c_int, c_int, c_size_t, c_size_t, c_size_t, c_size_t,
+                                 c_size_t, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                 c_void_p, c_void_p, c_void_p, c_double, c_void_p]),
+    "h2x_softmax_channel_forward": (c_int, [c_int, c_int, c_int, c_size_t, c_void_p, c_void_p,
+                                            c_void_p]),
+    "h2x_softmax_channel_backward": (c_int, [c_int, c_int, c_int, c_size_t, c_void_p, c_void_p,
+                                             c_void_p, c_void_p]),
+    "h2x_halo_size": (c_size_t, [c_int, POINTER(c_int64), c_int, c_int]),
+    "h2x_halo_pack_or_unpack": (c_int, [c_int, c_void_p, c_int, POINTER(c_int64), c_int, c_int,
+                                        c_int, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "h2x_halo_pack_or_unpack_batched": (c_int, [c_int, POINTER(HaloFace), c_int, c_void_p]),
+    "h2x_halo_clear": (c_int, [c_int, c_void_p, c_int, POINTER(c_int64), c_int, c_int, c_void_p]),
+    "h2x_shuffle_plan_create": (c_int, [POINTER(ShuffleGeometry), POINTER(c_void_p)]),
+    "h2x_shuffle_plan_destroy": (c_int, [c_void_p]),
+    "h2x_shuffle_pack": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p]),
+    "h2x_shuffle_unpack": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p]),
+    "h2x_shuffle_pack_batched": (c_int, [POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p),
+                                         c_int, c_void_p]),
+    "h2x_shuffle_unpack_batched": (c_int, [POINTER(c_void_p), POINTER(c_void_p),
+                                           POINTER(c_void_p), c_int, c_void_p]),
+}
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    """Loads libh2x.so and checks its ABI version.  Raises if it is absent."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise H2XError(
+            f"{LIB_PATH} is missing: build it with `make -C dihydrogen_amd/csrc` "
+            "(or __graft_entry__.build()); there is no fallback path")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (restype, argtypes) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if the symbol is not exported
+        fn.restype = restype
+        fn.argtypes = argtypes
+    if lib.h2x_abi_version() != ABI_VERSION:
+        raise H2XError(f"libh2x.so has ABI {lib.h2x_abi_version()}, binding expects {ABI_VERSION}")
+    _lib = lib
+    return lib
+
+
+def check(status: int, what: str = "") -> None:
+    if status != 0:
+        msg = load().h2x_status_string(status).decode()
+        raise H2XError(f"{what or 'h2x call'} failed: {msg} ({status})")
+
+
+def i64_array(values):
+    arr = (c_int64 * H2X_MAX_DIMS)()
+    for i, v in enumerate(values):
+        arr[i] = int(v)
+    return arr

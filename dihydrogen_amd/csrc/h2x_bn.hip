@@ -1,0 +1,806 @@
+// Channel-wise batch-normalisation kernels for gfx950 and their C entry points.
+//
+// Layout: element (n, c, i) of a tensor lives at base[(n*C + c)*real + i],
+// i < spatial -- the geometry of the reference's optimised kernels
+// (legacy/src/dnn_backend/batchnorm.cu:134-190).  Every kernel is a pure HBM
+// stream: 16-byte loads when the geometry allows, several loads in flight per
+// lane, per-channel parameters fetched once per workgroup.
+//
+// Reductions (forward sums, backward sums) cut every channel into contiguous
+// chunks, one workgroup per chunk.  A thread accumulates in fp64, the
+// workgroup combines lanes with DPP permutes and waves through LDS, and writes
+// one fp64 partial per sum.  The workgroup that finishes last for a channel
+// (per-channel completion counter) adds the partials in index order and writes
+// the channel's result.  All orders are fixed, so results are deterministic;
+// the reference's float atomics are not (batchnorm.cu:127-131,1047-1053).
+#include "h2x_device.hpp"
+
+#include <algorithm>
+
+namespace h2x
+{
+namespace
+{
+
+constexpr int kUnroll = 4;
+// Upper bound on workgroups per channel; sizes the workspace.
+constexpr int kTargetGroups = 8192;
+constexpr int kMinGroupsPerChannel = 8;
+constexpr int kMaxGroupsPerChannel = 2048;
+constexpr int kMaxSums = 4;
+
+int max_groups_per_channel(int num_channels)
+{
+    const int g = (kTargetGroups + num_channels - 1) / std::max(num_channels, 1);
+    return std::min(std::max(g, kMinGroupsPerChannel), kMaxGroupsPerChannel);
+}
+
+size_t counters_offset(int num_channels)
+{
+    return static_cast<size_t>(num_channels) * max_groups_per_channel(num_channels) * kMaxSums
+           * sizeof(double);
+}
+
+// How one (sample, channel) segment of `spatial` elements is cut into chunks.
+struct Chunking
+{
+    size_t chunk;        // elements per workgroup, multiple of the tile
+    int chunks_per_seg;  // workgroups per (sample, channel) segment
+};
+
+// `segments`: segments that contribute workgroups to one scheduling unit
+// (num_samples for a per-channel reduction, N*C for an elementwise pass);
+// `budget`: workgroups wanted (reduction: cap per channel; elementwise: total).
+Chunking make_chunking(size_t spatial, size_t segments, size_t budget, size_t tile, size_t min_chunk)
+{
+    Chunking c;
+    size_t per_seg = std::max<size_t>(budget / std::max<size_t>(segments, 1), 1);
+    size_t chunk = (spatial + per_seg - 1) / per_seg;
+    chunk = std::max(chunk, min_chunk);
+    chunk = (chunk + tile - 1) / tile * tile;
+    c.chunk = chunk;
+    c.chunks_per_seg = static_cast<int>((spatial + chunk - 1) / chunk);
+    if (c.chunks_per_seg < 1)
+        c.chunks_per_seg = 1;
+    return c;
+}
+
+#define H2X_RETURN_IF_ERROR(expr)                                                                  \
+    do                                                                                             \
+    {                                                                                              \
+        int h2x_err_ = (expr);                                                                     \
+        if (h2x_err_ != 0)                                                                         \
+            return h2x_err_;                                                                       \
+    } while (0)
+
+template <typename T, int VEC>
+__device__ __forceinline__ void load_vec(const T* p, T (&r)[VEC])
+{
+    if constexpr (VEC == 1)
+    {
+        r[0] = *p;
+    }
+    else
+    {
+        typedef T V __attribute__((ext_vector_type(VEC)));
+        const V t = *reinterpret_cast<const V*>(p);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j)
+            r[j] = t[j];
+    }
+}
+
+template <typename T, int VEC>
+__device__ __forceinline__ void store_vec(T* p, const T (&r)[VEC])
+{
+    if constexpr (VEC == 1)
+    {
+        *p = r[0];
+    }
+    else
+    {
+        typedef T V __attribute__((ext_vector_type(VEC)));
+        V t;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j)
+            t[j] = r[j];
+        *reinterpret_cast<V*>(p) = t;
+    }
+}
+
+__device__ __forceinline__ float fma_t(float a, float b, float c)
+{
+    return __builtin_fmaf(a, b, c);
+}
+__device__ __forceinline__ double fma_t(double a, double b, double c)
+{
+    return __builtin_fma(a, b, c);
+}
+__device__ __forceinline__ float inv_sqrt_t(float v)
+{
+    return 1.0f / __builtin_sqrtf(v);
+}
+__device__ __forceinline__ double inv_sqrt_t(double v)
+{
+    return 1.0 / __builtin_sqrt(v);
+}
+
+// Combines the K per-thread sums of a workgroup and, in the workgroup that
+// completes a channel, the partials of all workgroups of that channel.
+// Returns true in that last workgroup, with the channel totals in acc[].
+template <int K>
+__device__ __forceinline__ bool finish_channel(double (&acc)[K], double* partials,
+                                               unsigned int* counters, int channel,
+                                               int groups_per_channel_max)
+{
+    __shared__ double lds[K * kWavesPerBlock];
+    __shared__ int is_last;
+    block_sum<K>(acc, lds);
+    const unsigned int groups = gridDim.x;
+    if (groups == 1)
+        return true;
+    double* mine = partials + (static_cast<size_t>(channel) * groups_per_channel_max) * K;
+    if (threadIdx.x == 0)
+    {
+#pragma unroll
+        for (int k = 0; k < K; ++k)
+            __hip_atomic_store(mine + static_cast<size_t>(blockIdx.x) * K + k, acc[k],
+                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __threadfence();
+        const unsigned int done = atomicAdd(counters + channel, 1u);
+        is_last = (done == groups - 1) ? 1 : 0;
+    }
+    __syncthreads();
+    if (!is_last)
+        return false;
+    __threadfence();
+    double t[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k)
+        t[k] = 0.0;
+    for (unsigned int g = threadIdx.x; g < groups; g += kBlockSize)
+    {
+#pragma unroll
+        for (int k = 0; k < K; ++k)
+            t[k] += __hip_atomic_load(mine + static_cast<size_t>(g) * K + k, __ATOMIC_RELAXED,
+                                      __HIP_MEMORY_SCOPE_AGENT);
+    }
+    block_sum<K>(t, lds);
+#pragma unroll
+    for (int k = 0; k < K; ++k)
+        acc[k] = t[k];
+    if (threadIdx.x == 0)
+        counters[channel] = 0u; // ready for the next launch on this workspace
+    return true;
+}
+
+// ---- forward: sums and sums of squares --------------------------------------
+// Replaces channel_sums_and_sqsums_opt_kernel, batchnorm.cu:92-132.
+template <typename T, int VEC>
+__global__ __launch_bounds__(kBlockSize) void bn_sums_kernel(
+    const T* __restrict__ x, T* __restrict__ sums, T* __restrict__ sqsums, double* partials,
+    unsigned int* counters, int num_channels, size_t spatial, size_t spatial_real, size_t chunk,
+    int chunks_per_seg, unsigned int num_units, int groups_per_channel_max)
+{
+    const int c = blockIdx.y;
+    constexpr size_t kStride = static_cast<size_t>(kBlockSize) * VEC;
+    constexpr size_t kTile = kStride * kUnroll;
+    double acc[2] = {0.0, 0.0};
+    // unit = (sample, chunk); a workgroup takes units blockIdx.x, +gridDim.x, ...
+    for (unsigned int unit = blockIdx.x; unit < num_units; unit += gridDim.x)
+    {
+    const int n = unit / chunks_per_seg;
+    const int k = unit - n * chunks_per_seg;
+    const size_t begin = static_cast<size_t>(k) * chunk;
+    const size_t end = begin + chunk < spatial ? begin + chunk : spatial;
+    const T* p = x + (static_cast<size_t>(n) * num_channels + c) * spatial_real;
+    size_t tile = begin;
+    for (; tile + kTile <= end; tile += kTile)
+    {
+        T v[kUnroll][VEC];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+            load_vec<T, VEC>(p + tile + u * kStride + threadIdx.x * VEC, v[u]);
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+            for (int j = 0; j < VEC; ++j)
+            {
+                const double d = static_cast<double>(v[u][j]);
+                acc[0] += d;
+                if constexpr (sizeof(T) == 4)
+                    acc[1] = __builtin_fma(d, d, acc[1]); // product of two floats is exact
+                else
+                    acc[1] += d * d;
+            }
+    }
+    for (size_t i = tile + threadIdx.x * VEC; i < end; i += kStride)
+    {
+        T v[VEC];
+        load_vec<T, VEC>(p + i, v);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j)
+        {
+            const double d = static_cast<double>(v[j]);
+            acc[0] += d;
+            if constexpr (sizeof(T) == 4)
+                acc[1] = __builtin_fma(d, d, acc[1]);
+            else
+                acc[1] += d * d;
+        }
+    }
+    }
+    if (finish_channel<2>(acc, partials, counters, c, groups_per_channel_max) && threadIdx.x == 0)
+    {
+        sums[c] = static_cast<T>(acc[0]);
+        sqsums[c] = static_cast<T>(acc[1]);
+    }
+}
+
+template <typename T>
+__global__ void fill_kernel(T* p, size_t n, T value)
+{
+    for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < n;
+         i += static_cast<size_t>(gridDim.x) * blockDim.x)
+        p[i] = value;
+}
+
+// ---- forward: sums -> mean / unbiased variance / running statistics ---------
+// Replaces sums_to_statistics_functor, batchnorm.cu:288-346.
+template <typename T>
+__global__ void bn_statistics_kernel(int num_channels, size_t num_per_sum, T decay, T* mean,
+                                     T* var, T* running_mean, T* running_var)
+{
+    const T n = static_cast<T>(num_per_sum);
+    for (int c = blockIdx.x * blockDim.x + threadIdx.x; c < num_channels;
+         c += gridDim.x * blockDim.x)
+    {
+        if (num_per_sum == 0)
+        {
+            var[c] = T(1);
+            continue;
+        }
+        const T m = mean[c] / n;
+        const T sqmean = var[c] / n;
+        T v = fma_t(-m, m, sqmean);
+        v = v > T(0) ? v : T(0);
+        v *= n / (n - T(1));
+        mean[c] = m;
+        var[c] = v;
+        running_mean[c] = fma_t(decay, running_mean[c], (T(1) - decay) * m);
+        running_var[c] = fma_t(decay, running_var[c], (T(1) - decay) * v);
+    }
+}
+
+// ---- forward: normalise ------------------------------------------------------
+// Replaces batch_normalization_opt_kernel, batchnorm.cu:420-455.
+template <typename T, int VEC>
+__global__ __launch_bounds__(kBlockSize) void bn_apply_kernel(
+    const T* __restrict__ x, const T* __restrict__ mean, const T* __restrict__ var,
+    const T* __restrict__ scale, const T* __restrict__ bias, T* __restrict__ y, T epsilon,
+    int num_channels, size_t spatial, size_t x_real, size_t y_real, size_t chunk,
+    int chunks_per_seg)
+{
+    const size_t seg = blockIdx.x / chunks_per_seg;
+    const int k = blockIdx.x - seg * chunks_per_seg;
+    const int c = seg % num_channels;
+    const T m = mean[c];
+    const T inv_stdev = inv_sqrt_t(var[c] + epsilon);
+    const T sc = scale[c];
+    const T bi = bias[c];
+    const size_t begin = static_cast<size_t>(k) * chunk;
+    const size_t end = begin + chunk < spatial ? begin + chunk : spatial;
+    const T* xp = x + seg * x_real;
+    T* yp = y + seg * y_real;
+
+    constexpr size_t kStride = static_cast<size_t>(kBlockSize) * VEC;
+    constexpr size_t kTile = kStride * kUnroll;
+    size_t tile = begin;
+    for (; tile + kTile <= end; tile += kTile)
+    {
+        T v[kUnroll][VEC];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+            load_vec<T, VEC>(xp + tile + u * kStride + threadIdx.x * VEC, v[u]);
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+        {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j)
+                v[u][j] = fma_t((v[u][j] - m) * inv_stdev, sc, bi);
+            store_vec<T, VEC>(yp + tile + u * kStride + threadIdx.x * VEC, v[u]);
+        }
+    }
+    for (size_t i = tile + threadIdx.x * VEC; i < end; i += kStride)
+    {
+        T v[VEC];
+        load_vec<T, VEC>(xp + i, v);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j)
+            v[j] = fma_t((v[j] - m) * inv_stdev, sc, bi);
+        store_vec<T, VEC>(yp + i, v);
+    }
+}
+
+// ---- backward: per-channel sums ----------------------------------------------
+// Replaces backprop1_opt_kernel, batchnorm.cu:982-1054.
+template <typename T, int VEC>
+__global__ __launch_bounds__(kBlockSize) void bn_backprop1_kernel(
+    const T* __restrict__ x, const T* __restrict__ dy, const T* __restrict__ mean,
+    const T* __restrict__ var, const T* __restrict__ scale, T* __restrict__ dscale,
+    T* __restrict__ dbias, T* __restrict__ dmean, T* __restrict__ dvar, T epsilon,
+    double* partials, unsigned int* counters, int num_channels, size_t spatial, size_t x_real,
+    size_t dy_real, size_t chunk, int chunks_per_seg, unsigned int num_units,
+    int groups_per_channel_max)
+{
+    const int c = blockIdx.y;
+    const T m = mean[c];
+    const T sc = scale[c];
+    const T inv_stdev = inv_sqrt_t(var[c] + epsilon);
+    const T dvar_factor = inv_stdev * inv_stdev * inv_stdev / T(2);
+    const double neg_inv = -static_cast<double>(inv_stdev);
+    const double neg_fac = -static_cast<double>(dvar_factor);
+
+    constexpr size_t kStride = static_cast<size_t>(kBlockSize) * VEC;
+    constexpr int kUnroll2 = kUnroll / 2; // two streams: same bytes in flight
+    constexpr size_t kTile = kStride * kUnroll2;
+    double acc[4] = {0.0, 0.0, 0.0, 0.0};
+
+    auto accumulate = [&](T xv, T dv) {
+        const T xm = xv - m;
+        const T xhat = xm * inv_stdev;
+        const T dxhat = dv * sc;
+        const T t = dxhat * xm;
+        const double dd = static_cast<double>(dv);
+        acc[0] = __builtin_fma(dd, static_cast<double>(xhat), acc[0]);
+        acc[1] += dd;
+        acc[2] = __builtin_fma(static_cast<double>(dxhat), neg_inv, acc[2]);
+        acc[3] = __builtin_fma(static_cast<double>(t), neg_fac, acc[3]);
+    };
+
+    for (unsigned int unit = blockIdx.x; unit < num_units; unit += gridDim.x)
+    {
+        const int n = unit / chunks_per_seg;
+        const int k = unit - n * chunks_per_seg;
+        const size_t begin = static_cast<size_t>(k) * chunk;
+        const size_t end = begin + chunk < spatial ? begin + chunk : spatial;
+        const size_t seg = static_cast<size_t>(n) * num_channels + c;
+        const T* xp = x + seg * x_real;
+        const T* dp = dy + seg * dy_real;
+        size_t tile = begin;
+        for (; tile + kTile <= end; tile += kTile)
+        {
+            T xv[kUnroll2][VEC], dv[kUnroll2][VEC];
+#pragma unroll
+            for (int u = 0; u < kUnroll2; ++u)
+            {
+                load_vec<T, VEC>(xp + tile + u * kStride + threadIdx.x * VEC, xv[u]);
+                load_vec<T, VEC>(dp + tile + u * kStride + threadIdx.x * VEC, dv[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < kUnroll2; ++u)
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+                    accumulate(xv[u][j], dv[u][j]);
+        }
+        for (size_t i = tile + threadIdx.x * VEC; i < end; i += kStride)
+        {
+            T xv[VEC], dv[VEC];
+            load_vec<T, VEC>(xp + i, xv);
+            load_vec<T, VEC>(dp + i, dv);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j)
+                accumulate(xv[j], dv[j]);
+        }
+    }
+    if (finish_channel<4>(acc, partials, counters, c, groups_per_channel_max) && threadIdx.x == 0)
+    {
+        dscale[c] = static_cast<T>(acc[0]);
+        dbias[c] = static_cast<T>(acc[1]);
+        dmean[c] = static_cast<T>(acc[2]);
+        dvar[c] = static_cast<T>(acc[3]);
+    }
+}
+
+// ---- backward: input gradient ------------------------------------------------
+// Replaces backprop2_opt_kernel, batchnorm.cu:1371-1418.  x and dx may alias:
+// each thread reads its elements before it writes them, so neither is
+// restrict-qualified.
+template <typename T, int VEC>
+__global__ __launch_bounds__(kBlockSize) void bn_backprop2_kernel(
+    const T* x, const T* __restrict__ dy, const T* __restrict__ mean,
+    const T* __restrict__ var, const T* __restrict__ scale, const T* __restrict__ dmean,
+    const T* __restrict__ dvar, T* dx, T epsilon, size_t num_per_sum, int num_channels,
+    size_t spatial, size_t x_real, size_t dy_real, size_t dx_real, size_t chunk,
+    int chunks_per_seg)
+{
+    const size_t seg = blockIdx.x / chunks_per_seg;
+    const int k = blockIdx.x - seg * chunks_per_seg;
+    const int c = seg % num_channels;
+    const T m = mean[c];
+    const T sc = scale[c];
+    const T inv_stdev = inv_sqrt_t(var[c] + epsilon);
+    const T dmean_term = dmean[c] / static_cast<T>(num_per_sum);
+    const T dvar_term = dvar[c] * T(2) / static_cast<T>(num_per_sum - 1);
+    const size_t begin = static_cast<size_t>(k) * chunk;
+    const size_t end = begin + chunk < spatial ? begin + chunk : spatial;
+    const T* xp = x + seg * x_real;
+    const T* dp = dy + seg * dy_real;
+    T* op = dx + seg * dx_real;
+
+    constexpr size_t kStride = static_cast<size_t>(kBlockSize) * VEC;
+    constexpr int kUnroll2 = kUnroll / 2;
+    constexpr size_t kTile = kStride * kUnroll2;
+    size_t tile = begin;
+    for (; tile + kTile <= end; tile += kTile)
+    {
+        T xv[kUnroll2][VEC], dv[kUnroll2][VEC];
+#pragma unroll
+        for (int u = 0; u < kUnroll2; ++u)
+        {
+            load_vec<T, VEC>(xp + tile + u * kStride + threadIdx.x * VEC, xv[u]);
+            load_vec<T, VEC>(dp + tile + u * kStride + threadIdx.x * VEC, dv[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll2; ++u)
+        {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j)
+            {
+                T r = fma_t(dv[u][j] * sc, inv_stdev, dmean_term);
+                xv[u][j] = fma_t(xv[u][j] - m, dvar_term, r);
+            }
+            store_vec<T, VEC>(op + tile + u * kStride + threadIdx.x * VEC, xv[u]);
+        }
+    }
+    for (size_t i = tile + threadIdx.x * VEC; i < end; i += kStride)
+    {
+        T xv[VEC], dv[VEC];
+        load_vec<T, VEC>(xp + i, xv);
+        load_vec<T, VEC>(dp + i, dv);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j)
+        {
+            T r = fma_t(dv[j] * sc, inv_stdev, dmean_term);
+            xv[j] = fma_t(xv[j] - m, dvar_term, r);
+        }
+        store_vec<T, VEC>(op + i, xv);
+    }
+}
+
+// ---- host side ---------------------------------------------------------------
+
+template <typename T>
+constexpr int full_vec()
+{
+    return 16 / sizeof(T);
+}
+
+// 16-byte accesses need every segment start and the base on a 16-byte boundary.
+template <typename T>
+bool can_vectorize(const void* p, size_t spatial, size_t real)
+{
+    constexpr size_t v = full_vec<T>();
+    return aligned16(p) && spatial % v == 0 && real % v == 0;
+}
+
+bool grid_ok(size_t blocks)
+{
+    return blocks <= 0x7fffffffull;
+}
+
+template <typename T>
+int sums_impl(int num_samples, int num_channels, size_t spatial, size_t real, const void* x,
+              void* sums, void* sqsums, void* workspace, hipStream_t stream)
+{
+    if (num_channels == 0)
+        return H2X_SUCCESS;
+    if (num_samples == 0 || spatial == 0)
+    {
+        const int blocks = (num_channels + kBlockSize - 1) / kBlockSize;
+        fill_kernel<T><<<blocks, kBlockSize, 0, stream>>>(static_cast<T*>(sums), num_channels, T(0));
+        fill_kernel<T><<<blocks, kBlockSize, 0, stream>>>(static_cast<T*>(sqsums), num_channels, T(0));
+        return launch_status();
+    }
+    const bool vec = can_vectorize<T>(x, spatial, real);
+    const int vw = vec ? full_vec<T>() : 1;
+    const int gmax = max_groups_per_channel(num_channels);
+    const size_t tile = static_cast<size_t>(kBlockSize) * vw * kUnroll;
+    const Chunking ch = make_chunking(spatial, num_samples, gmax, tile, tile);
+    const size_t units = static_cast<size_t>(ch.chunks_per_seg) * num_samples;
+    if (units > 0xffffffffull || num_channels > 65535)
+        return H2X_ERR_TOO_LARGE;
+    const size_t groups = std::min<size_t>(units, gmax);
+    double* partials = static_cast<double*>(workspace);
+    unsigned int* counters = reinterpret_cast<unsigned int*>(static_cast<char*>(workspace)
+                                                             + counters_offset(num_channels));
+    const dim3 grid(static_cast<unsigned int>(groups), num_channels);
+    if (vec)
+        bn_sums_kernel<T, full_vec<T>()><<<grid, kBlockSize, 0, stream>>>(
+            static_cast<const T*>(x), static_cast<T*>(sums), static_cast<T*>(sqsums), partials,
+            counters, num_channels, spatial, real, ch.chunk, ch.chunks_per_seg,
+            static_cast<unsigned int>(units), gmax);
+    else
+        bn_sums_kernel<T, 1><<<grid, kBlockSize, 0, stream>>>(
+            static_cast<const T*>(x), static_cast<T*>(sums), static_cast<T*>(sqsums), partials,
+            counters, num_channels, spatial, real, ch.chunk, ch.chunks_per_seg,
+            static_cast<unsigned int>(units), gmax);
+    return launch_status();
+}
+
+template <typename T>
+int statistics_impl(int num_channels, size_t num_per_sum, double decay, void* mean, void* var,
+                    void* running_mean, void* running_var, hipStream_t stream)
+{
+    if (num_channels == 0)
+        return H2X_SUCCESS;
+    const int blocks = std::min((num_channels + kBlockSize - 1) / kBlockSize, 1024);
+    bn_statistics_kernel<T><<<blocks, kBlockSize, 0, stream>>>(
+        num_channels, num_per_sum, static_cast<T>(decay), static_cast<T*>(mean),
+        static_cast<T*>(var), static_cast<T*>(running_mean), static_cast<T*>(running_var));
+    return launch_status();
+}
+
+// Chunking of an elementwise pass over N*C segments.
+template <typename T>
+Chunking elementwise_chunking(size_t spatial, size_t segments, int vw, int unroll)
+{
+    const size_t tile = static_cast<size_t>(kBlockSize) * vw * unroll;
+    const size_t one_pass = static_cast<size_t>(kBlockSize) * vw;
+    // aim at >= 4096 workgroups, but at least one full vector per thread
+    return make_chunking(spatial, segments, 4096, one_pass, one_pass * 2 > tile ? one_pass : one_pass * 2);
+}
+
+template <typename T>
+int apply_impl(int num_samples, int num_channels, size_t spatial, size_t x_real, size_t y_real,
+               const void* x, const void* mean, const void* var, const void* scale,
+               const void* bias, void* y, double epsilon, hipStream_t stream)
+{
+    const size_t segments = static_cast<size_t>(num_samples) * num_channels;
+    if (segments == 0 || spatial == 0)
+        return H2X_SUCCESS;
+    const bool vec = can_vectorize<T>(x, spatial, x_real) && can_vectorize<T>(y, spatial, y_real);
+    const int vw = vec ? full_vec<T>() : 1;
+    const Chunking ch = elementwise_chunking<T>(spatial, segments, vw, kUnroll);
+    const size_t blocks = segments * ch.chunks_per_seg;
+    if (!grid_ok(blocks))
+        return H2X_ERR_TOO_LARGE;
+    const unsigned int grid = static_cast<unsigned int>(blocks);
+#define H2X_LAUNCH(V)                                                                              \
+    bn_apply_kernel<T, V><<<grid, kBlockSize, 0, stream>>>(                                        \
+        static_cast<const T*>(x), static_cast<const T*>(mean), static_cast<const T*>(var),         \
+        static_cast<const T*>(scale), static_cast<const T*>(bias), static_cast<T*>(y),             \
+        static_cast<T>(epsilon), num_channels, spatial, x_real, y_real, ch.chunk,                  \
+        ch.chunks_per_seg)
+    if (vec)
+        H2X_LAUNCH(full_vec<T>());
+    else
+        H2X_LAUNCH(1);
+#undef H2X_LAUNCH
+    return launch_status();
+}
+
+template <typename T>
+int backprop1_impl(int num_samples, int num_channels, size_t spatial, size_t x_real,
+                   size_t dy_real, const void* x, const void* dy, const void* mean,
+                   const void* var, const void* scale, void* dscale, void* dbias, void* dmean,
+                   void* dvar, double epsilon, void* workspace, hipStream_t stream)
+{
+    if (num_channels == 0)
+        return H2X_SUCCESS;
+    if (num_samples == 0 || spatial == 0)
+    {
+        const int blocks = (num_channels + kBlockSize - 1) / kBlockSize;
+        for (void* p : {dscale, dbias, dmean, dvar})
+            fill_kernel<T><<<blocks, kBlockSize, 0, stream>>>(static_cast<T*>(p), num_channels, T(0));
+        return launch_status();
+    }
+    const bool vec = can_vectorize<T>(x, spatial, x_real) && can_vectorize<T>(dy, spatial, dy_real);
+    const int vw = vec ? full_vec<T>() : 1;
+    const int gmax = max_groups_per_channel(num_channels);
+    const size_t tile = static_cast<size_t>(kBlockSize) * vw * (kUnroll / 2);
+    const Chunking ch = make_chunking(spatial, num_samples, gmax, tile, tile);
+    const size_t units = static_cast<size_t>(ch.chunks_per_seg) * num_samples;
+    if (units > 0xffffffffull || num_channels > 65535)
+        return H2X_ERR_TOO_LARGE;
+    const size_t groups = std::min<size_t>(units, gmax);
+    double* partials = static_cast<double*>(workspace);
+    unsigned int* counters = reinterpret_cast<unsigned int*>(static_cast<char*>(workspace)
+                                                             + counters_offset(num_channels));
+    const dim3 grid(static_cast<unsigned int>(groups), num_channels);
+#define H2X_LAUNCH(V)                                                                              \
+    bn_backprop1_kernel<T, V><<<grid, kBlockSize, 0, stream>>>(                                    \
+        static_cast<const T*>(x), static_cast<const T*>(dy), static_cast<const T*>(mean),          \
+        static_cast<const T*>(var), static_cast<const T*>(scale), static_cast<T*>(dscale),         \
+        static_cast<T*>(dbias), static_cast<T*>(dmean), static_cast<T*>(dvar),                     \
+        static_cast<T>(epsilon), partials, counters, num_channels, spatial, x_real, dy_real,       \
+        ch.chunk, ch.chunks_per_seg, static_cast<unsigned int>(units), gmax)
+    if (vec)
+        H2X_LAUNCH(full_vec<T>());
+    else
+        H2X_LAUNCH(1);
+#undef H2X_LAUNCH
+    return launch_status();
+}
+
+template <typename T>
+int backprop2_impl(int num_samples, int num_channels, size_t spatial, size_t x_real,
+                   size_t dy_real, size_t dx_real, size_t num_per_sum, const void* x,
+                   const void* dy, const void* mean, const void* var, const void* scale,
+                   const void* dmean, const void* dvar, void* dx, double epsilon,
+                   hipStream_t stream)
+{
+    const size_t segments = static_cast<size_t>(num_samples) * num_channels;
+    if (segments == 0 || spatial == 0)
+        return H2X_SUCCESS;
+    const bool vec = can_vectorize<T>(x, spatial, x_real) && can_vectorize<T>(dy, spatial, dy_real)
+                     && can_vectorize<T>(dx, spatial, dx_real);
+    const int vw = vec ? full_vec<T>() : 1;
+    const Chunking ch = elementwise_chunking<T>(spatial, segments, vw, kUnroll / 2);
+    const size_t blocks = segments * ch.chunks_per_seg;
+    if (!grid_ok(blocks))
+        return H2X_ERR_TOO_LARGE;
+    const unsigned int grid = static_cast<unsigned int>(blocks);
+#define H2X_LAUNCH(V)                                                                              \
+    bn_backprop2_kernel<T, V><<<grid, kBlockSize, 0, stream>>>(                                    \
+        static_cast<const T*>(x), static_cast<const T*>(dy), static_cast<const T*>(mean),          \
+        static_cast<const T*>(var), static_cast<const T*>(scale), static_cast<const T*>(dmean),    \
+        static_cast<const T*>(dvar), static_cast<T*>(dx), static_cast<T>(epsilon), num_per_sum,    \
+        num_channels, spatial, x_real, dy_real, dx_real, ch.chunk, ch.chunks_per_seg)
+    if (vec)
+        H2X_LAUNCH(full_vec<T>());
+    else
+        H2X_LAUNCH(1);
+#undef H2X_LAUNCH
+    return launch_status();
+}
+
+bool bad_geometry(int num_samples, int num_channels, size_t spatial, size_t real)
+{
+    return num_samples < 0 || num_channels < 0 || real < spatial;
+}
+
+} // namespace
+} // namespace h2x
+
+using namespace h2x;
+
+extern "C" size_t h2x_bn_workspace_bytes(int num_channels)
+{
+    if (num_channels <= 0)
+        return 256;
+    const size_t bytes = counters_offset(num_channels) + static_cast<size_t>(num_channels) * sizeof(unsigned int);
+    return (bytes + 255) / 256 * 256;
+}
+
+extern "C" int h2x_bn_workspace_init(void* workspace, int num_channels, h2x_stream_t stream)
+{
+    if (workspace == nullptr || num_channels < 0)
+        return H2X_ERR_INVALID_ARGUMENT;
+    const size_t words = h2x_bn_workspace_bytes(num_channels) / sizeof(unsigned int);
+    const unsigned int blocks = static_cast<unsigned int>(std::min<size_t>((words + kBlockSize - 1) / kBlockSize, 1024));
+    fill_kernel<unsigned int><<<blocks, kBlockSize, 0, as_stream(stream)>>>(
+        static_cast<unsigned int*>(workspace), words, 0u);
+    return launch_status();
+}
+
+extern "C" int h2x_bn_channel_sums_and_sqsums(h2x_dtype dtype, int num_samples, int num_channels,
+                                              size_t spatial_size, size_t spatial_real_size,
+                                              const void* x, void* sums, void* sqsums,
+                                              void* workspace, h2x_stream_t stream)
+{
+    if (bad_geometry(num_samples, num_channels, spatial_size, spatial_real_size) || !sums || !sqsums
+        || !workspace || (!x && num_samples > 0 && spatial_size > 0 && num_channels > 0))
+        return H2X_ERR_INVALID_ARGUMENT;
+    switch (dtype)
+    {
+    case H2X_F32:
+        return sums_impl<float>(num_samples, num_channels, spatial_size, spatial_real_size, x, sums,
+                                sqsums, workspace, as_stream(stream));
+    case H2X_F64:
+        return sums_impl<double>(num_samples, num_channels, spatial_size, spatial_real_size, x,
+                                 sums, sqsums, workspace, as_stream(stream));
+    }
+    return H2X_ERR_UNSUPPORTED;
+}
+
+extern "C" int h2x_bn_sums_to_statistics(h2x_dtype dtype, int num_channels, size_t num_per_sum,
+                                         double decay, void* mean_inout, void* var_inout,
+                                         void* running_mean, void* running_var,
+                                         h2x_stream_t stream)
+{
+    if (num_channels < 0 || !mean_inout || !var_inout || !running_mean || !running_var)
+        return H2X_ERR_INVALID_ARGUMENT;
+    switch (dtype)
+    {
+    case H2X_F32:
+        return statistics_impl<float>(num_channels, num_per_sum, decay, mean_inout, var_inout,
+                                      running_mean, running_var, as_stream(stream));
+    case H2X_F64:
+        return statistics_impl<double>(num_channels, num_per_sum, decay, mean_inout, var_inout,
+                                       running_mean, running_var, as_stream(stream));
+    }
+    return H2X_ERR_UNSUPPORTED;
+}
+
+extern "C" int h2x_bn_batch_normalization(h2x_dtype dtype, int num_samples, int num_channels,
+                                          size_t spatial_size, size_t x_spatial_real_size,
+                                          size_t y_spatial_real_size, const void* x,
+                                          const void* mean, const void* var, const void* scale,
+                                          const void* bias, void* y, double epsilon,
+                                          h2x_stream_t stream)
+{
+    if (bad_geometry(num_samples, num_channels, spatial_size, x_spatial_real_size)
+        || y_spatial_real_size < spatial_size || !mean || !var || !scale || !bias)
+        return H2X_ERR_INVALID_ARGUMENT;
+    if ((!x || !y) && static_cast<size_t>(num_samples) * num_channels * spatial_size > 0)
+        return H2X_ERR_INVALID_ARGUMENT;
+    switch (dtype)
+    {
+    case H2X_F32:
+        return apply_impl<float>(num_samples, num_channels, spatial_size, x_spatial_real_size,
+                                 y_spatial_real_size, x, mean, var, scale, bias, y, epsilon,
+                                 as_stream(stream));
+    case H2X_F64:
+        return apply_impl<double>(num_samples, num_channels, spatial_size, x_spatial_real_size,
+                                  y_spatial_real_size, x, mean, var, scale, bias, y, epsilon,
+                                  as_stream(stream));
+    }
+    return H2X_ERR_UNSUPPORTED;
+}
+
+extern "C" int h2x_bn_backprop1(h2x_dtype dtype, int num_samples, int num_channels,
+                                size_t spatial_size, size_t x_spatial_real_size,
+                                size_t dy_spatial_real_size, const void* x, const void* dy,
+                                const void* mean, const void* var, const void* scale, void* dscale,
+                                void* dbias, void* dmean, void* dvar, double epsilon,
+                                void* workspace, h2x_stream_t stream)
+{
+    if (bad_geometry(num_samples, num_channels, spatial_size, x_spatial_real_size)
+        || dy_spatial_real_size < spatial_size || !mean || !var || !scale || !dscale || !dbias
+        || !dmean || !dvar || !workspace)
+        return H2X_ERR_INVALID_ARGUMENT;
+    if ((!x || !dy) && static_cast<size_t>(num_samples) * num_channels * spatial_size > 0)
+        return H2X_ERR_INVALID_ARGUMENT;
+    switch (dtype)
+    {
+    case H2X_F32:
+        return backprop1_impl<float>(num_samples, num_channels, spatial_size, x_spatial_real_size,
+                                     dy_spatial_real_size, x, dy, mean, var, scale, dscale, dbias,
+                                     dmean, dvar, epsilon, workspace, as_stream(stream));
+    case H2X_F64:
+        return backprop1_impl<double>(num_samples, num_channels, spatial_size, x_spatial_real_size,
+                                      dy_spatial_real_size, x, dy, mean, var, scale, dscale, dbias,
+                                      dmean, dvar, epsilon, workspace, as_stream(stream));
+    }
+    return H2X_ERR_UNSUPPORTED;
+}
+
+extern "C" int h2x_bn_backprop2(h2x_dtype dtype, int num_samples, int num_channels,
+                                size_t spatial_size, size_t x_spatial_real_size,
+                                size_t dy_spatial_real_size, size_t dx_spatial_real_size,
+                                size_t num_per_sum, const void* x, const void* dy,
+                                const void* mean, const void* var, const void* scale,
+                                const void* dmean, const void* dvar, void* dx, double epsilon,
+                                h2x_stream_t stream)
+{
+    if (bad_geometry(num_samples, num_channels, spatial_size, x_spatial_real_size)
+        || dy_spatial_real_size < spatial_size || dx_spatial_real_size < spatial_size || !mean
+        || !var || !scale || !dmean || !dvar)
+        return H2X_ERR_INVALID_ARGUMENT;
+    if ((!x || !dy || !dx) && static_cast<size_t>(num_samples) * num_channels * spatial_size > 0)
+        return H2X_ERR_INVALID_ARGUMENT;
+    switch (dtype)
+    {
+    case H2X_F32:
+        return backprop2_impl<float>(num_samples, num_channels, spatial_size, x_spatial_real_size,
+                                     dy_spatial_real_size, dx_spatial_real_size, num_per_sum, x, dy,
+                                     mean, var, scale, dmean, dvar, dx, epsilon, as_stream(stream));
+    case H2X_F64:
+        return backprop2_impl<double>(num_samples, num_channels, spatial_size, x_spatial_real_size,
+                                      dy_spatial_real_size, dx_spatial_real_size, num_per_sum, x,
+                                      dy, mean, var, scale, dmean, dvar, dx, epsilon,
+                                      as_stream(stream));
+    }
+    return H2X_ERR_UNSUPPORTED;
+}

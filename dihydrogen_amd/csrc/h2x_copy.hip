@@ -1,0 +1,712 @@
+// Box copy engine for gfx950: halo pack/unpack/clear and tensor-shuffler
+// pack/unpack, with the C entry points of both.
+//
+// Both operations move a rectangular sub-box of a strided tensor to or from a
+// contiguous buffer that holds the box in natural (innermost-first) order of
+// the box's own extents:
+//   - a halo strip is the box {shape[0..dim-1], width, shape[dim+1..]} at the
+//     strip's start along `dim` (legacy/include/distconv/tensor/halo_cuda.hpp:34-88);
+//   - the part of a local tensor that goes to one peer rank of a shuffle is
+//     the intersection box of the two ranks' regions, and the order
+//     find_destination produces inside a peer's chunk is the natural order of
+//     that box (legacy/src/tensor/shuffle_mpi_cuda.cu:42-98).
+// The host reduces every box to as few dimensions as possible (extent-1
+// dimensions vanish, dimensions that are contiguous in the tensor merge), so a
+// halo strip becomes "outer runs of `run` contiguous elements" and the device
+// index arithmetic is one or two multiply-high divisions per 16 bytes moved,
+// instead of a division chain per element (halo_cuda.hpp:47-81) or a search
+// per element (shuffle_mpi_cuda.cu:70-84).  Up to kMaxBoxes boxes -- both
+// sides of a dimension, all peers of a rank, several virtual ranks -- share a
+// launch; their descriptors travel in the kernel arguments, so nothing is
+// allocated or copied to set a launch up.
+#include "h2x_device.hpp"
+
+#include <algorithm>
+#include <cstring>
+#include <new>
+#include <type_traits>
+#include <vector>
+
+namespace h2x
+{
+namespace
+{
+
+constexpr int kMaxBoxes = 16;
+constexpr int kMaxBoxDims = H2X_MAX_DIMS;
+constexpr int kCopyUnroll = 4;
+
+enum Mode : int
+{
+    kPack = 0,    // buffer <- tensor
+    kUnpack = 1,  // tensor <- op(tensor, buffer)
+    kClear = 2    // tensor <- 0
+};
+
+// n / d for n < 2^31 by multiply-high and shift.
+struct FastDiv
+{
+    uint32_t divisor;
+    uint32_t multiplier;
+    uint32_t shift;
+};
+
+FastDiv make_fastdiv(uint32_t d)
+{
+    FastDiv f{d, 0u, 0u};
+    if (d > 1)
+    {
+        uint32_t log2 = 0;
+        while ((1ull << log2) < d)
+            ++log2;
+        const uint32_t p = 31 + log2;
+        f.multiplier = static_cast<uint32_t>(((1ull << p) + d - 1) / d);
+        f.shift = p - 32;
+    }
+    return f;
+}
+
+__host__ __device__ inline uint32_t fastdiv(uint32_t n, const FastDiv& f)
+{
+#ifdef __HIP_DEVICE_COMPILE__
+    return f.divisor == 1 ? n : __umulhi(n, f.multiplier) >> f.shift;
+#else
+    return f.divisor == 1
+               ? n
+               : static_cast<uint32_t>((static_cast<uint64_t>(n) * f.multiplier) >> 32) >> f.shift;
+#endif
+}
+
+// One reduced box.  Packed element g (natural order of extent[]) lives at
+// tensor[tensor_offset + sum idx[i] * stride[i]].
+struct Box
+{
+    char* tensor;            // base the strides are relative to
+    char* buffer;            // start of this box's contiguous image
+    int64_t stride[kMaxBoxDims]; // elements
+    FastDiv div[kMaxBoxDims];    // by extent[i]; the last used one is never divided by
+    uint32_t count;          // elements in the box (< 2^31)
+    uint32_t first_block;    // first workgroup of this box in the launch
+    int32_t num_dims;
+    int32_t mode;            // Mode
+};
+
+struct BoxBatch
+{
+    Box box[kMaxBoxes];
+    int32_t num_boxes;
+    uint32_t num_blocks;
+};
+
+template <typename W, int VEC>
+struct Words
+{
+    typedef W aligned_t __attribute__((ext_vector_type(VEC)));
+    typedef W unaligned_t __attribute__((ext_vector_type(VEC), aligned(sizeof(W))));
+};
+
+struct OpId
+{
+    template <typename T>
+    __device__ __forceinline__ T operator()(T, T b) const { return b; }
+};
+struct OpSum
+{
+    template <typename T>
+    __device__ __forceinline__ T operator()(T a, T b) const { return a + b; }
+};
+struct OpMax
+{
+    template <typename T>
+    __device__ __forceinline__ T operator()(T a, T b) const { return a > b ? a : b; }
+};
+struct OpMin
+{
+    template <typename T>
+    __device__ __forceinline__ T operator()(T a, T b) const { return a < b ? a : b; }
+};
+
+// T: element type the op sees (an unsigned integer of the element's size for
+// plain copies).  VEC elements of one run move per thread and step; the buffer
+// side is VEC-aligned, the tensor side may start on any element.
+template <typename T, int VEC, typename Op>
+__global__ __launch_bounds__(kBlockSize) void box_copy_kernel(const BoxBatch batch, Op op)
+{
+    // which box does this workgroup belong to?
+    int b = 0;
+#pragma unroll 1
+    for (int i = 1; i < batch.num_boxes; ++i)
+        if (blockIdx.x >= batch.box[i].first_block)
+            b = i;
+    const Box& box = batch.box[b];
+    const uint32_t count = box.count;
+    const int nd = box.num_dims;
+    const int mode = box.mode;
+    T* const tensor = reinterpret_cast<T*>(box.tensor);
+    T* const buffer = reinterpret_cast<T*>(box.buffer);
+    using WA = typename Words<T, VEC>::aligned_t;
+    using WU = typename Words<T, VEC>::unaligned_t;
+
+    constexpr uint32_t kStride = kBlockSize * VEC;
+    const uint32_t block_base = (blockIdx.x - box.first_block) * (kStride * kCopyUnroll);
+
+    int64_t toff[kCopyUnroll];
+    uint32_t g[kCopyUnroll];
+#pragma unroll
+    for (int u = 0; u < kCopyUnroll; ++u)
+    {
+        g[u] = block_base + u * kStride + threadIdx.x * VEC;
+        uint32_t rem = g[u];
+        int64_t off = 0;
+#pragma unroll
+        for (int i = 0; i < kMaxBoxDims - 1; ++i)
+        {
+            if (i < nd - 1)
+            {
+                const uint32_t q = fastdiv(rem, box.div[i]);
+                off += static_cast<int64_t>(rem - q * box.div[i].divisor) * box.stride[i];
+                rem = q;
+            }
+        }
+        off += static_cast<int64_t>(rem) * box.stride[nd - 1];
+        toff[u] = off;
+    }
+
+    if (mode == kPack)
+    {
+        WU v[kCopyUnroll];
+#pragma unroll
+        for (int u = 0; u < kCopyUnroll; ++u)
+            if (g[u] < count)
+                v[u] = *reinterpret_cast<const WU*>(tensor + toff[u]);
+#pragma unroll
+        for (int u = 0; u < kCopyUnroll; ++u)
+            if (g[u] < count)
+                *reinterpret_cast<WA*>(buffer + g[u]) = v[u];
+    }
+    else if (mode == kUnpack)
+    {
+        WA v[kCopyUnroll];
+#pragma unroll
+        for (int u = 0; u < kCopyUnroll; ++u)
+            if (g[u] < count)
+                v[u] = *reinterpret_cast<const WA*>(buffer + g[u]);
+        if constexpr (std::is_same<Op, OpId>::value)
+        {
+#pragma unroll
+            for (int u = 0; u < kCopyUnroll; ++u)
+                if (g[u] < count)
+                    *reinterpret_cast<WU*>(tensor + toff[u]) = v[u];
+        }
+        else
+        {
+#pragma unroll
+            for (int u = 0; u < kCopyUnroll; ++u)
+                if (g[u] < count)
+                {
+                    WU t = *reinterpret_cast<const WU*>(tensor + toff[u]);
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j)
+                        t[j] = op(t[j], v[u][j]);
+                    *reinterpret_cast<WU*>(tensor + toff[u]) = t;
+                }
+        }
+    }
+    else
+    {
+        WU z;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j)
+            z[j] = T(0);
+#pragma unroll
+        for (int u = 0; u < kCopyUnroll; ++u)
+            if (g[u] < count)
+                *reinterpret_cast<WU*>(tensor + toff[u]) = z;
+    }
+}
+
+// ---- host: box reduction ------------------------------------------------------
+
+struct HostBox
+{
+    int nd = 0;
+    int64_t extent[kMaxBoxDims];
+    int64_t stride[kMaxBoxDims];
+    int64_t tensor_offset = 0; // elements from the tensor pointer to the box origin
+    int64_t buffer_offset = 0; // elements from the buffer pointer
+    int64_t count = 1;
+};
+
+// Drops extent-1 dimensions and merges neighbours that are contiguous in the
+// tensor; the natural order of the reduced box is the natural order of the
+// original one.
+HostBox reduce_box(int nd, const int64_t* extent, const int64_t* stride, int64_t tensor_offset,
+                   int64_t buffer_offset)
+{
+    HostBox h;
+    h.tensor_offset = tensor_offset;
+    h.buffer_offset = buffer_offset;
+    for (int i = 0; i < nd; ++i)
+    {
+        h.count *= extent[i];
+        if (extent[i] == 1)
+            continue;
+        if (h.nd > 0 && stride[i] == h.stride[h.nd - 1] * h.extent[h.nd - 1])
+        {
+            h.extent[h.nd - 1] *= extent[i];
+        }
+        else
+        {
+            h.extent[h.nd] = extent[i];
+            h.stride[h.nd] = stride[i];
+            ++h.nd;
+        }
+    }
+    if (h.nd == 0)
+    {
+        h.nd = 1;
+        h.extent[0] = 1;
+        h.stride[0] = 1;
+    }
+    return h;
+}
+
+// Largest power-of-two vector (elements, at most 16 bytes) that never crosses a
+// run of the box and keeps the buffer side aligned.
+int box_vector(const HostBox& h, int elem_size, const void* buffer)
+{
+    int v = 16 / elem_size;
+    if (h.stride[0] != 1)
+        return 1;
+    while (v > 1)
+    {
+        const bool ok = h.extent[0] % v == 0 && h.buffer_offset % v == 0
+                        && reinterpret_cast<uintptr_t>(buffer) % (static_cast<size_t>(v) * elem_size) == 0;
+        if (ok)
+            break;
+        v /= 2;
+    }
+    return v;
+}
+
+struct Launcher
+{
+    hipStream_t stream;
+    int elem_size;
+    h2x_dtype dtype; // meaningful for accumulate ops only
+    int op;          // h2x_halo_op
+    int vec = 0;
+    BoxBatch batch;
+
+    Launcher(hipStream_t s, int es, h2x_dtype dt, int o) : stream(s), elem_size(es), dtype(dt), op(o)
+    {
+        batch.num_boxes = 0;
+        batch.num_blocks = 0;
+    }
+
+    template <typename T, int VEC>
+    int launch_typed()
+    {
+        const dim3 grid(batch.num_blocks);
+        switch (op)
+        {
+        case H2X_HALO_ID: box_copy_kernel<T, VEC, OpId><<<grid, kBlockSize, 0, stream>>>(batch, OpId()); break;
+        default: return H2X_ERR_UNSUPPORTED;
+        }
+        return launch_status();
+    }
+
+    template <typename T, int VEC>
+    int launch_accumulate()
+    {
+        const dim3 grid(batch.num_blocks);
+        switch (op)
+        {
+        case H2X_HALO_SUM: box_copy_kernel<T, VEC, OpSum><<<grid, kBlockSize, 0, stream>>>(batch, OpSum()); break;
+        case H2X_HALO_MAX: box_copy_kernel<T, VEC, OpMax><<<grid, kBlockSize, 0, stream>>>(batch, OpMax()); break;
+        case H2X_HALO_MIN: box_copy_kernel<T, VEC, OpMin><<<grid, kBlockSize, 0, stream>>>(batch, OpMin()); break;
+        default: return H2X_ERR_UNSUPPORTED;
+        }
+        return launch_status();
+    }
+
+    template <typename U, typename F, int V>
+    int launch_width()
+    {
+        if constexpr (!std::is_void<F>::value)
+            if (op != H2X_HALO_ID)
+                return launch_accumulate<F, V>();
+        return launch_typed<U, V>();
+    }
+
+    template <typename U, typename F>
+    int launch_vec()
+    {
+        constexpr int kFull = 16 / sizeof(U);
+        switch (vec)
+        {
+        case 8:
+            if constexpr (kFull >= 8)
+                return launch_width<U, F, 8>();
+            break;
+        case 4:
+            if constexpr (kFull >= 4)
+                return launch_width<U, F, 4>();
+            break;
+        case 2: return launch_width<U, F, 2>();
+        case 1: return launch_width<U, F, 1>();
+        }
+        return H2X_ERR_UNSUPPORTED;
+    }
+
+    int flush()
+    {
+        if (batch.num_boxes == 0)
+            return H2X_SUCCESS;
+        int err;
+        switch (elem_size)
+        {
+        case 2: err = op == H2X_HALO_ID ? launch_vec<uint16_t, void>() : H2X_ERR_UNSUPPORTED; break;
+        case 4: err = launch_vec<uint32_t, float>(); break;
+        case 8: err = launch_vec<uint64_t, double>(); break;
+        default: err = H2X_ERR_UNSUPPORTED;
+        }
+        batch.num_boxes = 0;
+        batch.num_blocks = 0;
+        vec = 0;
+        return err;
+    }
+
+    // Queues one box; launches what is queued when the batch is full or the
+    // new box needs another vector width.
+    int add(const HostBox& h, void* tensor, void* buffer, int mode)
+    {
+        if (h.count == 0)
+            return H2X_SUCCESS;
+        if (h.count >= (1ll << 31))
+            return H2X_ERR_TOO_LARGE;
+        const int v = mode == kClear ? box_vector(h, elem_size, nullptr) : box_vector(h, elem_size, buffer);
+        if (batch.num_boxes == kMaxBoxes || (batch.num_boxes > 0 && v != vec))
+        {
+            const int err = flush();
+            if (err != 0)
+                return err;
+        }
+        vec = v;
+        Box& b = batch.box[batch.num_boxes];
+        b.tensor = static_cast<char*>(tensor) + h.tensor_offset * elem_size;
+        b.buffer = static_cast<char*>(buffer) + h.buffer_offset * elem_size;
+        for (int i = 0; i < kMaxBoxDims; ++i)
+        {
+            b.stride[i] = i < h.nd ? h.stride[i] : 0;
+            b.div[i] = make_fastdiv(i < h.nd ? static_cast<uint32_t>(h.extent[i]) : 1u);
+        }
+        b.count = static_cast<uint32_t>(h.count);
+        b.first_block = batch.num_blocks;
+        b.num_dims = h.nd;
+        b.mode = mode;
+        const uint64_t per_block = static_cast<uint64_t>(kBlockSize) * v * kCopyUnroll;
+        const uint64_t blocks = (static_cast<uint64_t>(h.count) + per_block - 1) / per_block;
+        if (batch.num_blocks + blocks > 0x7fffffffull)
+            return H2X_ERR_TOO_LARGE;
+        batch.num_blocks += static_cast<uint32_t>(blocks);
+        ++batch.num_boxes;
+        return H2X_SUCCESS;
+    }
+};
+
+int elem_size_of(h2x_dtype dtype)
+{
+    return dtype == H2X_F32 ? 4 : dtype == H2X_F64 ? 8 : 0;
+}
+
+// The strip of a halo face as a box over the real tensor.
+int halo_box(const h2x_halo_face& f, HostBox* out)
+{
+    const int nd = f.num_dims;
+    if (nd < 1 || nd > H2X_MAX_DIMS || f.dim < 0 || f.dim >= nd || f.width < 0
+        || (f.side != H2X_LHS && f.side != H2X_RHS))
+        return H2X_ERR_INVALID_ARGUMENT;
+    int64_t extent[kMaxBoxDims], stride[kMaxBoxDims];
+    int64_t s = 1;
+    for (int i = 0; i < nd; ++i)
+    {
+        if (f.real_shape[i] < 0)
+            return H2X_ERR_INVALID_ARGUMENT;
+        extent[i] = f.real_shape[i];
+        stride[i] = s;
+        s *= f.real_shape[i];
+    }
+    const int64_t len = f.real_shape[f.dim];
+    const int64_t w = f.width;
+    int64_t start;
+    if (f.side == H2X_RHS)
+        start = f.inner ? len - 2 * w : len - w;
+    else
+        start = f.inner ? w : 0;
+    if (w > 0 && (start < 0 || start + w > len))
+        return H2X_ERR_INVALID_ARGUMENT;
+    extent[f.dim] = w;
+    *out = reduce_box(nd, extent, stride, start * stride[f.dim], 0);
+    return H2X_SUCCESS;
+}
+
+} // namespace
+} // namespace h2x
+
+using namespace h2x;
+
+// ---- halo ----------------------------------------------------------------------
+
+extern "C" size_t h2x_halo_size(int num_dims, const int64_t* real_shape, int dim, int width)
+{
+    size_t s = 1;
+    for (int i = 0; i < num_dims; ++i)
+        s *= static_cast<size_t>(i == dim ? width : real_shape[i]);
+    return s;
+}
+
+extern "C" int h2x_halo_pack_or_unpack_batched(h2x_dtype dtype, const h2x_halo_face* faces,
+                                               int num_faces, h2x_stream_t stream)
+{
+    const int es = elem_size_of(dtype);
+    if (es == 0)
+        return H2X_ERR_UNSUPPORTED;
+    if (num_faces < 0 || (num_faces > 0 && !faces))
+        return H2X_ERR_INVALID_ARGUMENT;
+    // validate everything before anything is launched
+    std::vector<HostBox> boxes(num_faces);
+    for (int i = 0; i < num_faces; ++i)
+    {
+        const int err = halo_box(faces[i], &boxes[i]);
+        if (err != 0)
+            return err;
+        if (boxes[i].count > 0 && (!faces[i].tensor || !faces[i].buffer))
+            return H2X_ERR_INVALID_ARGUMENT;
+        if (boxes[i].count >= (1ll << 31))
+            return H2X_ERR_TOO_LARGE;
+        if (faces[i].op < H2X_HALO_ID || faces[i].op > H2X_HALO_MIN)
+            return H2X_ERR_INVALID_ARGUMENT;
+    }
+    // faces with the same effective op share launches
+    for (int op = H2X_HALO_ID; op <= H2X_HALO_MIN; ++op)
+    {
+        Launcher l(as_stream(stream), es, dtype, op);
+        for (int i = 0; i < num_faces; ++i)
+        {
+            const int eff = faces[i].is_pack ? H2X_HALO_ID : faces[i].op;
+            if (eff != op)
+                continue;
+            const int err = l.add(boxes[i], faces[i].tensor, faces[i].buffer,
+                                  faces[i].is_pack ? kPack : kUnpack);
+            if (err != 0)
+                return err;
+        }
+        const int err = l.flush();
+        if (err != 0)
+            return err;
+    }
+    return H2X_SUCCESS;
+}
+
+extern "C" int h2x_halo_pack_or_unpack(h2x_dtype dtype, void* tensor, int num_dims,
+                                       const int64_t* real_shape, int dim, int side, int width,
+                                       void* buffer, int is_pack, int is_reverse, int op,
+                                       h2x_stream_t stream)
+{
+    if (width == 0)
+        return H2X_SUCCESS; // halo_packing_cuda.hpp:153-154
+    if (!real_shape || num_dims < 1 || num_dims > H2X_MAX_DIMS)
+        return H2X_ERR_INVALID_ARGUMENT;
+    h2x_halo_face f;
+    std::memset(&f, 0, sizeof(f));
+    f.tensor = tensor;
+    f.buffer = buffer;
+    for (int i = 0; i < num_dims; ++i)
+        f.real_shape[i] = real_shape[i];
+    f.num_dims = num_dims;
+    f.dim = dim;
+    f.side = side;
+    f.width = width;
+    f.inner = ((is_pack && !is_reverse) || (!is_pack && is_reverse)) ? 1 : 0;
+    f.is_pack = is_pack ? 1 : 0;
+    f.op = op;
+    return h2x_halo_pack_or_unpack_batched(dtype, &f, 1, stream);
+}
+
+extern "C" int h2x_halo_clear(h2x_dtype dtype, void* tensor, int num_dims,
+                              const int64_t* real_shape, int dim, int width, h2x_stream_t stream)
+{
+    const int es = elem_size_of(dtype);
+    if (es == 0)
+        return H2X_ERR_UNSUPPORTED;
+    if (width == 0)
+        return H2X_SUCCESS;
+    if (!tensor || !real_shape || num_dims < 1 || num_dims > H2X_MAX_DIMS)
+        return H2X_ERR_INVALID_ARGUMENT;
+    Launcher l(as_stream(stream), es, dtype, H2X_HALO_ID);
+    for (int side = 0; side < 2; ++side)
+    {
+        h2x_halo_face f;
+        std::memset(&f, 0, sizeof(f));
+        for (int i = 0; i < num_dims; ++i)
+            f.real_shape[i] = real_shape[i];
+        f.num_dims = num_dims;
+        f.dim = dim;
+        f.side = side;
+        f.width = width;
+        f.inner = 0;
+        HostBox h;
+        int err = halo_box(f, &h);
+        if (err != 0)
+            return err;
+        err = l.add(h, tensor, nullptr, kClear);
+        if (err != 0)
+            return err;
+    }
+    return l.flush();
+}
+
+// ---- shuffle -------------------------------------------------------------------
+
+struct h2x_shuffle_plan
+{
+    int elem_size;
+    std::vector<HostBox> boxes; // one per peer with a non-empty intersection
+};
+
+extern "C" int h2x_shuffle_plan_create(const h2x_shuffle_geometry* g, h2x_shuffle_plan** plan)
+{
+    if (!g || !plan)
+        return H2X_ERR_INVALID_ARGUMENT;
+    *plan = nullptr;
+    const int nd = g->num_dims;
+    if (nd < 1 || nd > H2X_MAX_DIMS || !g->rank_limits || !g->displs)
+        return H2X_ERR_INVALID_ARGUMENT;
+    if (g->elem_size != 2 && g->elem_size != 4 && g->elem_size != 8)
+        return H2X_ERR_UNSUPPORTED;
+    int64_t num_peers = 1;
+    for (int i = 0; i < nd; ++i)
+    {
+        if (g->local_shape[i] < 0 || g->peer_locale_shape[i] < 1 || g->strides[i] < 0)
+            return H2X_ERR_INVALID_ARGUMENT;
+        num_peers *= g->peer_locale_shape[i];
+    }
+    // limits must be non-decreasing and end at the local extent
+    {
+        int rl = 0;
+        for (int i = 0; i < nd; ++i)
+        {
+            int prev = 0;
+            for (int j = 0; j < g->peer_locale_shape[i]; ++j)
+            {
+                const int lim = g->rank_limits[rl + j];
+                if (lim < prev || lim > g->local_shape[i])
+                    return H2X_ERR_INVALID_ARGUMENT;
+                prev = lim;
+            }
+            if (prev != g->local_shape[i] && g->local_shape[i] != 0)
+                return H2X_ERR_INVALID_ARGUMENT;
+            rl += static_cast<int>(g->peer_locale_shape[i]);
+        }
+    }
+    h2x_shuffle_plan* p = new (std::nothrow) h2x_shuffle_plan;
+    if (!p)
+        return static_cast<int>(hipErrorOutOfMemory);
+    p->elem_size = g->elem_size;
+    for (int64_t peer = 0; peer < num_peers; ++peer)
+    {
+        int64_t extent[kMaxBoxDims], rem = peer, origin = 0;
+        int rl = 0;
+        bool empty = false;
+        for (int i = 0; i < nd; ++i)
+        {
+            const int j = static_cast<int>(rem % g->peer_locale_shape[i]);
+            rem /= g->peer_locale_shape[i];
+            const int lo = j == 0 ? 0 : g->rank_limits[rl + j - 1];
+            const int hi = g->rank_limits[rl + j];
+            extent[i] = hi - lo;
+            origin += static_cast<int64_t>(lo) * g->strides[i];
+            empty = empty || extent[i] <= 0;
+            rl += static_cast<int>(g->peer_locale_shape[i]);
+        }
+        if (empty)
+            continue;
+        HostBox h = reduce_box(nd, extent, g->strides, origin, g->displs[peer]);
+        if (h.count >= (1ll << 31))
+        {
+            delete p;
+            return H2X_ERR_TOO_LARGE;
+        }
+        p->boxes.push_back(h);
+    }
+    *plan = p;
+    return H2X_SUCCESS;
+}
+
+extern "C" int h2x_shuffle_plan_destroy(h2x_shuffle_plan* plan)
+{
+    delete plan;
+    return H2X_SUCCESS;
+}
+
+static int shuffle_batched(const h2x_shuffle_plan* const* plans, void* const* tensors,
+                           void* const* buffers, int num_plans, int mode, h2x_stream_t stream)
+{
+    if (num_plans < 0 || (num_plans > 0 && (!plans || !tensors || !buffers)))
+        return H2X_ERR_INVALID_ARGUMENT;
+    for (int i = 0; i < num_plans; ++i)
+    {
+        if (!plans[i])
+            return H2X_ERR_INVALID_ARGUMENT;
+        if (!plans[i]->boxes.empty() && (!tensors[i] || !buffers[i]))
+            return H2X_ERR_INVALID_ARGUMENT;
+    }
+    for (int es : {2, 4, 8})
+    {
+        Launcher l(as_stream(stream), es, H2X_F32, H2X_HALO_ID);
+        for (int i = 0; i < num_plans; ++i)
+        {
+            if (plans[i]->elem_size != es)
+                continue;
+            for (const HostBox& h : plans[i]->boxes)
+            {
+                const int err = l.add(h, tensors[i], buffers[i], mode);
+                if (err != 0)
+                    return err;
+            }
+        }
+        const int err = l.flush();
+        if (err != 0)
+            return err;
+    }
+    return H2X_SUCCESS;
+}
+
+extern "C" int h2x_shuffle_pack(const h2x_shuffle_plan* plan, const void* tensor, void* buffer,
+                                h2x_stream_t stream)
+{
+    void* t = const_cast<void*>(tensor);
+    return shuffle_batched(&plan, &t, &buffer, 1, kPack, stream);
+}
+
+extern "C" int h2x_shuffle_unpack(const h2x_shuffle_plan* plan, void* tensor, const void* buffer,
+                                  h2x_stream_t stream)
+{
+    void* b = const_cast<void*>(buffer);
+    return shuffle_batched(&plan, &tensor, &b, 1, kUnpack, stream);
+}
+
+extern "C" int h2x_shuffle_pack_batched(const h2x_shuffle_plan* const* plans,
+                                        const void* const* tensors, void* const* buffers,
+                                        int num_plans, h2x_stream_t stream)
+{
+    return shuffle_batched(plans, const_cast<void* const*>(tensors), buffers, num_plans, kPack, stream);
+}
+
+extern "C" int h2x_shuffle_unpack_batched(const h2x_shuffle_plan* const* plans,
+                                          void* const* tensors, const void* const* buffers,
+                                          int num_plans, h2x_stream_t stream)
+{
+    return shuffle_batched(plans, tensors, const_cast<void* const*>(buffers), num_plans, kUnpack, stream);
+}

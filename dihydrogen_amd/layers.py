@@ -1,0 +1,497 @@
+"""Python mirror of the DistConv layer API for the non-convolution hot path,
+on top of the C ABI (``include/h2x.h``).  Method names, argument order and
+return values follow the reference classes; MPI ranks are replaced by virtual
+ranks whose local tensors live on one GPU, and every "transfer" between ranks
+is pointer wiring between device buffers.
+"""
+from __future__ import annotations
+
+import ctypes
+from enum import Enum
+from typing import Callable, List, Optional, Sequence
+
+import torch
+
+from . import capi
+from .tensor import Tensor, _prod
+
+
+def _stream_handle(stream: Optional[torch.cuda.Stream]) -> ctypes.c_void_p:
+    s = torch.cuda.current_stream() if stream is None else stream
+    return ctypes.c_void_p(s.cuda_stream)
+
+
+def _ptr(t) -> ctypes.c_void_p:
+    if t is None:
+        return ctypes.c_void_p(0)
+    if isinstance(t, torch.Tensor):
+        return ctypes.c_void_p(t.data_ptr())
+    return ctypes.c_void_p(int(t))
+
+
+def _channel_geometry(t: Tensor):
+    """(num_samples, num_channels, spatial, spatial_real) of a local tensor whose
+    inner spatial dimensions carry no halo -- the layout the batch-norm entry
+    points take (legacy/src/dnn_backend/batchnorm.cu:134-190,210-230)."""
+    nd = t.get_num_dims()
+    for d in range(nd - 3):
+        if t.overlap[d] != 0:
+            raise NotImplementedError("halo on an inner spatial dimension is not supported")
+    if t.overlap[nd - 2] != 0 or t.overlap[nd - 1] != 0:
+        raise NotImplementedError("halo on the channel or sample dimension is not supported")
+    n, c = t.local_shape[nd - 1], t.local_shape[nd - 2]
+    return n, c, _prod(t.local_shape[: nd - 2]), _prod(t.local_real_shape[: nd - 2])
+
+
+class BatchNormalization:
+    """BatchNormalization<Backend, DataType>
+    (legacy/include/distconv/dnn_backend/batchnorm.hpp:100-581).
+
+    ``allreduce``, if given, is called as ``allreduce(list_of_per_channel_tensors)``
+    where the reference sums over ranks (batchnorm.hpp:185-214,360-400); with the
+    default ``None`` the layer is a single rank and the step is the identity.
+    """
+
+    def __init__(self, num_dims: int, decay: float, epsilon: float, global_stats: bool = False,
+                 allreduce: Optional[Callable[[List[torch.Tensor]], None]] = None,
+                 stream: Optional[torch.cuda.Stream] = None):
+        if num_dims not in (4, 5):
+            raise ValueError("4-D (NCHW) or 5-D (NCDHW) tensors only")  # batchnorm.cu:259-270
+        self.num_dims, self.decay, self.epsilon = num_dims, float(decay), float(epsilon)
+        self.global_stats, self.allreduce, self.stream = global_stats, allreduce, stream
+        self.num_current_samples = 0
+        self._lib = capi.load()
+        self._workspace: Optional[torch.Tensor] = None
+        self._workspace_channels = -1
+
+    # batchnorm.hpp:467-475
+    def set_num_samples(self, n: int) -> None:
+        self.num_current_samples = int(n)
+
+    def _ws(self, num_channels: int) -> torch.Tensor:
+        if self._workspace is None or self._workspace_channels != num_channels:
+            nbytes = self._lib.h2x_bn_workspace_bytes(num_channels)
+            self._workspace = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+            capi.check(self._lib.h2x_bn_workspace_init(_ptr(self._workspace), num_channels,
+                                                       _stream_handle(self.stream)), "bn workspace init")
+            self._workspace_channels = num_channels
+        return self._workspace
+
+    def _num_per_sum(self, t: Tensor) -> int:
+        """Elements per channel of the global (global_stats) or local shape
+        (batchnorm.hpp:232-236,414-418)."""
+        nd = t.get_num_dims()
+        shape = t.shape if self.global_stats else t.local_shape
+        return _prod(shape) // shape[nd - 2] if shape[nd - 2] else 0
+
+    # ---- forward -----------------------------------------------------------
+    def forward_stage1(self, input: Tensor, mean: torch.Tensor, var: torch.Tensor,
+                       is_training: bool = True) -> int:
+        self.set_num_samples(input.local_shape[-1])
+        if not is_training:
+            return 0
+        n, c, s, sr = _channel_geometry(input)
+        active = input.is_split_root() and input.get_local_size() > 0
+        capi.check(self._lib.h2x_bn_channel_sums_and_sqsums(
+            input.h2x_dtype, self.num_current_samples if active else 0, c, s, sr,
+            _ptr(input.get_base_ptr()), _ptr(mean), _ptr(var), _ptr(self._ws(c)),
+            _stream_handle(self.stream)), "channel_sums_and_sqsums")
+        return 0
+
+    def forward_allreduce(self, mean: torch.Tensor, var: torch.Tensor, is_training: bool = True) -> int:
+        if is_training and self.global_stats and self.allreduce is not None:
+            self.allreduce([mean, var])
+        return 0
+
+    def forward_stage2(self, input: Tensor, mean, var, running_mean, running_var, scale, bias,
+                       output: Tensor, is_training: bool = True) -> int:
+        n, c, s, sr = _channel_geometry(input)
+        _, _, so, sro = _channel_geometry(output)
+        st = _stream_handle(self.stream)
+        if is_training:
+            capi.check(self._lib.h2x_bn_sums_to_statistics(
+                input.h2x_dtype, c, self._num_per_sum(input), self.decay, _ptr(mean), _ptr(var),
+                _ptr(running_mean), _ptr(running_var), st), "sums_to_statistics")
+            m, v = mean, var
+        else:
+            m, v = running_mean, running_var  # batchnorm.hpp:243-247
+        capi.check(self._lib.h2x_bn_batch_normalization(
+            input.h2x_dtype, self.num_current_samples, c, s, sr, sro, _ptr(input.get_base_ptr()),
+            _ptr(m), _ptr(v), _ptr(scale), _ptr(bias), _ptr(output.get_base_ptr()), self.epsilon, st),
+            "batch_normalization")
+        return 0
+
+    def forward(self, input, mean, var, running_mean, running_var, scale, bias, output,
+                is_training: bool = True) -> int:
+        self.forward_stage1(input, mean, var, is_training)
+        self.forward_allreduce(mean, var, is_training)
+        return self.forward_stage2(input, mean, var, running_mean, running_var, scale, bias, output,
+                                   is_training)
+
+    # ---- backward ----------------------------------------------------------
+    def backward_stage1(self, input: Tensor, d_output: Tensor, mean, var, scale, scale_gradient,
+                        bias_gradient, mean_gradient, var_gradient) -> int:
+        self.set_num_samples(input.local_shape[-1])
+        n, c, s, sr = _channel_geometry(input)
+        _, _, _, sro = _channel_geometry(d_output)
+        active = input.is_split_root() and input.get_local_size() > 0
+        capi.check(self._lib.h2x_bn_backprop1(
+            input.h2x_dtype, self.num_current_samples if active else 0, c, s, sr, sro,
+            _ptr(input.get_base_ptr()), _ptr(d_output.get_base_ptr()), _ptr(mean), _ptr(var),
+            _ptr(scale), _ptr(scale_gradient), _ptr(bias_gradient), _ptr(mean_gradient),
+            _ptr(var_gradient), self.epsilon, _ptr(self._ws(c)), _stream_handle(self.stream)),
+            "backprop1")
+        return 0
+
+    def backward_allreduce(self, scale_gradient, bias_gradient, mean_gradient, var_gradient,
+                           skip_weights: bool = False) -> int:
+        if not self.global_stats or self.allreduce is None:  # batchnorm.hpp:367-368
+            return 0
+        self.allreduce([mean_gradient, var_gradient])
+        if not skip_weights:
+            self.allreduce([scale_gradient])
+            self.allreduce([bias_gradient])
+        return 0
+
+    def backward_stage2(self, input: Tensor, d_output: Tensor, mean, var, scale, mean_gradient,
+                        var_gradient, d_input: Tensor) -> int:
+        n, c, s, sr = _channel_geometry(input)
+        _, _, _, sro = _channel_geometry(d_output)
+        _, _, _, sri = _channel_geometry(d_input)
+        capi.check(self._lib.h2x_bn_backprop2(
+            input.h2x_dtype, self.num_current_samples, c, s, sr, sro, sri, self._num_per_sum(input),
+            _ptr(input.get_base_ptr()), _ptr(d_output.get_base_ptr()), _ptr(mean), _ptr(var),
+            _ptr(scale), _ptr(mean_gradient), _ptr(var_gradient), _ptr(d_input.get_base_ptr()),
+            self.epsilon, _stream_handle(self.stream)), "backprop2")
+        return 0
+
+    def backward(self, input, d_output, mean, var, scale, scale_gradient, bias_gradient,
+                 mean_gradient, var_gradient, d_input) -> int:
+        self.backward_stage1(input, d_output, mean, var, scale, scale_gradient, bias_gradient,
+                             mean_gradient, var_gradient)
+        self.backward_allreduce(scale_gradient, bias_gradient, mean_gradient, var_gradient)
+        return self.backward_stage2(input, d_output, mean, var, scale, mean_gradient, var_gradient,
+                                    d_input)
+
+
+class SoftmaxMode(Enum):
+    """legacy/include/distconv/base.hpp (SoftmaxMode)."""
+    INSTANCE = 0
+    CHANNEL = 1
+
+
+class Softmax:
+    """Softmax<Backend> (legacy/include/distconv/dnn_backend/softmax.hpp:14-63);
+    channel mode only."""
+
+    def __init__(self, stream: Optional[torch.cuda.Stream] = None):
+        self.stream = stream
+        self.mode = SoftmaxMode.CHANNEL
+        self._lib = capi.load()
+
+    def setup(self, input: Tensor, mode: SoftmaxMode) -> None:
+        if mode != SoftmaxMode.CHANNEL:
+            raise NotImplementedError("only SoftmaxMode.CHANNEL is implemented")
+        self.mode = mode
+
+    @staticmethod
+    def _geometry(t: Tensor):
+        if any(t.overlap):
+            raise NotImplementedError("channel softmax assumes a dense local tensor")  # softmax.cu:562-563
+        nd = t.get_num_dims()
+        return t.local_shape[nd - 1], t.local_shape[nd - 2], _prod(t.local_shape[: nd - 2])
+
+    def forward(self, x: Tensor, y: Tensor) -> int:
+        n, c, s = self._geometry(x)
+        capi.check(self._lib.h2x_softmax_channel_forward(
+            x.h2x_dtype, n, c, s, _ptr(x.get_base_ptr()), _ptr(y.get_base_ptr()),
+            _stream_handle(self.stream)), "softmax forward")
+        return 0
+
+    def backward(self, y: Tensor, dy: Tensor, dx: Tensor) -> int:
+        n, c, s = self._geometry(dx)
+        capi.check(self._lib.h2x_softmax_channel_backward(
+            y.h2x_dtype, n, c, s, _ptr(y.get_base_ptr()), _ptr(dy.get_base_ptr()),
+            _ptr(dx.get_base_ptr()), _stream_handle(self.stream)), "softmax backward")
+        return 0
+
+
+class HaloExchangeAccumOp(Enum):
+    """legacy/include/distconv/tensor/halo_exchange.hpp:8-9."""
+    ID = capi.HALO_ID
+    SUM = capi.HALO_SUM
+    MAX = capi.HALO_MAX
+    MIN = capi.HALO_MIN
+
+
+class HaloExchangeVirtual:
+    """HaloExchange for all virtual ranks of one distributed tensor
+    (legacy/include/distconv/tensor/halo_exchange_cuda.hpp:18-423).
+
+    The reference object belongs to one rank and hands packed strips to a
+    transport.  Here the object holds every rank's local tensor; rank r's send
+    buffer for (dim, side) *is* the receive buffer of its neighbour on that
+    side for the opposite side, so the transfer is free, and each dimension
+    phase is two launches (pack all ranks and sides, unpack all ranks and
+    sides).  ``periodic`` wraps neighbours at the grid edge; the reference
+    never does (MPI_PROC_NULL, halo_exchange_cuda.hpp:343-345).
+    """
+
+    def __init__(self, tensors: Sequence[Tensor], periodic: bool = False,
+                 stream: Optional[torch.cuda.Stream] = None):
+        self.tensors = list(tensors)
+        self.periodic, self.stream = periodic, stream
+        self._lib = capi.load()
+        t0 = self.tensors[0]
+        self.dist = t0.dist
+        if len(self.tensors) != self.dist.num_ranks:
+            raise ValueError("one local tensor per rank of the distribution is required")
+        if t0.dist.num_ranks != _prod(t0.dist.split_shape):
+            raise NotImplementedError("shared (replicated) distributions are not exchanged")  # :30-31
+        self.nd = t0.get_num_dims()
+        self._recv = {}  # (rank, dim, side) -> torch buffer the rank unpacks from
+
+    def get_halo_size(self, rank: int, dim: int, width: int) -> int:
+        """halo_exchange_cuda.hpp:267-271."""
+        shape = list(self.tensors[rank].local_real_shape)
+        shape[dim] = width
+        return _prod(shape)
+
+    def is_exchange_required(self, rank: int, dim: int, widths=None) -> bool:
+        """halo_exchange_cuda.hpp:305-320."""
+        t = self.tensors[rank]
+        w = t.overlap[dim] if widths is None else max(widths)
+        return self.dist.is_distributed(dim) and self.dist.split_shape[dim] > 1 and w > 0 \
+            and t.get_local_size() > 0
+
+    def find_peer_rank(self, rank: int, dim: int, side: int) -> Optional[int]:
+        """halo_exchange_cuda.hpp:322-357; None stands for MPI_PROC_NULL."""
+        t = self.tensors[rank]
+        if not self.is_exchange_required(rank, dim):
+            return None
+        extent = self.dist.locale_shape[dim]
+        p = t.proc_index[dim] + (1 if side == capi.RHS else -1)
+        if p < 0 or p >= extent:
+            if not self.periodic:
+                return None
+            p %= extent
+        idx = list(t.proc_index)
+        idx[dim] = p
+        peer = self.dist.rank_of(idx)
+        if self.tensors[peer].get_local_size() == 0:
+            return None
+        return peer
+
+    def _recv_buffer(self, rank: int, dim: int, side: int) -> torch.Tensor:
+        key = (rank, dim, side)
+        if key not in self._recv:
+            t = self.tensors[rank]
+            n = self.get_halo_size(rank, dim, t.overlap[dim])  # sized for the full halo (:285-303)
+            self._recv[key] = torch.zeros(max(n, 1), dtype=t.dtype, device=t.device)
+        return self._recv[key]
+
+    def _face(self, rank, dim, side, width, buf, is_pack, is_reverse, op) -> capi.HaloFace:
+        t = self.tensors[rank]
+        f = capi.HaloFace()
+        f.tensor = t.get_buffer()
+        f.buffer = buf.data_ptr()
+        for i, e in enumerate(t.local_real_shape):
+            f.real_shape[i] = e
+        f.num_dims, f.dim, f.side, f.width = self.nd, dim, side, width
+        f.inner = int((is_pack and not is_reverse) or ((not is_pack) and is_reverse))
+        f.is_pack, f.op = int(is_pack), op.value
+        return f
+
+    def _run(self, faces: List[capi.HaloFace], dtype: int) -> None:
+        if not faces:
+            return
+        arr = (capi.HaloFace * len(faces))(*faces)
+        capi.check(self._lib.h2x_halo_pack_or_unpack_batched(dtype, arr, len(faces),
+                                                             _stream_handle(self.stream)),
+                   "halo pack/unpack")
+
+    def exchange_dim(self, dim: int, width_rhs_send: int, width_rhs_recv: int, width_lhs_send: int,
+                     width_lhs_recv: int, is_reverse: bool = False, skip_unpack: bool = False,
+                     op: HaloExchangeAccumOp = HaloExchangeAccumOp.ID) -> None:
+        """One dimension for all ranks; the order pack -> (transfer) -> unpack of
+        halo_exchange_cuda_mpi.hpp:25-100.  A rank's RHS strip goes to its RHS
+        neighbour's LHS receive buffer and vice versa."""
+        dtype = self.tensors[0].h2x_dtype
+        packs, unpacks = [], []
+        for r, t in enumerate(self.tensors):
+            if not self.is_exchange_required(
+                    r, dim, (width_rhs_send, width_rhs_recv, width_lhs_send, width_lhs_recv)):
+                continue
+            for side in (capi.LHS, capi.RHS):
+                peer = self.find_peer_rank(r, dim, side)
+                if peer is None:
+                    continue
+                w_send = width_rhs_send if side == capi.RHS else width_lhs_send
+                w_recv = width_rhs_recv if side == capi.RHS else width_lhs_recv
+                if w_send > 0:
+                    dst = self._recv_buffer(peer, dim, capi.LHS if side == capi.RHS else capi.RHS)
+                    packs.append(self._face(r, dim, side, w_send, dst, True, is_reverse, op))
+                if w_recv > 0 and not skip_unpack:
+                    src = self._recv_buffer(r, dim, side)
+                    unpacks.append(self._face(r, dim, side, w_recv, src, False, is_reverse, op))
+        self._run(packs, dtype)
+        self._run(unpacks, dtype)
+
+    def exchange(self, widths_rhs_send=None, widths_rhs_recv=None, widths_lhs_send=None,
+                 widths_lhs_recv=None, is_reverse: bool = False, skip_unpack: bool = False,
+                 op: HaloExchangeAccumOp = HaloExchangeAccumOp.ID) -> None:
+        """All dimensions, innermost first, each seeing the halo cells the previous
+        ones filled (halo_exchange_cuda.hpp:56-106)."""
+        ov = self.tensors[0].overlap
+        wrs = ov if widths_rhs_send is None else widths_rhs_send
+        wrr = ov if widths_rhs_recv is None else widths_rhs_recv
+        wls = ov if widths_lhs_send is None else widths_lhs_send
+        wlr = ov if widths_lhs_recv is None else widths_lhs_recv
+        for d in range(self.nd):
+            self.exchange_dim(d, wrs[d], wrr[d], wls[d], wlr[d], is_reverse, skip_unpack, op)
+
+    def clear_halo(self, dim: int) -> None:
+        """Tensor::clear_halo (legacy/src/tensor/tensor_mpi_cuda.cu:14-84) on every rank."""
+        for t in self.tensors:
+            if t.overlap[dim] == 0 or t.get_local_size() == 0:
+                continue
+            shape = capi.i64_array(t.local_real_shape)
+            capi.check(self._lib.h2x_halo_clear(t.h2x_dtype, _ptr(t.get_buffer()), self.nd, shape,
+                                                dim, t.overlap[dim], _stream_handle(self.stream)),
+                       "clear_halo")
+
+
+class TensorShufflerVirtual:
+    """TensorMPICUDAShuffler for all virtual ranks of a (src, dst) pair of
+    distributed tensors (legacy/include/distconv/tensor/shuffle_mpi_cuda.hpp:14-512,
+    legacy/src/tensor/shuffle_mpi_cuda.cu:378-476).
+
+    The tables are the reference constructor's (rank_limits per dimension,
+    counts and displacements in rank order).  All ranks' receive buffers live in
+    one arena and every rank packs straight into its peers' chunks of it -- the
+    all-to-all of the reference's ``transfer`` is therefore free -- and each
+    direction is two launches: pack for all ranks, unpack for all ranks.
+    """
+
+    def __init__(self, src_tensors: Sequence[Tensor], dst_tensors: Sequence[Tensor],
+                 stream: Optional[torch.cuda.Stream] = None):
+        self.src, self.dst, self.stream = list(src_tensors), list(dst_tensors), stream
+        self._lib = capi.load()
+        if len(self.src) != len(self.dst):
+            raise ValueError("source and destination must have the same number of ranks")
+        self.num_ranks = len(self.src)
+        self.elem_size = torch.empty(0, dtype=self.src[0].dtype).element_size()
+        self._keep = []  # ctypes arrays referenced by geometries
+        self._fwd = self._direction(self.src, self.dst)
+        self._bwd = self._direction(self.dst, self.src)
+
+    @staticmethod
+    def get_buf_size(t: Tensor) -> int:
+        """shuffle_mpi_cuda.hpp:83-90 (bytes)."""
+        return t.get_local_size() * torch.empty(0, dtype=t.dtype).element_size()
+
+    # -- tables (shuffle_mpi_cuda.hpp:129-287) --------------------------------
+    @staticmethod
+    def rank_limits(a: Tensor, b: Tensor) -> List[int]:
+        """End, in a's local coordinates, of each slab of b's process grid."""
+        out = []
+        for d in range(a.get_num_dims()):
+            extent = b.dist.locale_shape[d]
+            per = b.dist.get_num_ranks_per_split(d)
+            for j in range(extent):
+                nxt_root = (j // per + 1) * per  # next split root after j
+                nxt = b.get_dimension_rank_offset(d, nxt_root) if nxt_root < extent else b.shape[d]
+                lim = 0 if nxt < a.global_index[d] else min(nxt - a.global_index[d], a.local_shape[d])
+                out.append(lim)
+        return out
+
+    @staticmethod
+    def _overlap_size(a: Tensor, b: Tensor, b_index: Sequence[int]) -> int:
+        size = 1
+        for d in range(a.get_num_dims()):
+            b0 = b.get_dimension_rank_offset(d, b_index[d])
+            b1 = b0 + b.get_remote_dimension(d, b_index[d])
+            lo, hi = max(a.global_index[d], b0), min(a.global_index[d] + a.local_shape[d], b1)
+            size *= max(hi - lo, 0)
+        return size
+
+    def _counts(self, a: Tensor, b: Tensor) -> List[int]:
+        """Elements rank a exchanges with every rank of b's grid, in rank order."""
+        counts = []
+        for pid in range(self.num_ranks):
+            idx = b.dist.rank_index(pid)
+            ok = a.is_split_root() and b.dist.is_split_root_index(idx)
+            counts.append(self._overlap_size(a, b, idx) if ok else 0)
+        return counts
+
+    def _direction(self, src: List[Tensor], dst: List[Tensor]):
+        """Plans and buffers for src -> dst."""
+        n = self.num_ranks
+        send_counts = [self._counts(src[r], dst[r]) for r in range(n)]
+        recv_counts = [self._counts(dst[r], src[r]) for r in range(n)]
+        for r in range(n):
+            for p in range(n):
+                assert send_counts[r][p] == recv_counts[p][r]
+        recv_displs = [[sum(recv_counts[r][:p]) for p in range(n)] for r in range(n)]
+        recv_sizes = [sum(recv_counts[r]) for r in range(n)]
+        arena_offsets = [sum(recv_sizes[:r]) for r in range(n)]
+        arena = torch.zeros(max(sum(recv_sizes), 1), dtype=src[0].dtype, device=src[0].device)
+        if sum(recv_sizes) >= 2 ** 31:
+            raise ValueError("arena exceeds the 32-bit displacements of the shuffler tables")
+        pack_plans, unpack_plans = [], []
+        for r in range(n):
+            # pack: chunk for peer p lands in p's receive buffer at the slot reserved for r
+            displs = [arena_offsets[p] + recv_displs[p][r] for p in range(n)]
+            pack_plans.append(self._plan(src[r], dst[r], self.rank_limits(src[r], dst[r]), displs)
+                              if src[r].is_split_root() and src[r].get_local_size() > 0 else None)
+            displs = [arena_offsets[r] + recv_displs[r][p] for p in range(n)]
+            unpack_plans.append(self._plan(dst[r], src[r], self.rank_limits(dst[r], src[r]), displs)
+                                if dst[r].is_split_root() and dst[r].get_local_size() > 0 else None)
+        return dict(arena=arena, pack=pack_plans, unpack=unpack_plans,
+                    send_counts=send_counts, recv_counts=recv_counts, recv_displs=recv_displs)
+
+    def _plan(self, mine: Tensor, other: Tensor, limits: List[int], displs: List[int]):
+        g = capi.ShuffleGeometry()
+        g.num_dims, g.elem_size = mine.get_num_dims(), self.elem_size
+        for i in range(mine.get_num_dims()):
+            g.local_shape[i] = mine.local_shape[i]
+            g.strides[i] = mine.get_strides()[i]
+            g.peer_locale_shape[i] = other.dist.locale_shape[i]
+        rl = (ctypes.c_int32 * len(limits))(*limits)
+        dp = (ctypes.c_int32 * len(displs))(*displs)
+        g.rank_limits, g.displs = rl, dp
+        plan = ctypes.c_void_p()
+        capi.check(self._lib.h2x_shuffle_plan_create(ctypes.byref(g), ctypes.byref(plan)),
+                   "shuffle plan")
+        return plan
+
+    def _launch(self, fn, plans, tensors: List[Tensor], arena: torch.Tensor) -> None:
+        live = [(p, t) for p, t in zip(plans, tensors) if p is not None]
+        if not live:
+            return
+        n = len(live)
+        pa = (ctypes.c_void_p * n)(*[p for p, _ in live])
+        ta = (ctypes.c_void_p * n)(*[t.get_base_ptr() for _, t in live])
+        ba = (ctypes.c_void_p * n)(*[arena.data_ptr()] * n)
+        capi.check(fn(pa, ta, ba, n, _stream_handle(self.stream)), "shuffle")
+
+    def shuffle_forward(self) -> None:
+        """src tensors -> dst tensors (shuffle_mpi_cuda.cu:478-484)."""
+        d = self._fwd
+        self._launch(self._lib.h2x_shuffle_pack_batched, d["pack"], self.src, d["arena"])
+        self._launch(self._lib.h2x_shuffle_unpack_batched, d["unpack"], self.dst, d["arena"])
+
+    def shuffle_backward(self) -> None:
+        """dst tensors -> src tensors (shuffle_mpi_cuda.cu:485-490)."""
+        d = self._bwd
+        self._launch(self._lib.h2x_shuffle_pack_batched, d["pack"], self.dst, d["arena"])
+        self._launch(self._lib.h2x_shuffle_unpack_batched, d["unpack"], self.src, d["arena"])
+
+    def __del__(self):
+        try:
+            for d in (self._fwd, self._bwd):
+                for p in d["pack"] + d["unpack"]:
+                    if p is not None:
+                        self._lib.h2x_shuffle_plan_destroy(p)
+        except Exception:
+            pass

@@ -1,0 +1,392 @@
+/*
+ * h2x.h -- C ABI of the MI355X (gfx950) implementation of DistConv's
+ * data-parallel, non-convolution hot path: channel-wise batch-norm statistics
+ * (forward and backward), halo pack/unpack of spatially decomposed tensors,
+ * channel softmax (forward and backward) and the tensor-shuffler pack/unpack.
+ *
+ * Every entry point takes plain device pointers, sizes and a HIP stream, is
+ * asynchronous on that stream, performs no device synchronisation and no
+ * allocation unless stated, and returns 0 on success, a positive hipError_t
+ * value when the HIP runtime reported an error, or a negative h2x_status.
+ * The library never aborts the process.
+ *
+ * Conventions shared with the reference (paths relative to the reference
+ * checkout):
+ *   - dimension order is innermost first: an "NCHW" tensor has shape
+ *     {W, H, C, N}; channel is dimension nd-2, sample is nd-1
+ *     (legacy/include/distconv/distconv.hpp:103-109);
+ *   - "real" shape = local shape + 2 * halo width per dimension
+ *     (legacy/include/distconv/tensor/tensor_mpi.hpp:497-498);
+ *   - LHS = 0, RHS = 1 (legacy/include/distconv/base.hpp:23).
+ */
+#ifndef H2X_H_INCLUDED
+#define H2X_H_INCLUDED
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define H2X_MAX_DIMS 6
+
+/** A hipStream_t passed through an opaque pointer (NULL = the null stream). */
+typedef void* h2x_stream_t;
+
+typedef enum h2x_status
+{
+    H2X_SUCCESS = 0,
+    H2X_ERR_INVALID_ARGUMENT = -1,
+    H2X_ERR_UNSUPPORTED = -2,
+    H2X_ERR_TOO_LARGE = -3
+} h2x_status;
+
+/** Element type of floating-point tensors (batch-norm, softmax, halo accumulate). */
+typedef enum h2x_dtype
+{
+    H2X_F32 = 0,
+    H2X_F64 = 1
+} h2x_dtype;
+
+/** legacy/include/distconv/base.hpp:23 */
+typedef enum h2x_side
+{
+    H2X_LHS = 0,
+    H2X_RHS = 1
+} h2x_side;
+
+/** legacy/include/distconv/tensor/halo_exchange.hpp:8-9 */
+typedef enum h2x_halo_op
+{
+    H2X_HALO_ID = 0,
+    H2X_HALO_SUM = 1,
+    H2X_HALO_MAX = 2,
+    H2X_HALO_MIN = 3
+} h2x_halo_op;
+
+/* ------------------------------------------------------------------------ */
+/* Library                                                                   */
+/* ------------------------------------------------------------------------ */
+
+/** ABI version of this header; bumped on any incompatible change. */
+int h2x_abi_version(void);
+
+/** Human-readable text for a value returned by any h2x_* function. */
+const char* h2x_status_string(int status);
+
+/* ------------------------------------------------------------------------ */
+/* Batch normalisation                                                       */
+/*                                                                           */
+/* Tensor geometry of x, y, dy, dx: element (n, c, i) of the local tensor    */
+/* lives at base[(n * num_channels + c) * spatial_real_size + i] for         */
+/* 0 <= i < spatial_size.  spatial_size is the product of the local spatial  */
+/* extents, spatial_real_size the same product over the real (haloed)        */
+/* extents; they differ only when the outermost spatial dimension carries a  */
+/* halo, and `base` then is the tensor's get_base_ptr().  This is the        */
+/* geometry the reference's optimised kernels accept                         */
+/* (legacy/src/dnn_backend/batchnorm.cu:134-190,210-230).                    */
+/* Per-channel vectors (sums, mean, var, scale, ...) are dense arrays of     */
+/* num_channels elements.                                                    */
+/* ------------------------------------------------------------------------ */
+
+/**
+ * Bytes of device workspace the two reduction entry points need for
+ * `num_channels` channels.  The workspace holds per-workgroup partial sums
+ * and one completion counter per channel.  It must be cleared once with
+ * h2x_bn_workspace_init before its first use; afterwards the kernels leave it
+ * ready for the next call.  One workspace must not be used by two calls that
+ * may run concurrently.
+ */
+size_t h2x_bn_workspace_bytes(int num_channels);
+
+/** Clears a workspace of h2x_bn_workspace_bytes(num_channels) bytes (fill kernel, no memset node). */
+int h2x_bn_workspace_init(void* workspace, int num_channels, h2x_stream_t stream);
+
+/**
+ * sums[c] = sum over (n, i) of x; sqsums[c] = sum of x*x.
+ * Replaces batchnorm::channel_sums_and_sqsums
+ * (legacy/include/distconv/dnn_backend/batchnorm.hpp:22-28,
+ *  legacy/src/dnn_backend/batchnorm.cu:192-271).  Outputs are overwritten
+ * (the reference zeroes them and accumulates with atomics); with
+ * num_samples == 0 or spatial_size == 0 they are set to zero.  Accumulation
+ * is in fp64 with a fixed reduction order, so results are run-to-run
+ * deterministic.
+ */
+int h2x_bn_channel_sums_and_sqsums(h2x_dtype dtype,
+                                   int num_samples,
+                                   int num_channels,
+                                   size_t spatial_size,
+                                   size_t spatial_real_size,
+                                   const void* x,
+                                   void* sums,
+                                   void* sqsums,
+                                   void* workspace,
+                                   h2x_stream_t stream);
+
+/**
+ * In place: mean = sums / n; var = max(sqsums / n - mean^2, 0) * n / (n - 1);
+ * running_x = decay * running_x + (1 - decay) * x.  With num_per_sum == 0
+ * only var is written (set to 1).  Replaces batchnorm::sums_to_statistics
+ * (batchnorm.hpp:30-37, batchnorm.cu:288-346).
+ */
+int h2x_bn_sums_to_statistics(h2x_dtype dtype,
+                              int num_channels,
+                              size_t num_per_sum,
+                              double decay,
+                              void* mean_inout,
+                              void* var_inout,
+                              void* running_mean,
+                              void* running_var,
+                              h2x_stream_t stream);
+
+/**
+ * y = (x - mean) * rsqrt(var + epsilon) * scale + bias.
+ * Replaces batchnorm::batch_normalization (batchnorm.hpp:39-49,
+ * batchnorm.cu:420-573).  x and y have their own real sizes.
+ */
+int h2x_bn_batch_normalization(h2x_dtype dtype,
+                               int num_samples,
+                               int num_channels,
+                               size_t spatial_size,
+                               size_t x_spatial_real_size,
+                               size_t y_spatial_real_size,
+                               const void* x,
+                               const void* mean,
+                               const void* var,
+                               const void* scale,
+                               const void* bias,
+                               void* y,
+                               double epsilon,
+                               h2x_stream_t stream);
+
+/**
+ * Backward reductions per channel (r = rsqrt(var + epsilon)):
+ *   dscale = sum dy * (x - mean) * r;   dbias = sum dy;
+ *   dmean  = - sum dy * scale * r;
+ *   dvar   = - sum dy * scale * (x - mean) * r^3 / 2.
+ * Replaces batchnorm::backprop1 (batchnorm.hpp:68-81, batchnorm.cu:982-1230).
+ * Outputs are overwritten; fp64 accumulation, deterministic.
+ */
+int h2x_bn_backprop1(h2x_dtype dtype,
+                     int num_samples,
+                     int num_channels,
+                     size_t spatial_size,
+                     size_t x_spatial_real_size,
+                     size_t dy_spatial_real_size,
+                     const void* x,
+                     const void* dy,
+                     const void* mean,
+                     const void* var,
+                     const void* scale,
+                     void* dscale,
+                     void* dbias,
+                     void* dmean,
+                     void* dvar,
+                     double epsilon,
+                     void* workspace,
+                     h2x_stream_t stream);
+
+/**
+ * dx = dy * scale * r + dmean / n + dvar * 2 / (n - 1) * (x - mean), with
+ * n = num_per_sum.  dx may alias x.  Replaces batchnorm::backprop2
+ * (batchnorm.hpp:83-96, batchnorm.cu:1371-1559).
+ */
+int h2x_bn_backprop2(h2x_dtype dtype,
+                     int num_samples,
+                     int num_channels,
+                     size_t spatial_size,
+                     size_t x_spatial_real_size,
+                     size_t dy_spatial_real_size,
+                     size_t dx_spatial_real_size,
+                     size_t num_per_sum,
+                     const void* x,
+                     const void* dy,
+                     const void* mean,
+                     const void* var,
+                     const void* scale,
+                     const void* dmean,
+                     const void* dvar,
+                     void* dx,
+                     double epsilon,
+                     h2x_stream_t stream);
+
+/* ------------------------------------------------------------------------ */
+/* Channel softmax: dense [num_samples][num_channels][spatial_size] tensors,  */
+/* softmax taken over the channel dimension.                                  */
+/* ------------------------------------------------------------------------ */
+
+/**
+ * m = max(FLT_MIN, max_c x); e = exp(x - m); y = max(e * (1 / sum_c e), FLT_MIN)
+ * (DBL_MIN for f64).  Replaces Softmax::forward in SoftmaxMode::CHANNEL
+ * (legacy/src/dnn_backend/softmax.cu:538-619,705-747).
+ */
+int h2x_softmax_channel_forward(h2x_dtype dtype,
+                                int num_samples,
+                                int num_channels,
+                                size_t spatial_size,
+                                const void* x,
+                                void* y,
+                                h2x_stream_t stream);
+
+/**
+ * dp = sum_c y * dy; dx = y > FLT_MIN ? y * (dy - dp) : 0.
+ * Replaces Softmax::backward in SoftmaxMode::CHANNEL
+ * (legacy/src/dnn_backend/softmax.cu:621-701,749-768).
+ */
+int h2x_softmax_channel_backward(h2x_dtype dtype,
+                                 int num_samples,
+                                 int num_channels,
+                                 size_t spatial_size,
+                                 const void* y,
+                                 const void* dy,
+                                 void* dx,
+                                 h2x_stream_t stream);
+
+/* ------------------------------------------------------------------------ */
+/* Halo pack / unpack                                                        */
+/* ------------------------------------------------------------------------ */
+
+/**
+ * One halo strip of one tensor.  `tensor` is the start of the real (haloed)
+ * allocation (get_buffer()), `real_shape` its real extents, innermost first.
+ * The strip is `width` cells thick along `dim`, spans the full real extent of
+ * every other dimension and starts, along `dim`, at
+ *   LHS outer: 0              LHS inner: width
+ *   RHS outer: shape - width  RHS inner: shape - 2 * width
+ * (legacy/include/distconv/tensor/halo_cuda.hpp:59-81).  `buffer` holds the
+ * strip in natural (innermost-first) order of the strip's own extents, the
+ * layout of the reference's generic traversal (halo_cuda.hpp:53-86).
+ * pack:   buffer[o] = tensor[strip(o)]
+ * unpack: tensor[strip(o)] = op(tensor[strip(o)], buffer[o])
+ * (legacy/include/distconv/tensor/halo_packing_cuda.hpp:60-83).
+ */
+typedef struct h2x_halo_face
+{
+    void* tensor;
+    void* buffer;
+    int64_t real_shape[H2X_MAX_DIMS];
+    int32_t num_dims;
+    int32_t dim;
+    int32_t side;    /* h2x_side */
+    int32_t width;
+    int32_t inner;   /* 0: outer (halo) strip, 1: inner (boundary) strip */
+    int32_t is_pack; /* 1: tensor -> buffer, 0: buffer -> tensor */
+    int32_t op;      /* h2x_halo_op, used when unpacking */
+    int32_t reserved;
+} h2x_halo_face;
+
+/** Number of elements of the strip described by (real_shape, dim, width): legacy/include/distconv/tensor/halo_exchange_cuda.hpp:267-271. */
+size_t h2x_halo_size(int num_dims, const int64_t* real_shape, int dim, int width);
+
+/**
+ * Pack or unpack one strip.  `inner` follows
+ * (is_pack && !is_reverse) || (!is_pack && is_reverse)
+ * (halo_packing_cuda.hpp:100); width == 0 is a no-op.  Replaces
+ * halo_exchange_cuda::pack_or_unpack<T> (halo_packing_cuda.hpp:143-167,
+ * legacy/src/tensor/halo_exchange_cuda.cu:12-40).
+ */
+int h2x_halo_pack_or_unpack(h2x_dtype dtype,
+                            void* tensor,
+                            int num_dims,
+                            const int64_t* real_shape,
+                            int dim,
+                            int side,
+                            int width,
+                            void* buffer,
+                            int is_pack,
+                            int is_reverse,
+                            int op,
+                            h2x_stream_t stream);
+
+/**
+ * The same for `num_faces` independent strips in as few launches as possible
+ * (both sides of a dimension, several tensors).  Faces of one call must not
+ * overlap in what they write.  `faces` is host memory, read before return.
+ */
+int h2x_halo_pack_or_unpack_batched(h2x_dtype dtype,
+                                    const h2x_halo_face* faces,
+                                    int num_faces,
+                                    h2x_stream_t stream);
+
+/**
+ * tensor[strip] = 0 for the outer strips of `dim` on both sides, width =
+ * the real halo width.  Replaces TensorImplHelper::clear_halo
+ * (legacy/src/tensor/tensor_mpi_cuda.cu:14-84).
+ */
+int h2x_halo_clear(h2x_dtype dtype,
+                   void* tensor,
+                   int num_dims,
+                   const int64_t* real_shape,
+                   int dim,
+                   int width,
+                   h2x_stream_t stream);
+
+/* ------------------------------------------------------------------------ */
+/* Tensor shuffler pack / unpack                                             */
+/* ------------------------------------------------------------------------ */
+
+/**
+ * Geometry of one rank's side of a shuffle, taken from the tables the
+ * reference's shuffler constructor builds
+ * (legacy/include/distconv/tensor/shuffle_mpi_cuda.hpp:129-287):
+ * the rank's local tensor is cut into one box per peer rank; box p is sent to
+ * (pack) or received from (unpack) peer p and lives at displs[p] elements in
+ * the staging buffer, in natural order of the box's own extents -- the order
+ * find_destination produces (legacy/src/tensor/shuffle_mpi_cuda.cu:42-98).
+ */
+typedef struct h2x_shuffle_geometry
+{
+    int32_t num_dims;
+    int32_t elem_size;                     /* bytes per element: 2, 4 or 8 */
+    int64_t local_shape[H2X_MAX_DIMS];     /* local (halo-free) extents */
+    int64_t strides[H2X_MAX_DIMS];         /* element strides of the real tensor (get_strides()) */
+    int64_t peer_locale_shape[H2X_MAX_DIMS]; /* process grid of the other side */
+    /* rank_limits[d][j]: end, in local coordinates of dimension d, of the slab
+     * that belongs to index j of the peer grid along d; concatenated over d
+     * (sum of peer_locale_shape entries).  Plain limits only: the reference's
+     * "-1" encoding for evenly partitioned grids of >= 16 ranks is a lookup
+     * optimisation with the same meaning (shuffle_mpi_cuda.hpp:175-213). */
+    const int32_t* rank_limits;
+    /* displs[p]: offset (elements) of peer p's chunk, p in rank order of the
+     * peer grid (dimension 0 fastest); product of peer_locale_shape entries. */
+    const int32_t* displs;
+} h2x_shuffle_geometry;
+
+typedef struct h2x_shuffle_plan h2x_shuffle_plan;
+
+/**
+ * Builds the device-side box table for one geometry.  Allocates a few hundred
+ * bytes of device memory and copies synchronously; call once per shuffler.
+ */
+int h2x_shuffle_plan_create(const h2x_shuffle_geometry* geometry, h2x_shuffle_plan** plan);
+int h2x_shuffle_plan_destroy(h2x_shuffle_plan* plan);
+
+/**
+ * buffer[displs[p] + o] = tensor[box_p(o)] for every peer p.  `tensor` is the
+ * get_base_ptr() of the local tensor (first interior element).  Replaces
+ * pack<T, packed> (legacy/src/tensor/shuffle_mpi_cuda.cu:114-248).
+ */
+int h2x_shuffle_pack(const h2x_shuffle_plan* plan, const void* tensor, void* buffer, h2x_stream_t stream);
+
+/**
+ * tensor[box_p(o)] = buffer[displs[p] + o].  Replaces unpack<T, packed>
+ * (legacy/src/tensor/shuffle_mpi_cuda.cu:251-372).
+ */
+int h2x_shuffle_unpack(const h2x_shuffle_plan* plan, void* tensor, const void* buffer, h2x_stream_t stream);
+
+/**
+ * Several ranks' pack (or unpack) steps in one launch: plan i is applied to
+ * tensors[i] and buffers[i].  Pointer arrays are host memory.  For virtual
+ * ranks living on one GPU; what each plan does is unchanged.
+ */
+int h2x_shuffle_pack_batched(const h2x_shuffle_plan* const* plans, const void* const* tensors,
+                             void* const* buffers, int num_plans, h2x_stream_t stream);
+int h2x_shuffle_unpack_batched(const h2x_shuffle_plan* const* plans, void* const* tensors,
+                               const void* const* buffers, int num_plans, h2x_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* H2X_H_INCLUDED */

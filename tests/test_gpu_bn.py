@@ -1,0 +1,175 @@
+"""GPU parity: batch-norm entry points of libh2x.so against the CPU oracle.
+
+Tolerance: 1e-5 relative with the reference's metric max(|d/v1|, |d/v2|)
+(legacy/tests/compare_binary_files.cpp:47-49, legacy/tests/dnn_backend/
+test_cudnn_util.sh.in:64-72 uses 1.5e-5).  The oracle performs the same fp32
+operations in the same order with fp64 accumulation, so the match is in fact
+much tighter; the asserted bound is the contract.
+"""
+import numpy as np
+import pytest
+
+from helpers import bn_inputs, max_rel
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-5
+
+CASES = [
+    # (N, C, spatial dims...) numpy order
+    (8, 64, 56, 56),        # BASELINE config 1
+    (2, 3, 4, 5),           # tiny, spatial % 4 == 0
+    (2, 3, 5, 7),           # scalar path (spatial % 4 != 0)
+    (3, 5, 3, 4, 5),        # 5-D
+    (1, 1, 1, 1),           # n == 1: unbiased variance is 0 * inf = NaN in the reference too
+    (64, 16, 7, 7),         # more samples than chunks
+    (2, 130, 33, 31),       # many channels, odd sizes
+    (4, 8, 16, 16, 16),     # 5-D vector path
+]
+
+
+def _run_forward(x, scale, bias, eps=1e-5, decay=0.9, dtype="float32"):
+    import torch
+    from dihydrogen_amd.layers import BatchNormalization
+    from dihydrogen_amd.tensor import Distribution, LocaleVirtual, Tensor
+
+    nd = x.ndim
+    shape = list(x.shape[::-1])
+    tdt = getattr(torch, dtype)
+    dist = Distribution.make_localized_distribution(nd)
+    loc = LocaleVirtual(0, 1)
+    xin = Tensor(shape, loc, dist, tdt).allocate()
+    yout = Tensor(shape, loc, dist, tdt).allocate()
+    xin.real_view().copy_(torch.from_numpy(x))
+    c = x.shape[1]
+    dev = lambda a: torch.from_numpy(a.copy()).cuda()
+    mean = torch.empty(c, dtype=tdt, device="cuda")
+    var = torch.empty(c, dtype=tdt, device="cuda")
+    rm = torch.zeros(c, dtype=tdt, device="cuda")
+    rv = torch.ones(c, dtype=tdt, device="cuda")
+    bn = BatchNormalization(nd, decay, eps)
+    assert bn.forward(xin, mean, var, rm, rv, dev(scale), dev(bias), yout, True) == 0
+    torch.cuda.synchronize()
+    return bn, xin, yout, mean, var, rm, rv
+
+
+@pytest.mark.parametrize("shape", CASES)
+def test_forward_matches_oracle(shape, oracle_mod):
+    x, dy, scale, bias = bn_inputs(shape, seed=1234)
+    bn, xin, yout, mean, var, rm, rv = _run_forward(x, scale, bias)
+    rm_o = np.zeros(shape[1], np.float32)
+    rv_o = np.ones(shape[1], np.float32)
+    y_o, mean_o, var_o = oracle_mod.bn_forward(x, scale, bias, rm_o, rv_o, 1e-5, 0.9)
+    got = lambda t: t.cpu().numpy()
+    if int(np.prod(shape)) // shape[1] == 1:
+        assert np.isnan(got(var)).all() and np.isnan(var_o).all()
+        return
+    assert max_rel(got(mean), mean_o) <= TOL
+    assert max_rel(got(var), var_o) <= TOL
+    assert max_rel(got(rm), rm_o) <= TOL
+    assert max_rel(got(rv), rv_o) <= TOL
+    assert max_rel(got(yout.real_view()), y_o) <= TOL
+
+
+@pytest.mark.parametrize("shape", CASES)
+def test_backward_matches_oracle(shape, oracle_mod):
+    import torch
+    from dihydrogen_amd.tensor import Distribution, LocaleVirtual, Tensor
+
+    if int(np.prod(shape)) // shape[1] == 1:
+        pytest.skip("n == 1 gives NaN statistics")
+    x, dy, scale, bias = bn_inputs(shape, seed=4321)
+    bn, xin, yout, mean, var, rm, rv = _run_forward(x, scale, bias)
+    c = shape[1]
+    dist = Distribution.make_localized_distribution(x.ndim)
+    loc = LocaleVirtual(0, 1)
+    dyt = Tensor(list(x.shape[::-1]), loc, dist).allocate()
+    dxt = Tensor(list(x.shape[::-1]), loc, dist).allocate()
+    dyt.real_view().copy_(torch.from_numpy(dy))
+    outs = [torch.empty(c, device="cuda") for _ in range(4)]
+    sc = torch.from_numpy(scale).cuda()
+    assert bn.backward(xin, dyt, mean, var, sc, outs[0], outs[1], outs[2], outs[3], dxt) == 0
+    torch.cuda.synchronize()
+    mean_h, var_h = mean.cpu().numpy(), var.cpu().numpy()
+    dx_o, dscale_o, dbias_o, dmean_o, dvar_o = oracle_mod.bn_backward(x, dy, mean_h, var_h, scale, 1e-5)
+    for got, want, name in zip(outs, (dscale_o, dbias_o, dmean_o, dvar_o),
+                               ("dscale", "dbias", "dmean", "dvar")):
+        assert max_rel(got.cpu().numpy(), want) <= TOL, name
+    assert max_rel(dxt.real_view().cpu().numpy(), dx_o) <= TOL
+
+
+def test_backprop2_in_place(oracle_mod):
+    """dx may alias x (legacy/src/dnn_backend/batchnorm.cu:1303-1314)."""
+    import torch
+    from dihydrogen_amd.tensor import Distribution, LocaleVirtual, Tensor
+
+    shape = (2, 6, 8, 12)
+    x, dy, scale, bias = bn_inputs(shape, seed=7)
+    bn, xin, yout, mean, var, rm, rv = _run_forward(x, scale, bias)
+    dist = Distribution.make_localized_distribution(4)
+    dyt = Tensor(list(shape[::-1]), LocaleVirtual(0, 1), dist).allocate()
+    dyt.real_view().copy_(torch.from_numpy(dy))
+    outs = [torch.empty(shape[1], device="cuda") for _ in range(4)]
+    sc = torch.from_numpy(scale).cuda()
+    bn.backward(xin, dyt, mean, var, sc, *outs, xin)  # d_input aliases input
+    torch.cuda.synchronize()
+    dx_o = oracle_mod.bn_backward(x, dy, mean.cpu().numpy(), var.cpu().numpy(), scale, 1e-5)[0]
+    assert max_rel(xin.real_view().cpu().numpy(), dx_o) <= TOL
+
+
+def test_inference_uses_running_statistics(oracle_mod):
+    import torch
+    shape = (2, 4, 6, 6)
+    x, dy, scale, bias = bn_inputs(shape, seed=11)
+    bn, xin, yout, mean, var, rm, rv = _run_forward(x, scale, bias)
+    sc, bi = torch.from_numpy(scale).cuda(), torch.from_numpy(bias).cuda()
+    bn.forward(xin, mean, var, rm, rv, sc, bi, yout, False)
+    torch.cuda.synchronize()
+    y_o = oracle_mod.bn_batch_normalization(x, rm.cpu().numpy(), rv.cpu().numpy(), scale, bias, 1e-5)
+    assert max_rel(yout.real_view().cpu().numpy(), y_o) <= TOL
+
+
+def test_deterministic_and_workspace_reuse():
+    """Same input several times through one workspace: bit-identical sums (the
+    reference's atomics are not, legacy/src/dnn_backend/batchnorm.cu:127-131)."""
+    import torch
+    shape = (4, 32, 24, 24, 24)
+    x, dy, scale, bias = bn_inputs(shape, seed=3)
+    bn, xin, yout, mean, var, rm, rv = _run_forward(x, scale, bias)
+    results = []
+    for _ in range(4):
+        bn.forward_stage1(xin, mean, var, True)
+        torch.cuda.synchronize()
+        results.append((mean.cpu().numpy().copy(), var.cpu().numpy().copy()))
+    for m, v in results[1:]:
+        assert np.array_equal(m, results[0][0]) and np.array_equal(v, results[0][1])
+    s64 = x.astype(np.float64).sum(axis=(0, 2, 3, 4))
+    assert max_rel(results[0][0], s64.astype(np.float32)) <= 1e-6
+
+
+def test_float64(oracle_mod):
+    shape = (2, 5, 6, 10)
+    x, dy, scale, bias = bn_inputs(shape, seed=5, dtype=np.float64)
+    bn, xin, yout, mean, var, rm, rv = _run_forward(x, scale, bias, dtype="float64")
+    rm_o, rv_o = np.zeros(5), np.ones(5)
+    y_o, mean_o, var_o = oracle_mod.bn_forward(x, scale, bias, rm_o, rv_o, 1e-5, 0.9)
+    assert max_rel(mean.cpu().numpy(), mean_o) <= 1e-10
+    assert max_rel(var.cpu().numpy(), var_o) <= 1e-10
+    assert max_rel(yout.real_view().cpu().numpy(), y_o) <= 1e-10
+
+
+def test_empty_tensor_zeroes_sums():
+    """No samples: outputs are zeroed, nothing else happens
+    (legacy/src/dnn_backend/batchnorm.cu:201-208)."""
+    import ctypes
+    import torch
+    from dihydrogen_amd import capi
+    lib = capi.load()
+    c = 7
+    ws = torch.empty(lib.h2x_bn_workspace_bytes(c), dtype=torch.uint8, device="cuda")
+    capi.check(lib.h2x_bn_workspace_init(ws.data_ptr(), c, None))
+    s = torch.full((c,), 3.0, device="cuda")
+    q = torch.full((c,), 3.0, device="cuda")
+    capi.check(lib.h2x_bn_channel_sums_and_sqsums(capi.F32, 0, c, 16, 16, None, s.data_ptr(),
+                                                  q.data_ptr(), ws.data_ptr(), None))
+    torch.cuda.synchronize()
+    assert (s == 0).all() and (q == 0).all()

@@ -1,0 +1,128 @@
+"""GPU parity: channel softmax entry points against the CPU oracle.
+
+Tolerance 1e-5 relative, metric max(|d/v1|, |d/v2|).  The reference holds no
+softmax test; the oracle is pinned by torch.softmax and its autograd in fp64
+(tests/test_oracle_softmax.py).
+"""
+import numpy as np
+import pytest
+
+from helpers import max_rel
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-5
+
+CASES = [
+    (16, 21, 64, 64),     # BASELINE config 4 at reduced spatial size (full size in test_gpu_full_size.py)
+    (2, 21, 7, 9),        # scalar path
+    (3, 4, 8, 8),
+    (2, 1, 4, 4),         # one channel
+    (1, 33, 6, 10),       # float2 tile
+    (2, 70, 3, 5),        # CMAX 128, scalar
+    (1, 200, 4, 4),       # streaming fallback
+    (2, 19, 4, 6, 10),    # 5-D
+]
+
+
+def _tensors(shape, dtype="float32"):
+    import torch
+    from dihydrogen_amd.tensor import Distribution, LocaleVirtual, Tensor
+    dist = Distribution.make_localized_distribution(len(shape))
+    mk = lambda: Tensor(list(shape[::-1]), LocaleVirtual(0, 1), dist, getattr(torch, dtype)).allocate()
+    return mk
+
+
+@pytest.mark.parametrize("shape", CASES)
+def test_forward_backward(shape, oracle_mod):
+    import torch
+    from dihydrogen_amd.layers import Softmax, SoftmaxMode
+    rng = np.random.default_rng(99)
+    x = (2.0 * rng.standard_normal(shape)).astype(np.float32)
+    dy = rng.standard_normal(shape).astype(np.float32)
+    mk = _tensors(shape)
+    xt, yt, dyt, dxt = mk(), mk(), mk(), mk()
+    xt.real_view().copy_(torch.from_numpy(x))
+    dyt.real_view().copy_(torch.from_numpy(dy))
+    sm = Softmax()
+    sm.setup(xt, SoftmaxMode.CHANNEL)
+    assert sm.forward(xt, yt) == 0
+    torch.cuda.synchronize()
+    y = yt.real_view().cpu().numpy()
+    y_o = oracle_mod.softmax_channel_forward(x)
+    assert max_rel(y, y_o) <= TOL
+    assert np.abs(y.sum(axis=1) - 1).max() < 1e-5
+    # backward from the GPU's own y, compared with the oracle on the same y
+    assert sm.backward(yt, dyt, dxt) == 0
+    torch.cuda.synchronize()
+    dx = dxt.real_view().cpu().numpy()
+    dx_o = oracle_mod.softmax_channel_backward(y, dy)
+    assert np.array_equal(dx, dx_o) or max_rel(dx, dx_o) <= TOL
+
+
+def test_underflow_clamp_and_guard(oracle_mod):
+    """A logit gap > 104 underflows exp: y is clamped to FLT_MIN and the
+    backward guard y > FLT_MIN zeroes the gradient
+    (legacy/src/dnn_backend/softmax.cu:557,590,634,666)."""
+    import torch
+    from dihydrogen_amd.layers import Softmax, SoftmaxMode
+    shape = (1, 4, 2, 4)
+    x = np.zeros(shape, np.float32)
+    x[:, 0] = 120.0
+    x[:, 3] = -50.0
+    dy = np.ones(shape, np.float32)
+    dy[:, 1] = 2.0
+    mk = _tensors(shape)
+    xt, yt, dyt, dxt = mk(), mk(), mk(), mk()
+    xt.real_view().copy_(torch.from_numpy(x))
+    dyt.real_view().copy_(torch.from_numpy(dy))
+    sm = Softmax()
+    sm.setup(xt, SoftmaxMode.CHANNEL)
+    sm.forward(xt, yt)
+    sm.backward(yt, dyt, dxt)
+    torch.cuda.synchronize()
+    y = yt.real_view().cpu().numpy()
+    dx = dxt.real_view().cpu().numpy()
+    flt_min = np.finfo(np.float32).tiny
+    assert (y[:, 1:] == flt_min).all() and (y[:, 0] == 1.0).all()
+    assert (dx[:, 1:] == 0).all()
+    assert np.array_equal(y, oracle_mod.softmax_channel_forward(x))
+    assert np.array_equal(dx, oracle_mod.softmax_channel_backward(y, dy))
+
+
+def test_all_negative_logits_keep_reference_maximum(oracle_mod):
+    """The running maximum starts at FLT_MIN, so all-negative logits are
+    shifted by ~0, not by their maximum (softmax.cu:565)."""
+    import torch
+    from dihydrogen_amd.layers import Softmax, SoftmaxMode
+    shape = (1, 5, 2, 4)
+    rng = np.random.default_rng(5)
+    x = (-1.0 - rng.uniform(0, 3, shape)).astype(np.float32)
+    mk = _tensors(shape)
+    xt, yt = mk(), mk()
+    xt.real_view().copy_(torch.from_numpy(x))
+    sm = Softmax()
+    sm.setup(xt, SoftmaxMode.CHANNEL)
+    sm.forward(xt, yt)
+    torch.cuda.synchronize()
+    assert max_rel(yt.real_view().cpu().numpy(), oracle_mod.softmax_channel_forward(x)) <= TOL
+
+
+def test_float64(oracle_mod):
+    import torch
+    from dihydrogen_amd.layers import Softmax, SoftmaxMode
+    shape = (2, 9, 4, 6)
+    rng = np.random.default_rng(17)
+    x = 2.0 * rng.standard_normal(shape)
+    dy = rng.standard_normal(shape)
+    mk = _tensors(shape, "float64")
+    xt, yt, dyt, dxt = mk(), mk(), mk(), mk()
+    xt.real_view().copy_(torch.from_numpy(x))
+    dyt.real_view().copy_(torch.from_numpy(dy))
+    sm = Softmax()
+    sm.setup(xt, SoftmaxMode.CHANNEL)
+    sm.forward(xt, yt)
+    sm.backward(yt, dyt, dxt)
+    torch.cuda.synchronize()
+    y = yt.real_view().cpu().numpy()
+    assert max_rel(y, oracle_mod.softmax_channel_forward(x)) <= 1e-12
+    assert max_rel(dxt.real_view().cpu().numpy(), oracle_mod.softmax_channel_backward(y, dy)) <= 1e-12
