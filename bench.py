@@ -1,0 +1,347 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X DistConv hot path (one GPU).
+
+One "step" is one pass of the path BASELINE.json's metric is quoted on:
+  * 3-D batch-norm forward + backward on NCDHW 4 x 64 x 64^3 fp32 (config 3),
+  * one full halo exchange (pack + unpack, 3 dimension phases, width 1) of a
+    periodic 2 x 2 x 2 grid of virtual ranks, each N1 C32 128^3 fp32 (config 2).
+`value` is the algorithmic bytes of a step divided by its wall time, inputs
+resident in HBM.  The other BASELINE configs (2-D batch-norm forward, channel
+softmax, shuffle) are timed once each and reported under "breakdown".
+
+Prints ONE JSON line.  `--gpus N` with N > 1 exits: this build runs on one GPU.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+SEED = 1234
+
+
+def _gbs(nbytes: float, ms: float) -> float:
+    return nbytes / (ms * 1e-3) / 1e9 if ms > 0 else 0.0
+
+
+def _time_events(fn, iters: int, warmup: int):
+    """Median and minimum milliseconds of fn() measured with events on the
+    current stream (the stream every kernel of fn is launched on)."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    times = []
+    for _ in range(iters):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        fn()
+        e1.record()
+        e1.synchronize()
+        times.append(e0.elapsed_time(e1))
+    return statistics.median(times), min(times)
+
+
+class BatchNormWorkload:
+    """BatchNormalization forward + backward on one rank."""
+
+    def __init__(self, shape_np, seed):
+        import torch
+        from dihydrogen_amd.layers import BatchNormalization
+        from dihydrogen_amd.tensor import Distribution, LocaleVirtual, Tensor
+        g = torch.Generator(device="cuda").manual_seed(seed)
+        nd = len(shape_np)
+        c = shape_np[1]
+        dist = Distribution.make_localized_distribution(nd)
+        mk = lambda: Tensor(list(shape_np[::-1]), LocaleVirtual(0, 1), dist).allocate()
+        self.x, self.y, self.dy, self.dx = mk(), mk(), mk(), mk()
+        self.x.data.normal_(0, 1, generator=g)
+        self.dy.data.normal_(0, 1, generator=g)
+        self.scale = torch.empty(c, device="cuda").uniform_(0.5, 1.5, generator=g)
+        self.bias = torch.empty(c, device="cuda").normal_(0, 0.1, generator=g)
+        self.mean, self.var = torch.empty(c, device="cuda"), torch.empty(c, device="cuda")
+        self.rm, self.rv = torch.zeros(c, device="cuda"), torch.ones(c, device="cuda")
+        self.grads = [torch.empty(c, device="cuda") for _ in range(4)]
+        self.bn = BatchNormalization(nd, 0.9, 1e-5)
+        self.elems = self.x.get_local_size()
+
+    def forward(self):
+        self.bn.forward(self.x, self.mean, self.var, self.rm, self.rv, self.scale, self.bias,
+                        self.y, True)
+
+    def backward_reduce(self):
+        self.bn.backward_stage1(self.x, self.dy, self.mean, self.var, self.scale, *self.grads)
+        self.bn.backward_allreduce(*self.grads)
+
+    def backward_apply(self):
+        self.bn.backward_stage2(self.x, self.dy, self.mean, self.var, self.scale, self.grads[2],
+                                self.grads[3], self.dx)
+
+    def backward(self):
+        self.backward_reduce()
+        self.backward_apply()
+
+
+class HaloWorkload:
+    """Halo exchange of a periodic 2 x 2 x 2 grid of virtual ranks."""
+
+    def __init__(self, local_spatial, channels, seed):
+        import torch
+        from dihydrogen_amd.layers import HaloExchangeVirtual
+        from dihydrogen_amd.tensor import Distribution, LocaleVirtual, Tensor
+        g = torch.Generator(device="cuda").manual_seed(seed)
+        locale, overlap = (2, 2, 2, 1, 1), (1, 1, 1, 0, 0)
+        gshape = [2 * local_spatial] * 3 + [channels, 1]
+        dist = Distribution.make_overlapped_distribution(locale, overlap)
+        self.ranks = [Tensor(gshape, LocaleVirtual(r, 8), dist).allocate() for r in range(8)]
+        for t in self.ranks:
+            t.interior_view().uniform_(-1, 1, generator=g)
+        self.xch = HaloExchangeVirtual(self.ranks, periodic=True)
+        face = (local_spatial + 2) ** 2 * channels
+        # per rank: 3 dims x 2 sides x (pack: read+write, unpack: read+write) x 4 bytes
+        self.bytes = 8 * 3 * 2 * 2 * 2 * face * 4
+        self.elems = 8 * 12 * face
+
+    def run(self):
+        self.xch.exchange()
+
+
+class SoftmaxWorkload:
+    def __init__(self, shape_np, seed):
+        import torch
+        from dihydrogen_amd.layers import Softmax, SoftmaxMode
+        from dihydrogen_amd.tensor import Distribution, LocaleVirtual, Tensor
+        g = torch.Generator(device="cuda").manual_seed(seed)
+        dist = Distribution.make_localized_distribution(len(shape_np))
+        mk = lambda: Tensor(list(shape_np[::-1]), LocaleVirtual(0, 1), dist).allocate()
+        self.x, self.y, self.dy, self.dx = mk(), mk(), mk(), mk()
+        self.x.data.normal_(0, 2, generator=g)  # sigma = 2
+        self.dy.data.normal_(0, 1, generator=g)
+        self.sm = Softmax()
+        self.sm.setup(self.x, SoftmaxMode.CHANNEL)
+        self.elems = self.x.get_local_size()
+
+    def forward(self):
+        self.sm.forward(self.x, self.y)
+
+    def backward(self):
+        self.sm.backward(self.y, self.dy, self.dx)
+
+
+class ShuffleWorkload:
+    """Sample-parallel (N over 4 ranks) <-> spatial-parallel (H/2 x W/2)."""
+
+    def __init__(self, gshape, seed):
+        import torch
+        from dihydrogen_amd.layers import TensorShufflerVirtual
+        from dihydrogen_amd.tensor import Distribution, LocaleVirtual, Tensor
+        g = torch.Generator(device="cuda").manual_seed(seed)
+        sd, dd = Distribution([1, 1, 1, 4]), Distribution([2, 2, 1, 1])
+        self.src = [Tensor(gshape, LocaleVirtual(r, 4), sd).allocate() for r in range(4)]
+        self.dst = [Tensor(gshape, LocaleVirtual(r, 4), dd).allocate() for r in range(4)]
+        for t in self.src:
+            t.data.uniform_(-1, 1, generator=g)
+        self.sh = TensorShufflerVirtual(self.src, self.dst)
+        self.elems = 1
+        for e in gshape:
+            self.elems *= e
+
+    def forward(self):
+        self.sh.shuffle_forward()
+
+    def backward(self):
+        self.sh.shuffle_backward()
+
+
+def cpu_baseline(repeats: int = 3):
+    """The CPU oracle (this repository's restatement of the reference kernels;
+    the reference has no CPU implementation of batch-norm, softmax or halo
+    packing) on the same step: config 3 batch-norm forward+backward plus the
+    config 2 exchange for 2 of the 8 virtual ranks' worth of faces."""
+    import numpy as np
+    import oracle
+    lib = oracle.lib()
+    lib.orc_num_threads.restype = __import__("ctypes").c_int
+    threads = lib.orc_num_threads()
+    rng = np.random.default_rng(SEED)
+    shp = (4, 64, 64, 64, 64)
+    x = rng.standard_normal(shp, dtype=np.float32)
+    dy = rng.standard_normal(shp, dtype=np.float32)
+    scale = rng.uniform(0.5, 1.5, 64).astype(np.float32)
+    bias = (0.1 * rng.standard_normal(64)).astype(np.float32)
+    halo_ranks = 2
+    fields = [rng.uniform(-1, 1, (1, 32, 130, 130, 130)).astype(np.float32) for _ in range(halo_ranks)]
+    bufs = {d: np.empty(oracle.halo_size((130, 130, 130, 32, 1), d, 1), np.float32) for d in range(3)}
+    bn_bytes = 8 * x.size * 4
+    halo_bytes = halo_ranks * 3 * 2 * 2 * 2 * bufs[0].size * 4
+
+    def step():
+        rm, rv = np.zeros(64, np.float32), np.ones(64, np.float32)
+        y, mean, var = oracle.bn_forward(x, scale, bias, rm, rv)
+        oracle.bn_backward(x, dy, mean, var, scale)
+        for f in fields:
+            for d in range(3):
+                for side in (0, 1):
+                    oracle.halo_pack_or_unpack(f, d, side, 1, bufs[d], True)
+                    oracle.halo_pack_or_unpack(f, d, side, 1, bufs[d], False)
+
+    step()
+    times = []
+    for _ in range(repeats):
+        t0 = time.perf_counter()
+        step()
+        times.append(time.perf_counter() - t0)
+    t = statistics.median(times)
+    return {
+        "value": (bn_bytes + halo_bytes) / t / 1e9,
+        "unit": "GB/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": (f"config 3 batch-norm fwd+bwd in full (67108864 elems) + config 2 exchange of "
+                   f"{halo_ranks} of 8 ranks; median of {repeats} runs, {t:.3f} s each; "
+                   f"gcc -O3 -fopenmp, OMP threads = {threads}"),
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-breakdown", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (virtual ranks share it); "
+              f"--gpus {args.gpus} is not supported", file=sys.stderr)
+        return 2
+
+    import torch
+    from dihydrogen_amd import capi
+    capi.load()  # raises if libh2x.so is missing: there is no fallback
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 2
+    torch.cuda.set_device(0)
+
+    bn3 = BatchNormWorkload((4, 64, 64, 64, 64), SEED + 3)
+    halo = HaloWorkload(128, 32, SEED + 2)
+    S3 = bn3.elems
+    bn_bytes = 8 * S3 * 4
+    step_bytes = bn_bytes + halo.bytes
+    step_elems = S3 + halo.elems
+
+    k_events = []
+
+    def step(timed: bool):
+        bn3.forward()
+        bn3.backward_reduce()
+        if timed:
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            bn3.backward_apply()
+            e1.record()
+            k_events.append((e0, e1))
+        else:
+            bn3.backward_apply()
+        halo.run()
+
+    for _ in range(args.warmup):
+        step(False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(True)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    value = _gbs(step_bytes, ms_per_step)
+
+    # dominant kernel: bn_backprop2_kernel (reads x and dy, writes dx: 3 * S * 4 bytes)
+    k_ms = statistics.mean(e0.elapsed_time(e1) for e0, e1 in k_events)
+    k_bytes = 3 * S3 * 4
+    roofline = {
+        "kernel": "bn_backprop2_kernel<float,4>",
+        "bound": "hbm",
+        "achieved": _gbs(k_bytes, k_ms),
+        "peak": HBM_PEAK_GBS,
+        "unit": "GB/s",
+        "frac": _gbs(k_bytes, k_ms) / HBM_PEAK_GBS,
+        "traffic": None,
+        "avg_launch_ms": k_ms,
+        "algorithmic_bytes": k_bytes,
+    }
+
+    breakdown = {}
+    if not args.no_breakdown:
+        it, wu = 20, 5
+
+        def entry(nbytes, elems, med, mn):
+            return {"bytes": nbytes, "ms_median": med, "ms_min": mn, "GB/s": _gbs(nbytes, med),
+                    "frac_of_peak": _gbs(nbytes, med) / HBM_PEAK_GBS, "Gelem/s": elems / (med * 1e-3) / 1e9}
+
+        breakdown["C3_bn3d_fwd"] = entry(3 * S3 * 4, S3, *_time_events(bn3.forward, it, wu))
+        breakdown["C3_bn3d_bwd"] = entry(5 * S3 * 4, S3, *_time_events(bn3.backward, it, wu))
+        breakdown["C3_bn3d_fwd_bwd"] = entry(
+            8 * S3 * 4, S3, *_time_events(lambda: (bn3.forward(), bn3.backward()), it, wu))
+        breakdown["C2_halo_8ranks"] = entry(halo.bytes, halo.elems, *_time_events(halo.run, it, wu))
+        for d, name in enumerate(("dim0_W", "dim1_H", "dim2_D")):
+            ov = [1 if k == d else 0 for k in range(5)]
+            fn = lambda ov=ov: halo.xch.exchange(ov, ov, ov, ov)
+            breakdown[f"C2_halo_{name}"] = entry(halo.bytes // 3, halo.elems // 3, *_time_events(fn, it, wu))
+        del bn3, halo
+        torch.cuda.empty_cache()
+        bn1 = BatchNormWorkload((8, 64, 56, 56), SEED + 1)
+        breakdown["C1_bn2d_fwd_warm"] = entry(3 * bn1.elems * 4, bn1.elems, *_time_events(bn1.forward, it, wu))
+        del bn1
+        sm = SoftmaxWorkload((16, 21, 256, 256), SEED + 4)
+        sm.forward()
+        breakdown["C4_softmax_fwd"] = entry(2 * sm.elems * 4, sm.elems, *_time_events(sm.forward, it, wu))
+        breakdown["C4_softmax_bwd"] = entry(3 * sm.elems * 4, sm.elems, *_time_events(sm.backward, it, wu))
+        del sm
+        shf = ShuffleWorkload((128, 128, 64, 32), SEED + 5)
+        breakdown["C5_shuffle_fwd"] = entry(4 * shf.elems * 4, shf.elems, *_time_events(shf.forward, it, wu))
+        breakdown["C5_shuffle_bwd"] = entry(4 * shf.elems * 4, shf.elems, *_time_events(shf.backward, it, wu))
+        del shf
+        torch.cuda.empty_cache()
+
+    out = {
+        "metric": "achieved HBM GB/s (% of MI355X peak) for BN fwd+bwd and halo pack/unpack",
+        "value": value,
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": ("C3 batch-norm fwd+bwd NCDHW 4x64x64^3 + C2 halo exchange 3x3x3 "
+                         "(8 virtual ranks 2x2x2 periodic, N1 C32 128^3, width 1)"),
+            "step_bytes": step_bytes,
+            "step_elements": step_elems,
+            "seed": SEED,
+        },
+        "frac_of_hbm_peak": value / HBM_PEAK_GBS,
+        "elements_per_s": step_elems / (ms_per_step * 1e-3),
+        "roofline": roofline,
+        "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline(),
+        "breakdown": breakdown,
+    }
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

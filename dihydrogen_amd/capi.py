@@ -59,7 +59,6 @@ SIGNATURES = {
     "h2x_abi_version": (c_int, []),
     "h2x_status_string": (ctypes.c_char_p, [c_int]),
     "h2x_bn_workspace_bytes": (c_size_t, [c_int]),
-    "h2x_bn_workspace_init": (c_int, [c_void_p, c_int, c_void_p]),
     "h2x_bn_channel_sums_and_sqsums": (c_int, [c_int, c_int, c_int, c_size_t, c_size_t, c_void_p,
                                                c_void_p, c_void_p, c_void_p, c_void_p]),
     "h2x_bn_sums_to_statistics": (c_int, [c_int, c_int, c_size_t, c_double, c_void_p, c_void_p,

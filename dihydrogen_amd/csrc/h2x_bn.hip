@@ -9,10 +9,14 @@
 // Reductions (forward sums, backward sums) cut every channel into contiguous
 // chunks, one workgroup per chunk.  A thread accumulates in fp64, the
 // workgroup combines lanes with DPP permutes and waves through LDS, and writes
-// one fp64 partial per sum.  The workgroup that finishes last for a channel
-// (per-channel completion counter) adds the partials in index order and writes
-// the channel's result.  All orders are fixed, so results are deterministic;
-// the reference's float atomics are not (batchnorm.cu:127-131,1047-1053).
+// one fp64 partial per sum into the workspace.  A second, tiny kernel adds the
+// partials of each channel in index order and writes the channel's result
+// (a kernel boundary is the cheapest device-wide ordering on this GPU: an
+// in-kernel "last workgroup finishes" scheme needs a device-scope fence per
+// workgroup, which costs an L2 write-back/invalidate each and was measured
+// 10x slower than the whole stream).  All orders are fixed, so results are
+// deterministic; the reference's float atomics are not
+// (batchnorm.cu:127-131,1047-1053).
 #include "h2x_device.hpp"
 
 #include <algorithm>
@@ -23,8 +27,10 @@ namespace
 {
 
 constexpr int kUnroll = 4;
-// Upper bound on workgroups per channel; sizes the workspace.
-constexpr int kTargetGroups = 8192;
+// Workgroups a reduction aims at over all channels (bounds the workspace) and
+// workgroups an elementwise pass aims at; both from a sweep on MI355X.
+constexpr int kTargetGroups = 4096;
+constexpr int kElementwiseBlocks = 16384;
 constexpr int kMinGroupsPerChannel = 8;
 constexpr int kMaxGroupsPerChannel = 2048;
 constexpr int kMaxSums = 4;
@@ -35,7 +41,7 @@ int max_groups_per_channel(int num_channels)
     return std::min(std::max(g, kMinGroupsPerChannel), kMaxGroupsPerChannel);
 }
 
-size_t counters_offset(int num_channels)
+size_t partials_bytes(int num_channels)
 {
     return static_cast<size_t>(num_channels) * max_groups_per_channel(num_channels) * kMaxSums
            * sizeof(double);
@@ -125,53 +131,57 @@ __device__ __forceinline__ double inv_sqrt_t(double v)
     return 1.0 / __builtin_sqrt(v);
 }
 
-// Combines the K per-thread sums of a workgroup and, in the workgroup that
-// completes a channel, the partials of all workgroups of that channel.
-// Returns true in that last workgroup, with the channel totals in acc[].
+// Combines the K per-thread sums of a workgroup.  With a single workgroup per
+// channel returns true (totals in acc[], to be written by the caller);
+// otherwise stores this workgroup's partials for the finishing kernel.
 template <int K>
-__device__ __forceinline__ bool finish_channel(double (&acc)[K], double* partials,
-                                               unsigned int* counters, int channel,
-                                               int groups_per_channel_max)
+__device__ __forceinline__ bool finish_workgroup(double (&acc)[K], double* partials, int channel,
+                                                 int groups_per_channel_max)
 {
     __shared__ double lds[K * kWavesPerBlock];
-    __shared__ int is_last;
     block_sum<K>(acc, lds);
-    const unsigned int groups = gridDim.x;
-    if (groups == 1)
+    if (gridDim.x == 1)
         return true;
-    double* mine = partials + (static_cast<size_t>(channel) * groups_per_channel_max) * K;
     if (threadIdx.x == 0)
     {
+        double* mine = partials
+                       + (static_cast<size_t>(channel) * groups_per_channel_max + blockIdx.x) * K;
 #pragma unroll
         for (int k = 0; k < K; ++k)
-            __hip_atomic_store(mine + static_cast<size_t>(blockIdx.x) * K + k, acc[k],
-                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __threadfence();
-        const unsigned int done = atomicAdd(counters + channel, 1u);
-        is_last = (done == groups - 1) ? 1 : 0;
+            mine[k] = acc[k];
     }
-    __syncthreads();
-    if (!is_last)
-        return false;
-    __threadfence();
+    return false;
+}
+
+// Adds the `groups` partials of every channel in index order: thread t takes
+// partials t, t + 256, ...; the workgroup then combines its threads in the
+// fixed order of block_sum.  out_k[c] receives sum k of channel c.
+template <typename T, int K>
+__global__ __launch_bounds__(kBlockSize) void bn_finish_kernel(
+    const double* __restrict__ partials, int groups, int groups_per_channel_max, T* out0, T* out1,
+    T* out2, T* out3)
+{
+    __shared__ double lds[K * kWavesPerBlock];
+    const int c = blockIdx.x;
+    const double* mine = partials + static_cast<size_t>(c) * groups_per_channel_max * K;
     double t[K];
 #pragma unroll
     for (int k = 0; k < K; ++k)
         t[k] = 0.0;
-    for (unsigned int g = threadIdx.x; g < groups; g += kBlockSize)
+    for (int g = threadIdx.x; g < groups; g += kBlockSize)
     {
 #pragma unroll
         for (int k = 0; k < K; ++k)
-            t[k] += __hip_atomic_load(mine + static_cast<size_t>(g) * K + k, __ATOMIC_RELAXED,
-                                      __HIP_MEMORY_SCOPE_AGENT);
+            t[k] += mine[static_cast<size_t>(g) * K + k];
     }
     block_sum<K>(t, lds);
-#pragma unroll
-    for (int k = 0; k < K; ++k)
-        acc[k] = t[k];
     if (threadIdx.x == 0)
-        counters[channel] = 0u; // ready for the next launch on this workspace
-    return true;
+    {
+        T* outs[4] = {out0, out1, out2, out3};
+#pragma unroll
+        for (int k = 0; k < K; ++k)
+            outs[k][c] = static_cast<T>(t[k]);
+    }
 }
 
 // ---- forward: sums and sums of squares --------------------------------------
@@ -179,7 +189,7 @@ __device__ __forceinline__ bool finish_channel(double (&acc)[K], double* partial
 template <typename T, int VEC>
 __global__ __launch_bounds__(kBlockSize) void bn_sums_kernel(
     const T* __restrict__ x, T* __restrict__ sums, T* __restrict__ sqsums, double* partials,
-    unsigned int* counters, int num_channels, size_t spatial, size_t spatial_real, size_t chunk,
+    int num_channels, size_t spatial, size_t spatial_real, size_t chunk,
     int chunks_per_seg, unsigned int num_units, int groups_per_channel_max)
 {
     const int c = blockIdx.y;
@@ -230,7 +240,7 @@ __global__ __launch_bounds__(kBlockSize) void bn_sums_kernel(
         }
     }
     }
-    if (finish_channel<2>(acc, partials, counters, c, groups_per_channel_max) && threadIdx.x == 0)
+    if (finish_workgroup<2>(acc, partials, c, groups_per_channel_max) && threadIdx.x == 0)
     {
         sums[c] = static_cast<T>(acc[0]);
         sqsums[c] = static_cast<T>(acc[1]);
@@ -329,7 +339,7 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop1_kernel(
     const T* __restrict__ x, const T* __restrict__ dy, const T* __restrict__ mean,
     const T* __restrict__ var, const T* __restrict__ scale, T* __restrict__ dscale,
     T* __restrict__ dbias, T* __restrict__ dmean, T* __restrict__ dvar, T epsilon,
-    double* partials, unsigned int* counters, int num_channels, size_t spatial, size_t x_real,
+    double* partials, int num_channels, size_t spatial, size_t x_real,
     size_t dy_real, size_t chunk, int chunks_per_seg, unsigned int num_units,
     int groups_per_channel_max)
 {
@@ -393,7 +403,7 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop1_kernel(
                 accumulate(xv[j], dv[j]);
         }
     }
-    if (finish_channel<4>(acc, partials, counters, c, groups_per_channel_max) && threadIdx.x == 0)
+    if (finish_workgroup<4>(acc, partials, c, groups_per_channel_max) && threadIdx.x == 0)
     {
         dscale[c] = static_cast<T>(acc[0]);
         dbias[c] = static_cast<T>(acc[1]);
@@ -512,19 +522,21 @@ int sums_impl(int num_samples, int num_channels, size_t spatial, size_t real, co
         return H2X_ERR_TOO_LARGE;
     const size_t groups = std::min<size_t>(units, gmax);
     double* partials = static_cast<double*>(workspace);
-    unsigned int* counters = reinterpret_cast<unsigned int*>(static_cast<char*>(workspace)
-                                                             + counters_offset(num_channels));
     const dim3 grid(static_cast<unsigned int>(groups), num_channels);
     if (vec)
         bn_sums_kernel<T, full_vec<T>()><<<grid, kBlockSize, 0, stream>>>(
             static_cast<const T*>(x), static_cast<T*>(sums), static_cast<T*>(sqsums), partials,
-            counters, num_channels, spatial, real, ch.chunk, ch.chunks_per_seg,
+            num_channels, spatial, real, ch.chunk, ch.chunks_per_seg,
             static_cast<unsigned int>(units), gmax);
     else
         bn_sums_kernel<T, 1><<<grid, kBlockSize, 0, stream>>>(
             static_cast<const T*>(x), static_cast<T*>(sums), static_cast<T*>(sqsums), partials,
-            counters, num_channels, spatial, real, ch.chunk, ch.chunks_per_seg,
+            num_channels, spatial, real, ch.chunk, ch.chunks_per_seg,
             static_cast<unsigned int>(units), gmax);
+    if (groups > 1)
+        bn_finish_kernel<T, 2><<<num_channels, kBlockSize, 0, stream>>>(
+            partials, static_cast<int>(groups), gmax, static_cast<T*>(sums),
+            static_cast<T*>(sqsums), nullptr, nullptr);
     return launch_status();
 }
 
@@ -548,7 +560,8 @@ Chunking elementwise_chunking(size_t spatial, size_t segments, int vw, int unrol
     const size_t tile = static_cast<size_t>(kBlockSize) * vw * unroll;
     const size_t one_pass = static_cast<size_t>(kBlockSize) * vw;
     // aim at >= 4096 workgroups, but at least one full vector per thread
-    return make_chunking(spatial, segments, 4096, one_pass, one_pass * 2 > tile ? one_pass : one_pass * 2);
+    return make_chunking(spatial, segments, kElementwiseBlocks, one_pass,
+                         one_pass * 2 > tile ? one_pass : one_pass * 2);
 }
 
 template <typename T>
@@ -605,21 +618,23 @@ int backprop1_impl(int num_samples, int num_channels, size_t spatial, size_t x_r
         return H2X_ERR_TOO_LARGE;
     const size_t groups = std::min<size_t>(units, gmax);
     double* partials = static_cast<double*>(workspace);
-    unsigned int* counters = reinterpret_cast<unsigned int*>(static_cast<char*>(workspace)
-                                                             + counters_offset(num_channels));
     const dim3 grid(static_cast<unsigned int>(groups), num_channels);
 #define H2X_LAUNCH(V)                                                                              \
     bn_backprop1_kernel<T, V><<<grid, kBlockSize, 0, stream>>>(                                    \
         static_cast<const T*>(x), static_cast<const T*>(dy), static_cast<const T*>(mean),          \
         static_cast<const T*>(var), static_cast<const T*>(scale), static_cast<T*>(dscale),         \
         static_cast<T*>(dbias), static_cast<T*>(dmean), static_cast<T*>(dvar),                     \
-        static_cast<T>(epsilon), partials, counters, num_channels, spatial, x_real, dy_real,       \
-        ch.chunk, ch.chunks_per_seg, static_cast<unsigned int>(units), gmax)
+        static_cast<T>(epsilon), partials, num_channels, spatial, x_real, dy_real, ch.chunk,       \
+        ch.chunks_per_seg, static_cast<unsigned int>(units), gmax)
     if (vec)
         H2X_LAUNCH(full_vec<T>());
     else
         H2X_LAUNCH(1);
 #undef H2X_LAUNCH
+    if (groups > 1)
+        bn_finish_kernel<T, 4><<<num_channels, kBlockSize, 0, stream>>>(
+            partials, static_cast<int>(groups), gmax, static_cast<T*>(dscale),
+            static_cast<T*>(dbias), static_cast<T*>(dmean), static_cast<T*>(dvar));
     return launch_status();
 }
 
@@ -669,19 +684,7 @@ extern "C" size_t h2x_bn_workspace_bytes(int num_channels)
 {
     if (num_channels <= 0)
         return 256;
-    const size_t bytes = counters_offset(num_channels) + static_cast<size_t>(num_channels) * sizeof(unsigned int);
-    return (bytes + 255) / 256 * 256;
-}
-
-extern "C" int h2x_bn_workspace_init(void* workspace, int num_channels, h2x_stream_t stream)
-{
-    if (workspace == nullptr || num_channels < 0)
-        return H2X_ERR_INVALID_ARGUMENT;
-    const size_t words = h2x_bn_workspace_bytes(num_channels) / sizeof(unsigned int);
-    const unsigned int blocks = static_cast<unsigned int>(std::min<size_t>((words + kBlockSize - 1) / kBlockSize, 1024));
-    fill_kernel<unsigned int><<<blocks, kBlockSize, 0, as_stream(stream)>>>(
-        static_cast<unsigned int*>(workspace), words, 0u);
-    return launch_status();
+    return (partials_bytes(num_channels) + 255) / 256 * 256;
 }
 
 extern "C" int h2x_bn_channel_sums_and_sqsums(h2x_dtype dtype, int num_samples, int num_channels,

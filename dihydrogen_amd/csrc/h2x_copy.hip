@@ -83,6 +83,8 @@ struct Box
 {
     char* tensor;            // base the strides are relative to
     char* buffer;            // start of this box's contiguous image
+    char* tensor2;           // second box of identical geometry (sparse pairs), or null
+    char* buffer2;
     int64_t stride[kMaxBoxDims]; // elements
     FastDiv div[kMaxBoxDims];    // by extent[i]; the last used one is never divided by
     uint32_t count;          // elements in the box (< 2^31)
@@ -126,10 +128,26 @@ struct OpMin
     __device__ __forceinline__ T operator()(T a, T b) const { return a < b ? a : b; }
 };
 
+// Loads and stores of "sparse" boxes: runs shorter than a cache line that are
+// a row apart (a halo face of the innermost dimension).  Every element costs a
+// whole 128-byte line of HBM traffic; stores are write-through so that the
+// line is not allocated for a 4-byte write.
+template <typename T>
+__device__ __forceinline__ void sparse_store_scalar(T* p, T v)
+{
+    if constexpr (sizeof(T) >= 4)
+        __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else
+        *p = v;
+}
+
 // T: element type the op sees (an unsigned integer of the element's size for
 // plain copies).  VEC elements of one run move per thread and step; the buffer
-// side is VEC-aligned, the tensor side may start on any element.
-template <typename T, int VEC, typename Op>
+// side is VEC-aligned, the tensor side may start on any element.  SPARSE boxes
+// come in pairs of identical geometry (the LHS and RHS face of one tensor):
+// one thread serves the same index of both, so that neighbouring rows' ends,
+// which share a cache line, are touched by neighbouring lanes of one wave.
+template <typename T, int VEC, typename Op, bool SPARSE>
 __global__ __launch_bounds__(kBlockSize) void box_copy_kernel(const BoxBatch batch, Op op)
 {
     // which box does this workgroup belong to?
@@ -142,8 +160,6 @@ __global__ __launch_bounds__(kBlockSize) void box_copy_kernel(const BoxBatch bat
     const uint32_t count = box.count;
     const int nd = box.num_dims;
     const int mode = box.mode;
-    T* const tensor = reinterpret_cast<T*>(box.tensor);
-    T* const buffer = reinterpret_cast<T*>(box.buffer);
     using WA = typename Words<T, VEC>::aligned_t;
     using WU = typename Words<T, VEC>::unaligned_t;
 
@@ -172,31 +188,87 @@ __global__ __launch_bounds__(kBlockSize) void box_copy_kernel(const BoxBatch bat
         toff[u] = off;
     }
 
-    if (mode == kPack)
+    constexpr int kSides = SPARSE ? 2 : 1;
+#pragma unroll
+    for (int side = 0; side < kSides; ++side)
     {
-        WU v[kCopyUnroll];
-#pragma unroll
-        for (int u = 0; u < kCopyUnroll; ++u)
-            if (g[u] < count)
-                v[u] = *reinterpret_cast<const WU*>(tensor + toff[u]);
-#pragma unroll
-        for (int u = 0; u < kCopyUnroll; ++u)
-            if (g[u] < count)
-                *reinterpret_cast<WA*>(buffer + g[u]) = v[u];
-    }
-    else if (mode == kUnpack)
-    {
-        WA v[kCopyUnroll];
-#pragma unroll
-        for (int u = 0; u < kCopyUnroll; ++u)
-            if (g[u] < count)
-                v[u] = *reinterpret_cast<const WA*>(buffer + g[u]);
-        if constexpr (std::is_same<Op, OpId>::value)
+        T* const tensor = reinterpret_cast<T*>(side == 0 ? box.tensor : box.tensor2);
+        T* const buffer = reinterpret_cast<T*>(side == 0 ? box.buffer : box.buffer2);
+        if (side == 1 && tensor == nullptr)
+            break;
+        if (mode == kPack)
         {
+            if constexpr (SPARSE)
+            {
+                // both faces' loads are issued before any store, so that the
+                // two touches of a shared line meet in the cache
+                if (side == 1)
+                    break;
+                T* const tensor_b = reinterpret_cast<T*>(box.tensor2);
+                T* const buffer_b = reinterpret_cast<T*>(box.buffer2);
+                WU va[kCopyUnroll], vb[kCopyUnroll];
+#pragma unroll
+                for (int u = 0; u < kCopyUnroll; ++u)
+                    if (g[u] < count)
+                    {
+                        va[u] = *reinterpret_cast<const WU*>(tensor + toff[u]);
+                        if (tensor_b != nullptr)
+                            vb[u] = *reinterpret_cast<const WU*>(tensor_b + toff[u]);
+                    }
+#pragma unroll
+                for (int u = 0; u < kCopyUnroll; ++u)
+                    if (g[u] < count)
+                    {
+                        *reinterpret_cast<WA*>(buffer + g[u]) = va[u];
+                        if (tensor_b != nullptr)
+                            *reinterpret_cast<WA*>(buffer_b + g[u]) = vb[u];
+                    }
+            }
+            else
+            {
+                WU v[kCopyUnroll];
+#pragma unroll
+                for (int u = 0; u < kCopyUnroll; ++u)
+                    if (g[u] < count)
+                        v[u] = *reinterpret_cast<const WU*>(tensor + toff[u]);
+#pragma unroll
+                for (int u = 0; u < kCopyUnroll; ++u)
+                    if (g[u] < count)
+                        *reinterpret_cast<WA*>(buffer + g[u]) = v[u];
+            }
+        }
+        else if (mode == kUnpack)
+        {
+            WA v[kCopyUnroll];
 #pragma unroll
             for (int u = 0; u < kCopyUnroll; ++u)
                 if (g[u] < count)
-                    *reinterpret_cast<WU*>(tensor + toff[u]) = v[u];
+                    v[u] = *reinterpret_cast<const WA*>(buffer + g[u]);
+            if constexpr (std::is_same<Op, OpId>::value)
+            {
+#pragma unroll
+                for (int u = 0; u < kCopyUnroll; ++u)
+                    if (g[u] < count)
+                    {
+                        if constexpr (SPARSE && VEC == 1)
+                            sparse_store_scalar(tensor + toff[u], v[u][0]);
+                        else
+                            *reinterpret_cast<WU*>(tensor + toff[u]) = v[u];
+                    }
+            }
+            else
+            {
+#pragma unroll
+                for (int u = 0; u < kCopyUnroll; ++u)
+                    if (g[u] < count)
+                    {
+                        WU t = *reinterpret_cast<const WU*>(tensor + toff[u]);
+#pragma unroll
+                        for (int j = 0; j < VEC; ++j)
+                            t[j] = op(t[j], v[u][j]);
+                        *reinterpret_cast<WU*>(tensor + toff[u]) = t;
+                    }
+            }
         }
         else
         {
@@ -204,24 +276,20 @@ __global__ __launch_bounds__(kBlockSize) void box_copy_kernel(const BoxBatch bat
             for (int u = 0; u < kCopyUnroll; ++u)
                 if (g[u] < count)
                 {
-                    WU t = *reinterpret_cast<const WU*>(tensor + toff[u]);
+                    if constexpr (SPARSE && VEC == 1)
+                    {
+                        sparse_store_scalar(tensor + toff[u], T(0));
+                    }
+                    else
+                    {
+                        WU z;
 #pragma unroll
-                    for (int j = 0; j < VEC; ++j)
-                        t[j] = op(t[j], v[u][j]);
-                    *reinterpret_cast<WU*>(tensor + toff[u]) = t;
+                        for (int j = 0; j < VEC; ++j)
+                            z[j] = T(0);
+                        *reinterpret_cast<WU*>(tensor + toff[u]) = z;
+                    }
                 }
         }
-    }
-    else
-    {
-        WU z;
-#pragma unroll
-        for (int j = 0; j < VEC; ++j)
-            z[j] = T(0);
-#pragma unroll
-        for (int u = 0; u < kCopyUnroll; ++u)
-            if (g[u] < count)
-                *reinterpret_cast<WU*>(tensor + toff[u]) = z;
     }
 }
 
@@ -289,6 +357,16 @@ int box_vector(const HostBox& h, int elem_size, const void* buffer)
     return v;
 }
 
+bool same_geometry(const HostBox& a, const HostBox& b)
+{
+    if (a.nd != b.nd || a.count != b.count)
+        return false;
+    for (int i = 0; i < a.nd; ++i)
+        if (a.extent[i] != b.extent[i] || a.stride[i] != b.stride[i])
+            return false;
+    return true;
+}
+
 struct Launcher
 {
     hipStream_t stream;
@@ -296,6 +374,9 @@ struct Launcher
     h2x_dtype dtype; // meaningful for accumulate ops only
     int op;          // h2x_halo_op
     int vec = 0;
+    bool sparse = false;
+    HostBox last;         // geometry of the most recently queued box
+    int last_mode = -1;
     BoxBatch batch;
 
     Launcher(hipStream_t s, int es, h2x_dtype dt, int o) : stream(s), elem_size(es), dtype(dt), op(o)
@@ -310,7 +391,12 @@ struct Launcher
         const dim3 grid(batch.num_blocks);
         switch (op)
         {
-        case H2X_HALO_ID: box_copy_kernel<T, VEC, OpId><<<grid, kBlockSize, 0, stream>>>(batch, OpId()); break;
+        case H2X_HALO_ID:
+            if (sparse)
+                box_copy_kernel<T, VEC, OpId, true><<<grid, kBlockSize, 0, stream>>>(batch, OpId());
+            else
+                box_copy_kernel<T, VEC, OpId, false><<<grid, kBlockSize, 0, stream>>>(batch, OpId());
+            break;
         default: return H2X_ERR_UNSUPPORTED;
         }
         return launch_status();
@@ -322,9 +408,24 @@ struct Launcher
         const dim3 grid(batch.num_blocks);
         switch (op)
         {
-        case H2X_HALO_SUM: box_copy_kernel<T, VEC, OpSum><<<grid, kBlockSize, 0, stream>>>(batch, OpSum()); break;
-        case H2X_HALO_MAX: box_copy_kernel<T, VEC, OpMax><<<grid, kBlockSize, 0, stream>>>(batch, OpMax()); break;
-        case H2X_HALO_MIN: box_copy_kernel<T, VEC, OpMin><<<grid, kBlockSize, 0, stream>>>(batch, OpMin()); break;
+        case H2X_HALO_SUM:
+            if (sparse)
+                box_copy_kernel<T, VEC, OpSum, true><<<grid, kBlockSize, 0, stream>>>(batch, OpSum());
+            else
+                box_copy_kernel<T, VEC, OpSum, false><<<grid, kBlockSize, 0, stream>>>(batch, OpSum());
+            break;
+        case H2X_HALO_MAX:
+            if (sparse)
+                box_copy_kernel<T, VEC, OpMax, true><<<grid, kBlockSize, 0, stream>>>(batch, OpMax());
+            else
+                box_copy_kernel<T, VEC, OpMax, false><<<grid, kBlockSize, 0, stream>>>(batch, OpMax());
+            break;
+        case H2X_HALO_MIN:
+            if (sparse)
+                box_copy_kernel<T, VEC, OpMin, true><<<grid, kBlockSize, 0, stream>>>(batch, OpMin());
+            else
+                box_copy_kernel<T, VEC, OpMin, false><<<grid, kBlockSize, 0, stream>>>(batch, OpMin());
+            break;
         default: return H2X_ERR_UNSUPPORTED;
         }
         return launch_status();
@@ -374,6 +475,7 @@ struct Launcher
         batch.num_boxes = 0;
         batch.num_blocks = 0;
         vec = 0;
+        last_mode = -1;
         return err;
     }
 
@@ -386,16 +488,34 @@ struct Launcher
         if (h.count >= (1ll << 31))
             return H2X_ERR_TOO_LARGE;
         const int v = mode == kClear ? box_vector(h, elem_size, nullptr) : box_vector(h, elem_size, buffer);
-        if (batch.num_boxes == kMaxBoxes || (batch.num_boxes > 0 && v != vec))
+        // sparse: every run is shorter than a cache line and the runs are apart
+        const bool sp = h.nd > 1 ? h.extent[0] * h.stride[0] * elem_size < 128
+                                 : (h.stride[0] != 1 && h.extent[0] > 1);
+        char* const tptr = static_cast<char*>(tensor) + h.tensor_offset * elem_size;
+        char* const bptr = static_cast<char*>(buffer) + h.buffer_offset * elem_size;
+        // second box of a sparse pair: same geometry and mode as the box queued last
+        if (sp && batch.num_boxes > 0 && sparse && v == vec && last_mode == mode
+            && batch.box[batch.num_boxes - 1].tensor2 == nullptr && same_geometry(h, last))
+        {
+            batch.box[batch.num_boxes - 1].tensor2 = tptr;
+            batch.box[batch.num_boxes - 1].buffer2 = bptr;
+            return H2X_SUCCESS;
+        }
+        if (batch.num_boxes == kMaxBoxes || (batch.num_boxes > 0 && (v != vec || sp != sparse)))
         {
             const int err = flush();
             if (err != 0)
                 return err;
         }
         vec = v;
+        sparse = sp;
+        last = h;
+        last_mode = mode;
         Box& b = batch.box[batch.num_boxes];
-        b.tensor = static_cast<char*>(tensor) + h.tensor_offset * elem_size;
-        b.buffer = static_cast<char*>(buffer) + h.buffer_offset * elem_size;
+        b.tensor = tptr;
+        b.buffer = bptr;
+        b.tensor2 = nullptr;
+        b.buffer2 = nullptr;
         for (int i = 0; i < kMaxBoxDims; ++i)
         {
             b.stride[i] = i < h.nd ? h.stride[i] : 0;

@@ -72,8 +72,6 @@ class BatchNormalization:
         if self._workspace is None or self._workspace_channels != num_channels:
             nbytes = self._lib.h2x_bn_workspace_bytes(num_channels)
             self._workspace = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
-            capi.check(self._lib.h2x_bn_workspace_init(_ptr(self._workspace), num_channels,
-                                                       _stream_handle(self.stream)), "bn workspace init")
             self._workspace_channels = num_channels
         return self._workspace
 
@@ -250,6 +248,7 @@ class HaloExchangeVirtual:
             raise NotImplementedError("shared (replicated) distributions are not exchanged")  # :30-31
         self.nd = t0.get_num_dims()
         self._recv = {}  # (rank, dim, side) -> torch buffer the rank unpacks from
+        self._faces = {}  # exchange arguments -> (pack faces, unpack faces)
 
     def get_halo_size(self, rank: int, dim: int, width: int) -> int:
         """halo_exchange_cuda.hpp:267-271."""
@@ -302,14 +301,6 @@ class HaloExchangeVirtual:
         f.is_pack, f.op = int(is_pack), op.value
         return f
 
-    def _run(self, faces: List[capi.HaloFace], dtype: int) -> None:
-        if not faces:
-            return
-        arr = (capi.HaloFace * len(faces))(*faces)
-        capi.check(self._lib.h2x_halo_pack_or_unpack_batched(dtype, arr, len(faces),
-                                                             _stream_handle(self.stream)),
-                   "halo pack/unpack")
-
     def exchange_dim(self, dim: int, width_rhs_send: int, width_rhs_recv: int, width_lhs_send: int,
                      width_lhs_recv: int, is_reverse: bool = False, skip_unpack: bool = False,
                      op: HaloExchangeAccumOp = HaloExchangeAccumOp.ID) -> None:
@@ -317,25 +308,36 @@ class HaloExchangeVirtual:
         halo_exchange_cuda_mpi.hpp:25-100.  A rank's RHS strip goes to its RHS
         neighbour's LHS receive buffer and vice versa."""
         dtype = self.tensors[0].h2x_dtype
-        packs, unpacks = [], []
-        for r, t in enumerate(self.tensors):
-            if not self.is_exchange_required(
-                    r, dim, (width_rhs_send, width_rhs_recv, width_lhs_send, width_lhs_recv)):
-                continue
-            for side in (capi.LHS, capi.RHS):
-                peer = self.find_peer_rank(r, dim, side)
-                if peer is None:
+        key = (dim, width_rhs_send, width_rhs_recv, width_lhs_send, width_lhs_recv, is_reverse,
+               skip_unpack, op)
+        cached = self._faces.get(key)
+        if cached is None:
+            packs, unpacks = [], []
+            for r, t in enumerate(self.tensors):
+                if not self.is_exchange_required(
+                        r, dim, (width_rhs_send, width_rhs_recv, width_lhs_send, width_lhs_recv)):
                     continue
-                w_send = width_rhs_send if side == capi.RHS else width_lhs_send
-                w_recv = width_rhs_recv if side == capi.RHS else width_lhs_recv
-                if w_send > 0:
-                    dst = self._recv_buffer(peer, dim, capi.LHS if side == capi.RHS else capi.RHS)
-                    packs.append(self._face(r, dim, side, w_send, dst, True, is_reverse, op))
-                if w_recv > 0 and not skip_unpack:
-                    src = self._recv_buffer(r, dim, side)
-                    unpacks.append(self._face(r, dim, side, w_recv, src, False, is_reverse, op))
-        self._run(packs, dtype)
-        self._run(unpacks, dtype)
+                for side in (capi.LHS, capi.RHS):
+                    peer = self.find_peer_rank(r, dim, side)
+                    if peer is None:
+                        continue
+                    w_send = width_rhs_send if side == capi.RHS else width_lhs_send
+                    w_recv = width_rhs_recv if side == capi.RHS else width_lhs_recv
+                    if w_send > 0:
+                        dst = self._recv_buffer(peer, dim, capi.LHS if side == capi.RHS else capi.RHS)
+                        packs.append(self._face(r, dim, side, w_send, dst, True, is_reverse, op))
+                    if w_recv > 0 and not skip_unpack:
+                        src = self._recv_buffer(r, dim, side)
+                        unpacks.append(self._face(r, dim, side, w_recv, src, False, is_reverse, op))
+            # the face tables depend only on the arguments and on the tensors'
+            # addresses, which do not change: build them once
+            cached = tuple((capi.HaloFace * len(f))(*f) if f else None for f in (packs, unpacks))
+            self._faces[key] = cached
+        st = _stream_handle(self.stream)
+        for arr in cached:
+            if arr is not None:
+                capi.check(self._lib.h2x_halo_pack_or_unpack_batched(dtype, arr, len(arr), st),
+                           "halo pack/unpack")
 
     def exchange(self, widths_rhs_send=None, widths_rhs_recv=None, widths_lhs_send=None,
                  widths_lhs_recv=None, is_reverse: bool = False, skip_unpack: bool = False,

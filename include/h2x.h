@@ -92,16 +92,11 @@ const char* h2x_status_string(int status);
 
 /**
  * Bytes of device workspace the two reduction entry points need for
- * `num_channels` channels.  The workspace holds per-workgroup partial sums
- * and one completion counter per channel.  It must be cleared once with
- * h2x_bn_workspace_init before its first use; afterwards the kernels leave it
- * ready for the next call.  One workspace must not be used by two calls that
- * may run concurrently.
+ * `num_channels` channels.  The workspace holds fp64 partial sums, one set per
+ * workgroup; it needs no initialisation and keeps no state between calls.  One
+ * workspace must not be used by two calls that may run concurrently.
  */
 size_t h2x_bn_workspace_bytes(int num_channels);
-
-/** Clears a workspace of h2x_bn_workspace_bytes(num_channels) bytes (fill kernel, no memset node). */
-int h2x_bn_workspace_init(void* workspace, int num_channels, h2x_stream_t stream);
 
 /**
  * sums[c] = sum over (n, i) of x; sqsums[c] = sum of x*x.

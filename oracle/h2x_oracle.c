@@ -17,6 +17,7 @@
  */
 #include <float.h>
 #include <math.h>
+#include <omp.h>
 #include <stddef.h>
 #include <stdint.h>
 #include <string.h>
@@ -50,6 +51,12 @@
 #undef T_FMA
 
 #define ORC_MAX_DIMS 6
+
+/* OpenMP threads the parallel loops of this file use. */
+int orc_num_threads(void)
+{
+    return omp_get_max_threads();
+}
 
 /*
  * Destination rank and offset inside that rank's chunk of the packed buffer
