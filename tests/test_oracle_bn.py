@@ -1,0 +1,230 @@
+"""Pins the batch-norm functions of the CPU oracle (oracle/h2x_oracle.c).
+
+The reference holds no stored vectors and no CPU implementation for this part
+(its own validation is opt-kernel vs generic-kernel on the GPU), so the oracle
+is pinned by what the mathematics fixes:
+  * float64 closed forms (tests/golden fixtures, written independently in numpy),
+  * torch autograd in float64 through the unbiased-variance expression,
+  * invariants (sum dx = 0, y statistics, running-average recurrence),
+  * special cases (constant input, n == 0, aliasing dx = x),
+  * brute-force Python loops on a tiny tensor.
+Each check would fail for a dropped term, a wrong sign or n vs n-1.
+
+Comparisons with float64 references use the conditioning of each formula:
+|d| <= tol * (sum of |terms|), the bound an fp32 evaluation can meet; a plain
+relative bound is meaningless where terms cancel.
+"""
+import glob
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from helpers import bn_inputs, max_rel
+
+GOLDEN = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "bn_*.npz")))
+EPS = 1e-5
+
+
+def _bshape(x):
+    return (1, x.shape[1]) + (1,) * (x.ndim - 2)
+
+
+def _axes(x):
+    return (0,) + tuple(range(2, x.ndim))
+
+
+@pytest.mark.parametrize("path", GOLDEN)
+def test_golden_forward(path):
+    g = np.load(path)
+    x, scale, bias = g["x"], g["scale"], g["bias"]
+    c = x.shape[1]
+    rm, rv = np.zeros(c, np.float32), np.ones(c, np.float32)
+    y, mean, var = oracle.bn_forward(x, scale, bias, rm, rv, EPS, 0.9)
+    assert max_rel(var, g["var"]) < 2e-6
+    assert np.abs(mean - g["mean"]).max() < 1e-6 * np.abs(x).mean()
+    assert np.abs(rm - g["running_mean"]).max() < 1e-7
+    assert max_rel(rv, g["running_var"]) < 1e-6
+    bs = _bshape(x)
+    r = 1 / np.sqrt(g["var"] + EPS)
+    cond = np.abs((x - g["mean"].reshape(bs)) * (r * scale).reshape(bs)) + np.abs(bias).reshape(bs)
+    assert (np.abs(y - g["y"]) <= 4e-7 * cond + 1e-12).all()
+
+
+@pytest.mark.parametrize("path", GOLDEN)
+def test_golden_backward(path):
+    g = np.load(path)
+    x, dy, scale = g["x"], g["dy"], g["scale"]
+    mean, var = g["mean"].astype(np.float32), g["var"].astype(np.float32)
+    dx, dscale, dbias, dmean, dvar = oracle.bn_backward(x, dy, mean, var, scale, EPS)
+    ax, bs = _axes(x), _bshape(x)
+    r = 1 / np.sqrt(g["var"] + EPS)
+    xm = x - g["mean"].reshape(bs)
+    mag_scale = np.abs(dy * xm * r.reshape(bs)).sum(axis=ax)
+    mag_bias = np.abs(dy).sum(axis=ax)
+    assert (np.abs(dscale - g["dscale"]) <= 1e-6 * mag_scale).all()
+    assert (np.abs(dbias - g["dbias"]) <= 1e-6 * mag_bias).all()
+    assert (np.abs(dmean - g["dmean"]) <= 1e-6 * mag_bias * scale * r).all()
+    assert (np.abs(dvar - g["dvar"]) <= 1e-6 * mag_scale * scale * r * r / 2).all()
+    n = x.size // x.shape[1]
+    cond = (np.abs(dy * (scale * r).reshape(bs)) + np.abs(g["dmean"] / n).reshape(bs)
+            + np.abs((g["dvar"] * 2 / (n - 1)).reshape(bs) * xm))
+    assert (np.abs(dx - g["dx"]) <= 2e-6 * cond + 1e-12).all()
+
+
+@pytest.mark.parametrize("shape", [(4, 6, 8, 8), (2, 3, 5, 7), (2, 4, 3, 4, 5)])
+def test_against_torch_autograd(shape):
+    """dx, dscale, dbias equal autograd through y = (x-mean)*rsqrt(var_unbiased+eps)*scale+bias.
+    torch.nn.functional.batch_norm is NOT equivalent (it normalises with the biased variance)."""
+    import torch
+    x, dy, scale, bias = bn_inputs(shape, seed=21)
+    xt = torch.tensor(x, dtype=torch.float64, requires_grad=True)
+    st = torch.tensor(scale, dtype=torch.float64, requires_grad=True)
+    bt = torch.tensor(bias, dtype=torch.float64, requires_grad=True)
+    dims = [0] + list(range(2, len(shape)))
+    bs = _bshape(x)
+    mean = xt.mean(dim=dims)
+    var = xt.var(dim=dims, unbiased=True)
+    y = (xt - mean.view(bs)) * torch.rsqrt(var.view(bs) + EPS) * st.view(bs) + bt.view(bs)
+    y.backward(torch.tensor(dy, dtype=torch.float64))
+    c = shape[1]
+    rm, rv = np.zeros(c, np.float32), np.ones(c, np.float32)
+    y_o, mean_o, var_o = oracle.bn_forward(x, scale, bias, rm, rv, EPS, 0.9)
+    dx_o, dscale_o, dbias_o, _, _ = oracle.bn_backward(x, dy, mean_o, var_o, scale, EPS)
+    assert np.abs(y_o - y.detach().numpy()).max() < 5e-6
+    assert max_rel(var_o, var.detach().numpy()) < 2e-6
+    assert np.abs(dx_o - xt.grad.numpy()).max() < 2e-5
+    ax = _axes(x)
+    assert (np.abs(dscale_o - st.grad.numpy()) <= 2e-6 * np.abs(dy * y_o).sum(axis=ax) / scale + 1e-4).all()
+    assert (np.abs(dbias_o - bt.grad.numpy()) <= 1e-6 * np.abs(dy).sum(axis=ax)).all()
+    # the biased-variance library routine differs by more than the tolerance at this n
+    yb = torch.nn.functional.batch_norm(xt.detach(), None, None, st.detach(), bt.detach(), True, 0.1, EPS)
+    n = x.size // c
+    assert np.abs(yb.numpy() - y_o).max() > 0.1 / n
+
+
+def test_invariants():
+    shape = (3, 5, 6, 7)
+    x, dy, scale, bias = bn_inputs(shape, seed=33)
+    c = shape[1]
+    rm = np.full(c, 2.0, np.float32)
+    rv = np.full(c, 3.0, np.float32)
+    y, mean, var = oracle.bn_forward(x, scale, bias, rm, rv, EPS, 0.9)
+    ax = _axes(x)
+    n = x.size // c
+    # mean_c(y) = bias_c ; var_unbiased_c(y) = scale^2 * var / (var + eps)
+    assert np.abs(y.astype(np.float64).mean(axis=ax) - bias).max() < 1e-6
+    assert max_rel(y.astype(np.float64).var(axis=ax, ddof=1), scale.astype(np.float64) ** 2 * var / (var + EPS)) < 1e-5
+    # running = 0.9 * old + 0.1 * new
+    assert np.abs(rm - (0.9 * 2.0 + 0.1 * mean)).max() < 1e-6
+    assert max_rel(rv, 0.9 * 3.0 + 0.1 * var) < 1e-6
+    dx, dscale, dbias, dmean, dvar = oracle.bn_backward(x, dy, mean, var, scale, EPS)
+    # sum dx = 0 and sum dx*(x-mean) = scale*r*(eps/(var+eps)) * sum dy*(x-mean), per channel
+    d64 = dx.astype(np.float64)
+    assert np.abs(d64.sum(axis=ax)).max() < 1e-4
+    r = 1 / np.sqrt(var.astype(np.float64) + EPS)
+    xm = x.astype(np.float64) - mean.reshape(_bshape(x))
+    lhs = (d64 * xm).sum(axis=ax)
+    rhs = scale * r * (EPS / (var + EPS)) * (dy.astype(np.float64) * xm).sum(axis=ax)
+    assert np.abs(lhs - rhs).max() < 1e-4
+    # dmean = -scale*r*dbias ; dvar = -scale*r^2/2 * dscale
+    assert max_rel(dmean, -scale * r * dbias) < 1e-5
+    assert max_rel(dvar, -scale * r * r / 2 * dscale) < 1e-5
+    assert n > 1
+
+
+def test_special_cases():
+    # constant input: var = 0, y = bias
+    x = np.full((2, 3, 4, 4), 1.5, np.float32)
+    scale = np.array([1, 2, 3], np.float32)
+    bias = np.array([0.5, -1, 2], np.float32)
+    rm, rv = np.zeros(3, np.float32), np.ones(3, np.float32)
+    y, mean, var = oracle.bn_forward(x, scale, bias, rm, rv, EPS, 0.9)
+    assert (var == 0).all() and (mean == 1.5).all()
+    assert np.array_equal(y, np.broadcast_to(bias.reshape(1, 3, 1, 1), x.shape))
+    # n == 0: only var is written, to 1 (legacy/src/dnn_backend/batchnorm.cu:337-345)
+    m, v = np.array([7.0], np.float32), np.array([9.0], np.float32)
+    r1, r2 = np.array([3.0], np.float32), np.array([4.0], np.float32)
+    oracle.bn_sums_to_statistics(0, 0.9, m, v, r1, r2)
+    assert (m, v, r1, r2) == (7.0, 1.0, 3.0, 4.0)
+    # n == 1: n/(n-1) = inf and 0*inf = NaN, as in the reference
+    m, v = np.array([2.0], np.float32), np.array([4.0], np.float32)
+    with np.errstate(all="ignore"):
+        oracle.bn_sums_to_statistics(1, 0.9, m, v, r1, r2)
+    assert np.isnan(v[0])
+
+
+def test_backprop2_may_alias_input():
+    shape = (2, 3, 4, 6)
+    x, dy, scale, bias = bn_inputs(shape, seed=44)
+    rm, rv = np.zeros(3, np.float32), np.ones(3, np.float32)
+    _, mean, var = oracle.bn_forward(x, scale, bias, rm, rv)
+    dscale, dbias, dmean, dvar = oracle.bn_backprop1(x, dy, mean, var, scale, EPS)
+    want = oracle.bn_backprop2(x, dy, mean, var, scale, dmean, dvar, EPS, x.size // 3)
+    xin = x.copy()
+    oracle.bn_backprop2(xin, dy, mean, var, scale, dmean, dvar, EPS, x.size // 3, out=xin)
+    assert np.array_equal(xin, want)
+
+
+def test_brute_force_tiny():
+    """Plain Python loops in float64 over N2 C3 H4 W5."""
+    shape = (2, 3, 4, 5)
+    x, dy, scale, bias = bn_inputs(shape, seed=55)
+    n = 2 * 4 * 5
+    rm, rv = np.zeros(3, np.float32), np.ones(3, np.float32)
+    y, mean, var = oracle.bn_forward(x, scale, bias, rm, rv)
+    dx, dscale, dbias, dmean, dvar = oracle.bn_backward(x, dy, mean, var, scale)
+    for c in range(3):
+        s = q = 0.0
+        for b in range(2):
+            for h in range(4):
+                for w in range(5):
+                    v = float(x[b, c, h, w])
+                    s += v
+                    q += v * v
+        m = s / n
+        va = max(q / n - m * m, 0.0) * n / (n - 1)
+        assert abs(mean[c] - m) < 1e-6 and abs(var[c] - va) < 1e-5 * va
+        r = 1.0 / (va + EPS) ** 0.5
+        ds = db = dm = dv = 0.0
+        for b in range(2):
+            for h in range(4):
+                for w in range(5):
+                    g = float(dy[b, c, h, w])
+                    xm = float(x[b, c, h, w]) - m
+                    assert abs(y[b, c, h, w] - (xm * r * scale[c] + bias[c])) < 2e-6
+                    ds += g * xm * r
+                    db += g
+                    dm -= g * scale[c] * r
+                    dv -= g * scale[c] * xm * r ** 3 / 2
+        assert abs(dscale[c] - ds) < 1e-5 and abs(dbias[c] - db) < 1e-5
+        assert abs(dmean[c] - dm) < 1e-5 and abs(dvar[c] - dv) < 1e-5
+        for b in range(2):
+            for h in range(4):
+                for w in range(5):
+                    want = float(dy[b, c, h, w]) * scale[c] * r + dm / n + dv * 2 / (n - 1) * (float(x[b, c, h, w]) - m)
+                    assert abs(dx[b, c, h, w] - want) < 3e-6
+
+
+def test_halo_in_outermost_spatial_dimension():
+    """spatial < spatial_real: the interior of each (n, c) block is a prefix of
+    its real extent (the layout of a tensor whose outermost spatial dimension
+    carries a halo, legacy/src/dnn_backend/batchnorm.cu:134-160)."""
+    rng = np.random.default_rng(9)
+    n, c, real, spatial = 2, 3, 40, 24
+    x = rng.standard_normal((n, c, real)).astype(np.float32)
+    s, q = oracle.bn_channel_sums_and_sqsums(x, spatial)
+    x64 = x[:, :, :spatial].astype(np.float64)
+    assert max_rel(s, x64.sum(axis=(0, 2))) < 1e-6
+    assert max_rel(q, (x64 ** 2).sum(axis=(0, 2))) < 1e-6
+
+
+def test_float64_variant():
+    shape = (2, 3, 4, 5)
+    x, dy, scale, bias = bn_inputs(shape, seed=66, dtype=np.float64)
+    rm, rv = np.zeros(3), np.ones(3)
+    y, mean, var = oracle.bn_forward(x, scale, bias, rm, rv)
+    ax = _axes(x)
+    assert max_rel(mean, x.mean(axis=ax)) < 1e-12
+    assert max_rel(var, x.var(axis=ax, ddof=1)) < 1e-12
