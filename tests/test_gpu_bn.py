@@ -172,3 +172,28 @@ def test_empty_tensor_zeroes_sums():
                                                   q.data_ptr(), ws.data_ptr(), None))
     torch.cuda.synchronize()
     assert (s == 0).all() and (q == 0).all()
+
+
+def test_golden_fixtures():
+    """The committed float64 fixtures (tests/golden) through the GPU library."""
+    import glob
+    import os
+    import torch
+    from dihydrogen_amd.tensor import Distribution, LocaleVirtual, Tensor
+    for path in sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "bn_*.npz"))):
+        g = np.load(path)
+        x, dy, scale, bias = g["x"], g["dy"], g["scale"], g["bias"]
+        bn, xin, yout, mean, var, rm, rv = _run_forward(x, scale, bias)
+        assert max_rel(var.cpu().numpy(), g["var"]) < 2e-6
+        assert np.abs(mean.cpu().numpy() - g["mean"]).max() < 1e-6
+        assert np.abs(yout.real_view().cpu().numpy() - g["y"]).max() < 5e-6
+        dist = Distribution.make_localized_distribution(x.ndim)
+        dyt = Tensor(list(x.shape[::-1]), LocaleVirtual(0, 1), dist).allocate()
+        dxt = Tensor(list(x.shape[::-1]), LocaleVirtual(0, 1), dist).allocate()
+        dyt.real_view().copy_(torch.from_numpy(dy))
+        outs = [torch.empty(x.shape[1], device="cuda") for _ in range(4)]
+        bn.backward(xin, dyt, mean, var, torch.from_numpy(scale).cuda(), *outs, dxt)
+        torch.cuda.synchronize()
+        assert np.abs(dxt.real_view().cpu().numpy() - g["dx"]).max() < 2e-5
+        assert np.abs(outs[0].cpu().numpy() - g["dscale"]).max() < 2e-5
+        assert np.abs(outs[1].cpu().numpy() - g["dbias"]).max() < 2e-5
