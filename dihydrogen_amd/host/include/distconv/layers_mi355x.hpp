@@ -1,0 +1,410 @@
+// BatchNormalization and Softmax layer classes of the DistConv API on top of
+// the h2x C ABI, plus the free functions that are the reference's kernel seam.
+// Signatures follow legacy/include/distconv/dnn_backend/batchnorm.hpp:22-96,
+// 100-581 and softmax.hpp:14-63; the backend tag is BackendMI355X.
+#pragma once
+
+#include <functional>
+#include <map>
+
+#include "distconv/tensor_mi355x.hpp"
+
+namespace distconv
+{
+
+// The part of DNNBackend<> the two layers use: a stream
+// (legacy/src/dnn_backend/dnn_backend.cpp:164-180).
+class BackendMI355X
+{
+public:
+    explicit BackendMI355X(hipStream_t stream = nullptr) : m_stream(stream) {}
+    hipStream_t get_stream() const { return m_stream; }
+
+private:
+    hipStream_t m_stream;
+};
+
+namespace batchnorm
+{
+
+// (num_samples, num_channels, spatial, spatial_real) of a tensor the
+// optimised layout covers: no halo in the inner spatial dimensions
+// (legacy/src/dnn_backend/batchnorm.cu:210-219).
+template <typename Tensor>
+struct ChannelGeometry
+{
+    int num_channels;
+    size_t spatial, spatial_real;
+    explicit ChannelGeometry(const Tensor& t)
+    {
+        const int nd = t.get_num_dims();
+        for (int i = 0; i < nd - 3; ++i)
+            assert_always(t.get_halo_width(i) == 0);
+        assert_always(t.get_halo_width(nd - 2) == 0 && t.get_halo_width(nd - 1) == 0);
+        num_channels = static_cast<int>(t.get_local_shape()[-2]);
+        spatial = spatial_real = 1;
+        for (int i = 0; i < nd - 2; ++i)
+        {
+            spatial *= t.get_local_shape()[i];
+            spatial_real *= t.get_local_real_shape()[i];
+        }
+    }
+};
+
+// Workspace of fp64 partial sums, owned by the caller (one per layer object).
+class Workspace
+{
+public:
+    void* get(int num_channels)
+    {
+        const size_t need = h2x_bn_workspace_bytes(num_channels);
+        if (m_mem.is_null() || m_mem.get_size() < need)
+            m_mem.allocate(need);
+        return m_mem.get();
+    }
+
+private:
+    tensor::Memory<tensor::CUDAAllocator> m_mem;
+};
+
+// Workspace used by the overloads that keep the reference's exact signatures:
+// one per stream, created on first use and kept for the life of the process
+// (calls on one stream are ordered, so they can share it).
+inline Workspace& default_workspace(hipStream_t stream)
+{
+    static std::map<hipStream_t, Workspace> table;
+    return table[stream];
+}
+
+// batchnorm.hpp:22-28
+template <typename Tensor>
+void channel_sums_and_sqsums(int num_dims, int num_samples, const Tensor& input, Tensor& sums,
+                             Tensor& sqsums, hipStream_t stream, Workspace& ws)
+{
+    assert_always(num_dims == 4 || num_dims == 5);
+    const ChannelGeometry<Tensor> g(input);
+    // a rank that is not a split root, or holds nothing, only zeroes the sums
+    // (batchnorm.cu:201-208)
+    const bool active = input.get_local_size() > 0 && input.is_split_root();
+    DISTCONV_CHECK_H2X(h2x_bn_channel_sums_and_sqsums(
+        Tensor::h2x_type(), active ? num_samples : 0, g.num_channels, g.spatial, g.spatial_real,
+        input.get_const_base_ptr(), sums.get_base_ptr(), sqsums.get_base_ptr(),
+        ws.get(g.num_channels), stream));
+}
+
+template <typename Tensor>
+void channel_sums_and_sqsums(int num_dims, int num_samples, const Tensor& input, Tensor& sums,
+                             Tensor& sqsums, hipStream_t stream)
+{
+    channel_sums_and_sqsums(num_dims, num_samples, input, sums, sqsums, stream,
+                            default_workspace(stream));
+}
+
+// batchnorm.hpp:30-37
+template <typename Tensor>
+void sums_to_statistics(index_t num_per_sum, typename Tensor::data_type decay, Tensor& global_mean,
+                        Tensor& global_var, Tensor& running_mean, Tensor& running_var,
+                        hipStream_t stream)
+{
+    DISTCONV_CHECK_H2X(h2x_bn_sums_to_statistics(
+        Tensor::h2x_type(), static_cast<int>(global_mean.get_local_size()), num_per_sum, decay,
+        global_mean.get_base_ptr(), global_var.get_base_ptr(), running_mean.get_base_ptr(),
+        running_var.get_base_ptr(), stream));
+}
+
+// batchnorm.hpp:39-49
+template <typename Tensor>
+void batch_normalization(int num_dims, int num_samples, const Tensor& input, const Tensor& mean,
+                         const Tensor& var, const Tensor& scale, const Tensor& bias, Tensor& output,
+                         typename Tensor::data_type epsilon, hipStream_t stream)
+{
+    assert_always(num_dims == 4 || num_dims == 5);
+    if (input.get_local_size() == 0)
+        return;
+    const ChannelGeometry<Tensor> gi(input), go(output);
+    DISTCONV_CHECK_H2X(h2x_bn_batch_normalization(
+        Tensor::h2x_type(), num_samples, gi.num_channels, gi.spatial, gi.spatial_real,
+        go.spatial_real, input.get_const_base_ptr(), mean.get_const_base_ptr(),
+        var.get_const_base_ptr(), scale.get_const_base_ptr(), bias.get_const_base_ptr(),
+        output.get_base_ptr(), epsilon, stream));
+}
+
+// batchnorm.hpp:68-81
+template <typename Tensor>
+void backprop1(int num_dims, int num_samples, const Tensor& input, const Tensor& d_output,
+               const Tensor& mean, const Tensor& var, const Tensor& scale, Tensor& scale_gradient,
+               Tensor& bias_gradient, Tensor& mean_gradient, Tensor& var_gradient,
+               typename Tensor::data_type epsilon, hipStream_t stream, Workspace& ws)
+{
+    assert_always(num_dims == 4 || num_dims == 5);
+    const ChannelGeometry<Tensor> gi(input), go(d_output);
+    const bool active = input.get_local_size() > 0 && input.is_split_root();
+    DISTCONV_CHECK_H2X(h2x_bn_backprop1(
+        Tensor::h2x_type(), active ? num_samples : 0, gi.num_channels, gi.spatial, gi.spatial_real,
+        go.spatial_real, input.get_const_base_ptr(), d_output.get_const_base_ptr(),
+        mean.get_const_base_ptr(), var.get_const_base_ptr(), scale.get_const_base_ptr(),
+        scale_gradient.get_base_ptr(), bias_gradient.get_base_ptr(), mean_gradient.get_base_ptr(),
+        var_gradient.get_base_ptr(), epsilon, ws.get(gi.num_channels), stream));
+}
+
+template <typename Tensor>
+void backprop1(int num_dims, int num_samples, const Tensor& input, const Tensor& d_output,
+               const Tensor& mean, const Tensor& var, const Tensor& scale, Tensor& scale_gradient,
+               Tensor& bias_gradient, Tensor& mean_gradient, Tensor& var_gradient,
+               typename Tensor::data_type epsilon, hipStream_t stream)
+{
+    backprop1(num_dims, num_samples, input, d_output, mean, var, scale, scale_gradient,
+              bias_gradient, mean_gradient, var_gradient, epsilon, stream,
+              default_workspace(stream));
+}
+
+// batchnorm.hpp:83-96; d_input may be the same tensor as input
+template <typename Tensor>
+void backprop2(int num_dims, index_t num_samples, index_t num_per_sum, const Tensor& input,
+               const Tensor& d_output, const Tensor& mean, const Tensor& var, const Tensor& scale,
+               const Tensor& mean_gradient, const Tensor& var_gradient, Tensor& d_input,
+               typename Tensor::data_type epsilon, hipStream_t stream)
+{
+    assert_always(num_dims == 4 || num_dims == 5);
+    if (input.get_local_size() == 0)
+        return;
+    const ChannelGeometry<Tensor> gi(input), go(d_output), gd(d_input);
+    DISTCONV_CHECK_H2X(h2x_bn_backprop2(
+        Tensor::h2x_type(), static_cast<int>(num_samples), gi.num_channels, gi.spatial,
+        gi.spatial_real, go.spatial_real, gd.spatial_real, num_per_sum,
+        input.get_const_base_ptr(), d_output.get_const_base_ptr(), mean.get_const_base_ptr(),
+        var.get_const_base_ptr(), scale.get_const_base_ptr(), mean_gradient.get_const_base_ptr(),
+        var_gradient.get_const_base_ptr(), d_input.get_base_ptr(), epsilon, stream));
+}
+
+} // namespace batchnorm
+
+template <typename Backend, typename DataType>
+class BatchNormalization;
+
+// batchnorm.hpp:100-581.  The allreduce between the stages is a callable
+// `void(DataType* buf, size_t count)` (the reference's tensor::Allreduce<T>);
+// by default it is the identity: one rank, or local statistics.
+template <typename DataType>
+class BatchNormalization<BackendMI355X, DataType>
+{
+public:
+    using Allreduce = std::function<void(DataType*, size_t)>;
+
+    BatchNormalization(BackendMI355X& backend, int num_dims, DataType decay, DataType epsilon,
+                       bool global_stats, BatchnormImpl impl = BatchnormImpl::VIRTUAL)
+        : m_stream(backend.get_stream()), m_num_dims(num_dims), m_num_current_samples(0),
+          m_decay(decay), m_epsilon(epsilon), m_impl(impl), m_global_stats(global_stats)
+    {}
+
+    void set_allreducer(Allreduce fn) { m_allreducer = std::move(fn); }
+
+    template <typename Tensor>
+    int forward_stage1(const Tensor& input, Tensor& mean, Tensor& var, bool is_training)
+    {
+        set_num_samples(static_cast<int>(input.get_local_shape()[-1]));
+        if (is_training)
+            batchnorm::channel_sums_and_sqsums(m_num_dims, m_num_current_samples, input, mean, var,
+                                               m_stream, m_ws);
+        return 0;
+    }
+
+    template <typename Tensor>
+    int forward_allreduce(Tensor& mean, Tensor& var, bool is_training)
+    {
+        if (!is_training || !m_global_stats || !m_allreducer)
+            return 0;
+        fused_allreduce(mean, var);
+        return 0;
+    }
+
+    template <typename Tensor>
+    int forward_stage2(const Tensor& input, Tensor& mean, Tensor& var, Tensor& running_mean,
+                       Tensor& running_var, Tensor& scale, Tensor& bias, Tensor& output,
+                       bool is_training)
+    {
+        if (is_training)
+        {
+            batchnorm::sums_to_statistics(num_per_sum(input), m_decay, mean, var, running_mean,
+                                          running_var, m_stream);
+            batchnorm::batch_normalization(m_num_dims, m_num_current_samples, input, mean, var,
+                                           scale, bias, output, m_epsilon, m_stream);
+        }
+        else
+        {
+            batchnorm::batch_normalization(m_num_dims, m_num_current_samples, input, running_mean,
+                                           running_var, scale, bias, output, m_epsilon, m_stream);
+        }
+        return 0;
+    }
+
+    template <typename Tensor>
+    int forward(const Tensor& input, Tensor& mean, Tensor& var, Tensor& running_mean,
+                Tensor& running_var, Tensor& scale, Tensor& bias, Tensor& output, bool is_training)
+    {
+        forward_stage1(input, mean, var, is_training);
+        forward_allreduce(mean, var, is_training);
+        forward_stage2(input, mean, var, running_mean, running_var, scale, bias, output,
+                       is_training);
+        return 0;
+    }
+
+    template <typename Tensor>
+    int backward_stage1(const Tensor& input, const Tensor& d_output, const Tensor& mean,
+                        const Tensor& var, const Tensor& scale, Tensor& scale_gradient,
+                        Tensor& bias_gradient, Tensor& mean_gradient, Tensor& var_gradient)
+    {
+        set_num_samples(static_cast<int>(input.get_local_shape()[-1]));
+        batchnorm::backprop1(m_num_dims, m_num_current_samples, input, d_output, mean, var, scale,
+                             scale_gradient, bias_gradient, mean_gradient, var_gradient, m_epsilon,
+                             m_stream, m_ws);
+        return 0;
+    }
+
+    template <typename Tensor>
+    int backward_allreduce(Tensor& scale_gradient, Tensor& bias_gradient, Tensor& mean_gradient,
+                           Tensor& var_gradient, bool skip_weights = false)
+    {
+        if (!m_global_stats || !m_allreducer)
+            return 0;
+        fused_allreduce(mean_gradient, var_gradient);
+        if (!skip_weights)
+        {
+            m_allreducer(scale_gradient.get_buffer(), scale_gradient.get_local_pitched_size());
+            m_allreducer(bias_gradient.get_buffer(), bias_gradient.get_local_pitched_size());
+        }
+        return 0;
+    }
+
+    template <typename Tensor>
+    int backward_stage2(const Tensor& input, const Tensor& d_output, const Tensor& mean,
+                        const Tensor& var, const Tensor& scale, const Tensor& mean_gradient,
+                        const Tensor& var_gradient, Tensor& d_input)
+    {
+        batchnorm::backprop2(m_num_dims, m_num_current_samples, num_per_sum(input), input, d_output,
+                             mean, var, scale, mean_gradient, var_gradient, d_input, m_epsilon,
+                             m_stream);
+        return 0;
+    }
+
+    template <typename Tensor>
+    int backward(const Tensor& input, const Tensor& d_output, const Tensor& mean, const Tensor& var,
+                 const Tensor& scale, Tensor& scale_gradient, Tensor& bias_gradient,
+                 Tensor& mean_gradient, Tensor& var_gradient, Tensor& d_input)
+    {
+        backward_stage1(input, d_output, mean, var, scale, scale_gradient, bias_gradient,
+                        mean_gradient, var_gradient);
+        backward_allreduce(scale_gradient, bias_gradient, mean_gradient, var_gradient);
+        backward_stage2(input, d_output, mean, var, scale, mean_gradient, var_gradient, d_input);
+        return 0;
+    }
+
+    // n: number of samples of the current local mini-batch (batchnorm.hpp:467-475)
+    void set_num_samples(int n) { m_num_current_samples = n; }
+
+private:
+    // elements per channel of the global (global statistics) or local shape:
+    // batchnorm.hpp:232-236,414-418
+    template <typename Tensor>
+    index_t num_per_sum(const Tensor& input) const
+    {
+        const auto& s = m_global_stats ? input.get_shape() : input.get_local_shape();
+        return s[-2] ? s.get_size() / s[-2] : 0;
+    }
+
+    // mean|var (and their gradients) go out as one message when they are
+    // adjacent in memory: batchnorm.hpp:196-211,375-390
+    template <typename Tensor>
+    void fused_allreduce(Tensor& a, Tensor& b)
+    {
+        auto pa = a.get_buffer();
+        auto pb = b.get_buffer();
+        const size_t count = a.get_local_pitched_size();
+        assert_always(count == b.get_local_pitched_size());
+        if (pa + count == pb)
+            m_allreducer(pa, count * 2);
+        else if (pa == pb + count)
+            m_allreducer(pb, count * 2);
+        else
+        {
+            m_allreducer(pa, count);
+            m_allreducer(pb, count);
+        }
+    }
+
+    hipStream_t m_stream;
+    int m_num_dims;
+    int m_num_current_samples;
+    DataType m_decay;
+    DataType m_epsilon;
+    BatchnormImpl m_impl;
+    bool m_global_stats;
+    Allreduce m_allreducer;
+    batchnorm::Workspace m_ws;
+};
+
+template <typename Backend>
+class Softmax;
+
+// softmax.hpp:14-63, channel mode.
+template <>
+class Softmax<BackendMI355X>
+{
+public:
+    explicit Softmax(BackendMI355X const& backend) : m_stream(backend.get_stream()) {}
+    explicit Softmax(hipStream_t stream) : m_stream(stream) {}
+
+    template <typename Tensor>
+    void setup(const Tensor& input, SoftmaxMode mode)
+    {
+        (void) input;
+        assert_always(mode == SoftmaxMode::CHANNEL); // instance mode is not part of this path
+        m_mode = mode;
+    }
+
+    template <typename Tensor>
+    int forward(const Tensor& x, Tensor& y)
+    {
+        if (x.get_local_size() == 0)
+            return 0; // softmax.cu:600-603
+        size_t spatial;
+        int n, c;
+        geometry(x, n, c, spatial);
+        DISTCONV_CHECK_H2X(h2x_softmax_channel_forward(Tensor::h2x_type(), n, c, spatial,
+                                                       x.get_const_base_ptr(), y.get_base_ptr(),
+                                                       m_stream));
+        return 0;
+    }
+
+    template <typename Tensor>
+    int backward(const Tensor& y, const Tensor& dy, Tensor& dx)
+    {
+        if (dx.get_local_size() == 0)
+            return 0;
+        size_t spatial;
+        int n, c;
+        geometry(dx, n, c, spatial);
+        DISTCONV_CHECK_H2X(h2x_softmax_channel_backward(Tensor::h2x_type(), n, c, spatial,
+                                                        y.get_const_base_ptr(),
+                                                        dy.get_const_base_ptr(), dx.get_base_ptr(),
+                                                        m_stream));
+        return 0;
+    }
+
+private:
+    // dense [N][C][spatial] interior, as the reference assumes (softmax.cu:562-563)
+    template <typename Tensor>
+    static void geometry(const Tensor& t, int& n, int& c, size_t& spatial)
+    {
+        for (int i = 0; i < t.get_num_dims(); ++i)
+            assert_always(t.get_halo_width(i) == 0);
+        n = static_cast<int>(t.get_local_shape()[-1]);
+        c = static_cast<int>(t.get_local_shape()[-2]);
+        spatial = t.get_local_size() / n / c;
+    }
+
+    hipStream_t m_stream;
+    SoftmaxMode m_mode = SoftmaxMode::CHANNEL;
+};
+
+} // namespace distconv

@@ -1,0 +1,91 @@
+// Halo exchange through the C++ layer, checked by the closed form of
+// legacy/tests/tensor/test_halo_exchange_cuda.cu:104-233: after the exchange
+// every halo cell whose source exists (or wraps, on a periodic grid) holds the
+// global offset of its source.
+#include "test_common.hpp"
+
+static int run_case(const Shape& shape, const Shape& locale, const IntVector& overlap, bool periodic)
+{
+    const int nd = shape.length();
+    const int n = static_cast<int>(locale.get_size());
+    const Distribution dist = Distribution::make_overlapped_distribution(locale, overlap);
+    std::vector<std::unique_ptr<DevTensor<float>>> ranks;
+    std::vector<DevTensor<float>*> ptrs;
+    for (int r = 0; r < n; ++r)
+    {
+        ranks.emplace_back(new DevTensor<float>(shape, LocaleVirtual(r, n), dist));
+        CHECK(ranks.back()->allocate() == 0);
+        to_device(*ranks.back(), global_offset_field(*ranks.back(), -1.0f));
+        ptrs.push_back(ranks.back().get());
+    }
+    HaloExchangeVirtual<float> xch(ptrs, periodic);
+    for (int d = 0; d < nd; ++d) // Convolution clears the halo before every exchange
+        for (auto* t : ptrs)
+            t->clear_halo(d, nullptr);
+    xch.exchange(nullptr);
+    int errors = 0;
+    for (int r = 0; r < n; ++r)
+    {
+        auto& t = *ranks[r];
+        std::vector<float> h = to_host(t);
+        const Shape& rs = t.get_local_real_shape();
+        for (index_t o = 0; o < h.size(); ++o)
+        {
+            IndexVector idx = rs.get_index(o);
+            IndexVector g(nd, 0);
+            bool exists = true;
+            for (int i = 0; i < nd; ++i)
+            {
+                long long c = static_cast<long long>(idx[i] + t.get_global_index()[i]) - t.get_halo_width(i);
+                const long long ext = static_cast<long long>(shape[i]);
+                if (periodic && t.get_distribution().is_distributed(i))
+                    c = (c % ext + ext) % ext;
+                if (c < 0 || c >= ext)
+                    exists = false;
+                g[i] = static_cast<index_t>(c < 0 ? 0 : c);
+            }
+            const float want = exists ? static_cast<float>(get_offset(g, shape)) : 0.0f; // cleared
+            if (h[o] != want)
+            {
+                if (errors < 5)
+                    std::printf("rank %d offset %zu: got %f want %f\n", r, (size_t) o, h[o], want);
+                ++errors;
+            }
+        }
+    }
+    return errors;
+}
+
+int main()
+{
+    int errors = 0;
+    for (bool periodic : {false, true})
+    {
+        errors += run_case(Shape({12, 10, 3, 2}), Shape({2, 2, 1, 1}), IntVector({1, 1, 0, 0}), periodic);
+        errors += run_case(Shape({12, 10, 3, 2}), Shape({2, 2, 1, 1}), IntVector({2, 2, 0, 0}), periodic);
+        errors += run_case(Shape({13, 11, 3, 2}), Shape({3, 2, 1, 1}), IntVector({1, 2, 0, 0}), periodic);
+        errors += run_case(Shape({8, 10, 12, 3, 2}), Shape({2, 2, 2, 1, 1}), IntVector({1, 1, 1, 0, 0}), periodic);
+        errors += run_case(Shape({8, 9, 10, 2, 1}), Shape({1, 2, 2, 1, 1}), IntVector({0, 2, 1, 0, 0}), periodic);
+    }
+    // per-rank interface: pack one strip, unpack it on the neighbour
+    {
+        const Shape shape({8, 6, 2, 1}), locale({2, 1, 1, 1});
+        const Distribution dist = Distribution::make_overlapped_distribution(locale, IntVector({1, 0, 0, 0}));
+        DevTensor<float> a(shape, LocaleVirtual(0, 2), dist), b(shape, LocaleVirtual(1, 2), dist);
+        a.allocate();
+        b.allocate();
+        to_device(a, global_offset_field(a, -1.0f));
+        to_device(b, global_offset_field(b, -1.0f));
+        HaloExchangeVirtual<float> xch({&a, &b});
+        CHECK(xch.rank(0).get_peer(0, RHS) == 1 && xch.rank(0).get_peer(0, LHS) == kProcNull);
+        CHECK(xch.rank(0).get_halo_size(0, 1) == 6 * 2 * 1);
+        xch.rank(0).pack_dim(0, RHS, 1, nullptr, xch.rank(1).get_recv_buffer(0, LHS), false);
+        CHECK(xch.rank(1).unpack(0, 0, 1, nullptr, nullptr, false));
+        std::vector<float> h = to_host(b);
+        for (int y = 0; y < 6; ++y) // b's LHS halo column holds global x = 3
+            if (h[y * 6 + 0] != static_cast<float>(3 + 8 * y))
+                ++errors;
+    }
+    std::printf("test_halo_exchange_virtual: %d errors\n", errors);
+    return errors ? 1 : 0;
+}
