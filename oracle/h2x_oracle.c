@@ -9,8 +9,11 @@
  * Python binding) may call, link or import it.
  *
  * Each function names the reference file:line it follows (paths relative to
- * the reference checkout).  Parity status of each function -- what pins it
- * besides reading the reference -- is listed in oracle/README.md.
+ * the reference checkout).  What pins each function besides reading the
+ * reference is listed in oracle/README.md.  PARITY UNPINNED: the FLT_MIN
+ * clamp, the y > FLT_MIN guard and the FLT_MIN initial maximum of channel
+ * softmax -- the reference holds no softmax test or vector; everything else
+ * of softmax is pinned by the textbook routine.
  *
  * Build: see oracle/Makefile (gcc -O3 -fopenmp, -ffp-contract=off so that the
  * only fused multiply-adds are the ones written explicitly).
