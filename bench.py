@@ -32,9 +32,13 @@ def _gbs(nbytes: float, ms: float) -> float:
     return nbytes / (ms * 1e-3) / 1e9 if ms > 0 else 0.0
 
 
-def _time_events(fn, iters: int, warmup: int):
-    """Median and minimum milliseconds of fn() measured with events on the
-    current stream (the stream every kernel of fn is launched on)."""
+def _time_events(fn, iters: int, warmup: int, inner: int = 4):
+    """Median and minimum milliseconds of one fn() measured with events on the
+    current stream (the stream every kernel of fn is launched on).  `inner`
+    calls are issued back to back between the two events so that the launch
+    latency of a call is hidden behind the execution of the previous one -- the
+    reference's harness hides it with a spin kernel
+    (legacy/benchmarks/distconv_benchmark_bn.cpp:254-295)."""
     import torch
     for _ in range(warmup):
         fn()
@@ -43,10 +47,11 @@ def _time_events(fn, iters: int, warmup: int):
     for _ in range(iters):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
-        fn()
+        for _ in range(inner):
+            fn()
         e1.record()
         e1.synchronize()
-        times.append(e0.elapsed_time(e1))
+        times.append(e0.elapsed_time(e1) / inner)
     return statistics.median(times), min(times)
 
 
@@ -211,6 +216,37 @@ def cpu_baseline(repeats: int = 3):
     }
 
 
+# HBM traffic per launch measured with rocprofv3 --pmc (profiles/bench_pmc_traffic.txt):
+# FETCH_SIZE and WRITE_SIZE in KiB per dispatch; FETCH_SIZE reads 0.5x for full-line
+# streaming reads on this stack (calibrated there on a copy of known size), WRITE_SIZE 1.0x.
+PMC_KIB = {  # label -> (FETCH_SIZE KiB, fetch scale, WRITE_SIZE KiB)
+    "bn_sums": (131096, 2.0, 128),
+    "bn_apply": (131093, 2.0, 262144),
+    "bn_backprop1": (262185, 2.0, 128),
+    "bn_backprop2": (262174, 2.0, 262144),
+    "halo_dim0_pack": (314300, 2.0, 33800),
+    "halo_dim0_unpack": (16952, 2.0, 270400),
+    "halo_dim1_pack": (21104, 2.0, 33800),
+    "halo_dim1_unpack": (16960, 2.0, 35495),
+    "halo_dim2_pack": (17126, 2.0, 33800),
+    "halo_dim2_unpack": (16960, 2.0, 33909),
+}
+
+KERNEL_OF = {
+    "bn_sums": "bn_sums_kernel<float,4> (+bn_finish_kernel<float,2>)",
+    "bn_statistics": "bn_statistics_kernel<float>",
+    "bn_apply": "bn_apply_kernel<float,4>",
+    "bn_backprop1": "bn_backprop1_kernel<float,4> (+bn_finish_kernel<float,4>)",
+    "bn_backprop2": "bn_backprop2_kernel<float,4>",
+    "halo_dim0_pack": "box_copy_kernel<u32,1,OpId,sparse>",
+    "halo_dim0_unpack": "box_copy_kernel<u32,1,OpId,sparse>",
+    "halo_dim1_pack": "box_copy_kernel<u32,2,OpId>",
+    "halo_dim1_unpack": "box_copy_kernel<u32,2,OpId>",
+    "halo_dim2_pack": "box_copy_kernel<u32,4,OpId>",
+    "halo_dim2_unpack": "box_copy_kernel<u32,4,OpId>",
+}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -238,46 +274,103 @@ def main() -> int:
     bn_bytes = 8 * S3 * 4
     step_bytes = bn_bytes + halo.bytes
     step_elems = S3 + halo.elems
+    launch_bytes = halo.bytes // 6  # one launch: pack or unpack of the 16 faces of one dimension (read + write)
+    algo_bytes = {"bn_sums": S3 * 4, "bn_statistics": 0, "bn_apply": 2 * S3 * 4, "bn_backprop1": 2 * S3 * 4,
+                  "bn_backprop2": 3 * S3 * 4}
+    for d in range(3):
+        algo_bytes[f"halo_dim{d}_pack"] = launch_bytes
+        algo_bytes[f"halo_dim{d}_unpack"] = launch_bytes
 
-    k_events = []
+    # Every launch of the step is bracketed by a pair of events on the stream it is
+    # launched on (torch's current stream, whose handle the C ABI receives).
+    events = {}
+    recording = [False]
+    only = [None]  # labels to instrument; None = all
 
-    def step(timed: bool):
-        bn3.forward()
-        bn3.backward_reduce()
-        if timed:
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            bn3.backward_apply()
-            e1.record()
-            k_events.append((e0, e1))
-        else:
-            bn3.backward_apply()
+    def timed(label, launch):
+        if not recording[0] or (only[0] is not None and label not in only[0]):
+            launch()
+            return
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        launch()
+        e1.record()
+        events.setdefault(label, []).append((e0, e1))
+
+    halo.xch.launch_hook = timed
+    b = bn3.bn
+    nps = b._num_per_sum(bn3.x)
+
+    def step():
+        timed("bn_sums", lambda: b.forward_stage1(bn3.x, bn3.mean, bn3.var, True))
+        b.forward_allreduce(bn3.mean, bn3.var, True)
+        timed("bn_statistics", lambda: b.sums_to_statistics(nps, bn3.mean, bn3.var, bn3.rm, bn3.rv))
+        timed("bn_apply", lambda: b.batch_normalization(bn3.x, bn3.mean, bn3.var, bn3.scale, bn3.bias, bn3.y))
+        timed("bn_backprop1", bn3.backward_reduce)
+        timed("bn_backprop2", bn3.backward_apply)
         halo.run()
 
-    for _ in range(args.warmup):
-        step(False)
+    def kernel_share(evs):
+        tot = {}
+        for label, pairs in evs.items():
+            ms = statistics.mean(e0.elapsed_time(e1) for e0, e1 in pairs)
+            tot[KERNEL_OF[label]] = tot.get(KERNEL_OF[label], 0.0) + ms
+        return tot
+
+    # warm-up, with every launch bracketed by events: finds the dominant kernel
+    recording[0] = True
+    for _ in range(max(args.warmup, 1)):
+        step()
     torch.cuda.synchronize()
+    share0 = kernel_share(events)
+    dominant = max(share0, key=share0.get)
+    events.clear()
+
+    # timed region: only the dominant kernel's launches carry events
+    only[0] = {l for l, k in KERNEL_OF.items() if k == dominant}
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        step(True)
+        step()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / args.steps
     value = _gbs(step_bytes, ms_per_step)
+    dominant_events = dict(events)
+    events.clear()
 
-    # dominant kernel: bn_backprop2_kernel (reads x and dy, writes dx: 3 * S * 4 bytes)
-    k_ms = statistics.mean(e0.elapsed_time(e1) for e0, e1 in k_events)
-    k_bytes = 3 * S3 * 4
+    # a second, fully instrumented pass for the per-launch table
+    only[0] = None
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    recording[0] = False
+    halo.xch.launch_hook = None
+    for label, pairs in dominant_events.items():
+        events[label] = pairs  # the dominant kernel's figures come from the timed region
+
+    launches = {}
+    for label, pairs in events.items():
+        ms = statistics.mean(e0.elapsed_time(e1) for e0, e1 in pairs)
+        fetch_kib, scale, write_kib = PMC_KIB.get(label, (0, 0.0, 0))
+        launches[label] = {
+            "kernel": KERNEL_OF[label], "avg_launch_ms": ms, "algorithmic_bytes": algo_bytes[label],
+            "GB/s": _gbs(algo_bytes[label], ms), "frac": _gbs(algo_bytes[label], ms) / HBM_PEAK_GBS,
+            "traffic": int((fetch_kib * scale + write_kib) * 1024) if label in PMC_KIB else None,
+        }
+    # dominant kernel = the kernel with the largest share of the step's launch time
+    share = {}
+    for label, v in launches.items():
+        share.setdefault(v["kernel"], []).append(label)
+    dl = share[dominant]
+    d_ms = statistics.mean(launches[l]["avg_launch_ms"] for l in dl)
+    d_bytes = statistics.mean(launches[l]["algorithmic_bytes"] for l in dl)
+    d_traffic = statistics.mean(launches[l]["traffic"] for l in dl)
     roofline = {
-        "kernel": "bn_backprop2_kernel<float,4>",
-        "bound": "hbm",
-        "achieved": _gbs(k_bytes, k_ms),
-        "peak": HBM_PEAK_GBS,
-        "unit": "GB/s",
-        "frac": _gbs(k_bytes, k_ms) / HBM_PEAK_GBS,
-        "traffic": None,
-        "avg_launch_ms": k_ms,
-        "algorithmic_bytes": k_bytes,
+        "kernel": dominant, "launches_per_step": dl, "bound": "hbm",
+        "achieved": _gbs(d_bytes, d_ms), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": _gbs(d_bytes, d_ms) / HBM_PEAK_GBS, "traffic": int(d_traffic),
+        "avg_launch_ms": d_ms, "algorithmic_bytes": int(d_bytes),
+        "traffic_GB/s": _gbs(d_traffic, d_ms),
     }
 
     breakdown = {}
@@ -297,7 +390,10 @@ def main() -> int:
             ov = [1 if k == d else 0 for k in range(5)]
             fn = lambda ov=ov: halo.xch.exchange(ov, ov, ov, ov)
             breakdown[f"C2_halo_{name}"] = entry(halo.bytes // 3, halo.elems // 3, *_time_events(fn, it, wu))
-        del bn3, halo
+        yard_x, yard_y = bn3.x.data, bn3.y.data
+        breakdown["yardstick_torch_copy_268MB"] = entry(
+            2 * S3 * 4, S3, *_time_events(lambda: yard_y.copy_(yard_x), it, wu))
+        del bn3, halo, b, yard_x, yard_y
         torch.cuda.empty_cache()
         bn1 = BatchNormWorkload((8, 64, 56, 56), SEED + 1)
         breakdown["C1_bn2d_fwd_warm"] = entry(3 * bn1.elems * 4, bn1.elems, *_time_events(bn1.forward, it, wu))
@@ -337,6 +433,7 @@ def main() -> int:
         "elements_per_s": step_elems / (ms_per_step * 1e-3),
         "roofline": roofline,
         "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline(),
+        "launches": launches,
         "breakdown": breakdown,
     }
     print(json.dumps(out))

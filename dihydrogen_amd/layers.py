@@ -101,22 +101,30 @@ class BatchNormalization:
             self.allreduce([mean, var])
         return 0
 
-    def forward_stage2(self, input: Tensor, mean, var, running_mean, running_var, scale, bias,
-                       output: Tensor, is_training: bool = True) -> int:
+    def sums_to_statistics(self, num_per_sum: int, mean, var, running_mean, running_var,
+                           dtype: int = capi.F32) -> None:
+        """batchnorm.hpp:494-503."""
+        capi.check(self._lib.h2x_bn_sums_to_statistics(
+            dtype, mean.numel(), num_per_sum, self.decay, _ptr(mean), _ptr(var), _ptr(running_mean),
+            _ptr(running_var), _stream_handle(self.stream)), "sums_to_statistics")
+
+    def batch_normalization(self, input: Tensor, mean, var, scale, bias, output: Tensor) -> None:
+        """batchnorm.hpp:505-517."""
         n, c, s, sr = _channel_geometry(input)
         _, _, so, sro = _channel_geometry(output)
-        st = _stream_handle(self.stream)
-        if is_training:
-            capi.check(self._lib.h2x_bn_sums_to_statistics(
-                input.h2x_dtype, c, self._num_per_sum(input), self.decay, _ptr(mean), _ptr(var),
-                _ptr(running_mean), _ptr(running_var), st), "sums_to_statistics")
-            m, v = mean, var
-        else:
-            m, v = running_mean, running_var  # batchnorm.hpp:243-247
         capi.check(self._lib.h2x_bn_batch_normalization(
             input.h2x_dtype, self.num_current_samples, c, s, sr, sro, _ptr(input.get_base_ptr()),
-            _ptr(m), _ptr(v), _ptr(scale), _ptr(bias), _ptr(output.get_base_ptr()), self.epsilon, st),
-            "batch_normalization")
+            _ptr(mean), _ptr(var), _ptr(scale), _ptr(bias), _ptr(output.get_base_ptr()), self.epsilon,
+            _stream_handle(self.stream)), "batch_normalization")
+
+    def forward_stage2(self, input: Tensor, mean, var, running_mean, running_var, scale, bias,
+                       output: Tensor, is_training: bool = True) -> int:
+        if is_training:
+            self.sums_to_statistics(self._num_per_sum(input), mean, var, running_mean, running_var,
+                                    input.h2x_dtype)
+            self.batch_normalization(input, mean, var, scale, bias, output)
+        else:
+            self.batch_normalization(input, running_mean, running_var, scale, bias, output)  # :243-247
         return 0
 
     def forward(self, input, mean, var, running_mean, running_var, scale, bias, output,
@@ -249,6 +257,8 @@ class HaloExchangeVirtual:
         self.nd = t0.get_num_dims()
         self._recv = {}  # (rank, dim, side) -> torch buffer the rank unpacks from
         self._faces = {}  # exchange arguments -> (pack faces, unpack faces)
+        # optional callable(label, launch): wraps every launch, for per-kernel timing
+        self.launch_hook = None
 
     def get_halo_size(self, rank: int, dim: int, width: int) -> int:
         """halo_exchange_cuda.hpp:267-271."""
@@ -334,10 +344,15 @@ class HaloExchangeVirtual:
             cached = tuple((capi.HaloFace * len(f))(*f) if f else None for f in (packs, unpacks))
             self._faces[key] = cached
         st = _stream_handle(self.stream)
-        for arr in cached:
-            if arr is not None:
-                capi.check(self._lib.h2x_halo_pack_or_unpack_batched(dtype, arr, len(arr), st),
-                           "halo pack/unpack")
+        for what, arr in zip(("pack", "unpack"), cached):
+            if arr is None:
+                continue
+            launch = lambda arr=arr: capi.check(
+                self._lib.h2x_halo_pack_or_unpack_batched(dtype, arr, len(arr), st), "halo pack/unpack")
+            if self.launch_hook is None:
+                launch()
+            else:
+                self.launch_hook(f"halo_dim{dim}_{what}", launch)
 
     def exchange(self, widths_rhs_send=None, widths_rhs_recv=None, widths_lhs_send=None,
                  widths_lhs_recv=None, is_reverse: bool = False, skip_unpack: bool = False,
