@@ -41,6 +41,16 @@ class HaloFace(ctypes.Structure):
     ]
 
 
+class TensorGeometry(ctypes.Structure):
+    """struct h2x_tensor_geometry"""
+    _fields_ = [
+        ("num_dims", c_int32),
+        ("reserved", c_int32),
+        ("local_shape", c_int64 * H2X_MAX_DIMS),
+        ("strides", c_int64 * H2X_MAX_DIMS),
+    ]
+
+
 class ShuffleGeometry(ctypes.Structure):
     """struct h2x_shuffle_geometry"""
     _fields_ = [
@@ -72,6 +82,19 @@ SIGNATURES = {
     "h2x_bn_backprop2": (c_int, [c_int, c_int, c_int, c_size_t, c_size_t, c_size_t, c_size_t,
                                  c_size_t, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_void_p, c_void_p, c_void_p, c_double, c_void_p]),
+    "h2x_bn_channel_sums_and_sqsums_strided": (c_int, [c_int, c_int, POINTER(TensorGeometry), c_void_p,
+                                                       c_void_p, c_void_p, c_void_p, c_void_p]),
+    "h2x_bn_batch_normalization_strided": (c_int, [c_int, c_int, POINTER(TensorGeometry),
+                                                   POINTER(TensorGeometry), c_void_p, c_void_p,
+                                                   c_void_p, c_void_p, c_void_p, c_void_p, c_double,
+                                                   c_void_p]),
+    "h2x_bn_backprop1_strided": (c_int, [c_int, c_int, POINTER(TensorGeometry), POINTER(TensorGeometry),
+                                         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                         c_void_p, c_void_p, c_void_p, c_double, c_void_p, c_void_p]),
+    "h2x_bn_backprop2_strided": (c_int, [c_int, c_int, c_size_t, POINTER(TensorGeometry),
+                                         POINTER(TensorGeometry), POINTER(TensorGeometry), c_void_p,
+                                         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                         c_void_p, c_double, c_void_p]),
     "h2x_softmax_channel_forward": (c_int, [c_int, c_int, c_int, c_size_t, c_void_p, c_void_p,
                                             c_void_p]),
     "h2x_softmax_channel_backward": (c_int, [c_int, c_int, c_int, c_size_t, c_void_p, c_void_p,

@@ -1,10 +1,15 @@
 // Channel-wise batch-normalisation kernels for gfx950 and their C entry points.
 //
-// Layout: element (n, c, i) of a tensor lives at base[(n*C + c)*real + i],
-// i < spatial -- the geometry of the reference's optimised kernels
-// (legacy/src/dnn_backend/batchnorm.cu:134-190).  Every kernel is a pure HBM
-// stream: 16-byte loads when the geometry allows, several loads in flight per
-// lane, per-channel parameters fetched once per workgroup.
+// Two layouts.  Dense: element (n, c, i) of a tensor lives at
+// base[(n*C + c)*real + i], i < spatial -- the geometry of the reference's
+// optimised kernels (legacy/src/dnn_backend/batchnorm.cu:134-190).  Strided:
+// the interior of a tensor with halos on any spatial dimension, addressed
+// through the tensor's strides like the reference's generic kernels
+// (batchnorm.cu:39-90,369-418,899-980,1303-1369); the flat interior index of
+// an element is split into (x, y, z) with multiply-high divisions and rows are
+// read with unaligned vectors.  Every kernel is a pure HBM stream: 16-byte
+// accesses when the geometry allows, several loads in flight per lane,
+// per-channel parameters fetched once per workgroup.
 //
 // Reductions (forward sums, backward sums) cut every channel into contiguous
 // chunks, one workgroup per chunk.  A thread accumulates in fp64, the
@@ -71,15 +76,36 @@ Chunking make_chunking(size_t spatial, size_t segments, size_t budget, size_t ti
     return c;
 }
 
-#define H2X_RETURN_IF_ERROR(expr)                                                                  \
-    do                                                                                             \
-    {                                                                                              \
-        int h2x_err_ = (expr);                                                                     \
-        if (h2x_err_ != 0)                                                                         \
-            return h2x_err_;                                                                       \
-    } while (0)
+// Where the elements of one tensor live.  Element i (flat index over the
+// interior spatial extents, innermost first) of segment (n, c) is at
+// base[n*stride_n + c*stride_c + offset(i)]; offset(i) = i for the dense layout.
+struct TensorMap
+{
+    int64_t stride_n, stride_c;
+    FastDiv w, h;     // interior extents of spatial dimensions 0 and 1 (strided layout)
+    int64_t sy, sz;   // strides of spatial dimensions 1 and 2 (strided layout)
+};
 
-template <typename T, int VEC>
+template <bool STRIDED>
+__device__ __forceinline__ size_t seg_offset(const TensorMap& m, size_t i)
+{
+    if constexpr (!STRIDED)
+    {
+        return i;
+    }
+    else
+    {
+        const uint32_t t = fastdiv(static_cast<uint32_t>(i), m.w);
+        const uint32_t x = static_cast<uint32_t>(i) - t * m.w.divisor;
+        const uint32_t z = fastdiv(t, m.h);
+        const uint32_t y = t - z * m.h.divisor;
+        return x + y * static_cast<size_t>(m.sy) + z * static_cast<size_t>(m.sz);
+    }
+}
+
+// ALIGNED: the address is a multiple of the vector size (dense layout); rows
+// of a strided tensor may start on any element.
+template <typename T, int VEC, bool ALIGNED = true>
 __device__ __forceinline__ void load_vec(const T* p, T (&r)[VEC])
 {
     if constexpr (VEC == 1)
@@ -88,7 +114,7 @@ __device__ __forceinline__ void load_vec(const T* p, T (&r)[VEC])
     }
     else
     {
-        typedef T V __attribute__((ext_vector_type(VEC)));
+        typedef T V __attribute__((ext_vector_type(VEC), aligned(ALIGNED ? sizeof(T) * VEC : sizeof(T))));
         const V t = *reinterpret_cast<const V*>(p);
 #pragma unroll
         for (int j = 0; j < VEC; ++j)
@@ -96,7 +122,7 @@ __device__ __forceinline__ void load_vec(const T* p, T (&r)[VEC])
     }
 }
 
-template <typename T, int VEC>
+template <typename T, int VEC, bool ALIGNED = true>
 __device__ __forceinline__ void store_vec(T* p, const T (&r)[VEC])
 {
     if constexpr (VEC == 1)
@@ -105,7 +131,7 @@ __device__ __forceinline__ void store_vec(T* p, const T (&r)[VEC])
     }
     else
     {
-        typedef T V __attribute__((ext_vector_type(VEC)));
+        typedef T V __attribute__((ext_vector_type(VEC), aligned(ALIGNED ? sizeof(T) * VEC : sizeof(T))));
         V t;
 #pragma unroll
         for (int j = 0; j < VEC; ++j)
@@ -186,59 +212,56 @@ __global__ __launch_bounds__(kBlockSize) void bn_finish_kernel(
 
 // ---- forward: sums and sums of squares --------------------------------------
 // Replaces channel_sums_and_sqsums_opt_kernel, batchnorm.cu:92-132.
-template <typename T, int VEC>
+template <typename T, int VEC, bool STRIDED>
 __global__ __launch_bounds__(kBlockSize) void bn_sums_kernel(
     const T* __restrict__ x, T* __restrict__ sums, T* __restrict__ sqsums, double* partials,
-    int num_channels, size_t spatial, size_t spatial_real, size_t chunk,
-    int chunks_per_seg, unsigned int num_units, int groups_per_channel_max)
+    const TensorMap mx, size_t spatial, size_t chunk, int chunks_per_seg, unsigned int num_units,
+    int groups_per_channel_max)
 {
     const int c = blockIdx.y;
     constexpr size_t kStride = static_cast<size_t>(kBlockSize) * VEC;
     constexpr size_t kTile = kStride * kUnroll;
     double acc[2] = {0.0, 0.0};
-    // unit = (sample, chunk); a workgroup takes units blockIdx.x, +gridDim.x, ...
+
+    auto accumulate = [&](T v) {
+        const double d = static_cast<double>(v);
+        acc[0] += d;
+        if constexpr (sizeof(T) == 4)
+            acc[1] = __builtin_fma(d, d, acc[1]); // the product of two floats is exact in fp64
+        else
+            acc[1] += d * d;
+    };
+
+    // unit = (sample, chunk); a workgroup takes units blockIdx.x, blockIdx.x + gridDim.x, ...
     for (unsigned int unit = blockIdx.x; unit < num_units; unit += gridDim.x)
     {
-    const int n = unit / chunks_per_seg;
-    const int k = unit - n * chunks_per_seg;
-    const size_t begin = static_cast<size_t>(k) * chunk;
-    const size_t end = begin + chunk < spatial ? begin + chunk : spatial;
-    const T* p = x + (static_cast<size_t>(n) * num_channels + c) * spatial_real;
-    size_t tile = begin;
-    for (; tile + kTile <= end; tile += kTile)
-    {
-        T v[kUnroll][VEC];
+        const int n = unit / chunks_per_seg;
+        const int k = unit - n * chunks_per_seg;
+        const size_t begin = static_cast<size_t>(k) * chunk;
+        const size_t end = begin + chunk < spatial ? begin + chunk : spatial;
+        const T* p = x + n * mx.stride_n + c * mx.stride_c;
+        size_t tile = begin;
+        for (; tile + kTile <= end; tile += kTile)
+        {
+            T v[kUnroll][VEC];
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u)
-            load_vec<T, VEC>(p + tile + u * kStride + threadIdx.x * VEC, v[u]);
+            for (int u = 0; u < kUnroll; ++u)
+                load_vec<T, VEC, !STRIDED>(
+                    p + seg_offset<STRIDED>(mx, tile + u * kStride + threadIdx.x * VEC), v[u]);
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u)
+            for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+                    accumulate(v[u][j]);
+        }
+        for (size_t i = tile + threadIdx.x * VEC; i < end; i += kStride)
+        {
+            T v[VEC];
+            load_vec<T, VEC, !STRIDED>(p + seg_offset<STRIDED>(mx, i), v);
 #pragma unroll
             for (int j = 0; j < VEC; ++j)
-            {
-                const double d = static_cast<double>(v[u][j]);
-                acc[0] += d;
-                if constexpr (sizeof(T) == 4)
-                    acc[1] = __builtin_fma(d, d, acc[1]); // product of two floats is exact
-                else
-                    acc[1] += d * d;
-            }
-    }
-    for (size_t i = tile + threadIdx.x * VEC; i < end; i += kStride)
-    {
-        T v[VEC];
-        load_vec<T, VEC>(p + i, v);
-#pragma unroll
-        for (int j = 0; j < VEC; ++j)
-        {
-            const double d = static_cast<double>(v[j]);
-            acc[0] += d;
-            if constexpr (sizeof(T) == 4)
-                acc[1] = __builtin_fma(d, d, acc[1]);
-            else
-                acc[1] += d * d;
+                accumulate(v[j]);
         }
-    }
     }
     if (finish_workgroup<2>(acc, partials, c, groups_per_channel_max) && threadIdx.x == 0)
     {
@@ -284,11 +307,11 @@ __global__ void bn_statistics_kernel(int num_channels, size_t num_per_sum, T dec
 
 // ---- forward: normalise ------------------------------------------------------
 // Replaces batch_normalization_opt_kernel, batchnorm.cu:420-455.
-template <typename T, int VEC>
+template <typename T, int VEC, bool STRIDED>
 __global__ __launch_bounds__(kBlockSize) void bn_apply_kernel(
     const T* __restrict__ x, const T* __restrict__ mean, const T* __restrict__ var,
     const T* __restrict__ scale, const T* __restrict__ bias, T* __restrict__ y, T epsilon,
-    int num_channels, size_t spatial, size_t x_real, size_t y_real, size_t chunk,
+    int num_channels, size_t spatial, const TensorMap mx, const TensorMap my, size_t chunk,
     int chunks_per_seg)
 {
     const size_t seg = blockIdx.x / chunks_per_seg;
@@ -300,8 +323,9 @@ __global__ __launch_bounds__(kBlockSize) void bn_apply_kernel(
     const T bi = bias[c];
     const size_t begin = static_cast<size_t>(k) * chunk;
     const size_t end = begin + chunk < spatial ? begin + chunk : spatial;
-    const T* xp = x + seg * x_real;
-    T* yp = y + seg * y_real;
+    const size_t n = seg / num_channels;
+    const T* xp = x + n * mx.stride_n + c * mx.stride_c;
+    T* yp = y + n * my.stride_n + c * my.stride_c;
 
     constexpr size_t kStride = static_cast<size_t>(kBlockSize) * VEC;
     constexpr size_t kTile = kStride * kUnroll;
@@ -311,37 +335,38 @@ __global__ __launch_bounds__(kBlockSize) void bn_apply_kernel(
         T v[kUnroll][VEC];
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u)
-            load_vec<T, VEC>(xp + tile + u * kStride + threadIdx.x * VEC, v[u]);
+            load_vec<T, VEC, !STRIDED>(
+                xp + seg_offset<STRIDED>(mx, tile + u * kStride + threadIdx.x * VEC), v[u]);
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u)
         {
 #pragma unroll
             for (int j = 0; j < VEC; ++j)
                 v[u][j] = fma_t((v[u][j] - m) * inv_stdev, sc, bi);
-            store_vec<T, VEC>(yp + tile + u * kStride + threadIdx.x * VEC, v[u]);
+            store_vec<T, VEC, !STRIDED>(
+                yp + seg_offset<STRIDED>(my, tile + u * kStride + threadIdx.x * VEC), v[u]);
         }
     }
     for (size_t i = tile + threadIdx.x * VEC; i < end; i += kStride)
     {
         T v[VEC];
-        load_vec<T, VEC>(xp + i, v);
+        load_vec<T, VEC, !STRIDED>(xp + seg_offset<STRIDED>(mx, i), v);
 #pragma unroll
         for (int j = 0; j < VEC; ++j)
             v[j] = fma_t((v[j] - m) * inv_stdev, sc, bi);
-        store_vec<T, VEC>(yp + i, v);
+        store_vec<T, VEC, !STRIDED>(yp + seg_offset<STRIDED>(my, i), v);
     }
 }
 
 // ---- backward: per-channel sums ----------------------------------------------
 // Replaces backprop1_opt_kernel, batchnorm.cu:982-1054.
-template <typename T, int VEC>
+template <typename T, int VEC, bool STRIDED>
 __global__ __launch_bounds__(kBlockSize) void bn_backprop1_kernel(
     const T* __restrict__ x, const T* __restrict__ dy, const T* __restrict__ mean,
     const T* __restrict__ var, const T* __restrict__ scale, T* __restrict__ dscale,
     T* __restrict__ dbias, T* __restrict__ dmean, T* __restrict__ dvar, T epsilon,
-    double* partials, int num_channels, size_t spatial, size_t x_real,
-    size_t dy_real, size_t chunk, int chunks_per_seg, unsigned int num_units,
-    int groups_per_channel_max)
+    double* partials, size_t spatial, const TensorMap mx, const TensorMap md, size_t chunk,
+    int chunks_per_seg, unsigned int num_units, int groups_per_channel_max)
 {
     const int c = blockIdx.y;
     const T m = mean[c];
@@ -374,9 +399,8 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop1_kernel(
         const int k = unit - n * chunks_per_seg;
         const size_t begin = static_cast<size_t>(k) * chunk;
         const size_t end = begin + chunk < spatial ? begin + chunk : spatial;
-        const size_t seg = static_cast<size_t>(n) * num_channels + c;
-        const T* xp = x + seg * x_real;
-        const T* dp = dy + seg * dy_real;
+        const T* xp = x + n * mx.stride_n + c * mx.stride_c;
+        const T* dp = dy + n * md.stride_n + c * md.stride_c;
         size_t tile = begin;
         for (; tile + kTile <= end; tile += kTile)
         {
@@ -384,8 +408,9 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop1_kernel(
 #pragma unroll
             for (int u = 0; u < kUnroll2; ++u)
             {
-                load_vec<T, VEC>(xp + tile + u * kStride + threadIdx.x * VEC, xv[u]);
-                load_vec<T, VEC>(dp + tile + u * kStride + threadIdx.x * VEC, dv[u]);
+                const size_t i = tile + u * kStride + threadIdx.x * VEC;
+                load_vec<T, VEC, !STRIDED>(xp + seg_offset<STRIDED>(mx, i), xv[u]);
+                load_vec<T, VEC, !STRIDED>(dp + seg_offset<STRIDED>(md, i), dv[u]);
             }
 #pragma unroll
             for (int u = 0; u < kUnroll2; ++u)
@@ -396,8 +421,8 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop1_kernel(
         for (size_t i = tile + threadIdx.x * VEC; i < end; i += kStride)
         {
             T xv[VEC], dv[VEC];
-            load_vec<T, VEC>(xp + i, xv);
-            load_vec<T, VEC>(dp + i, dv);
+            load_vec<T, VEC, !STRIDED>(xp + seg_offset<STRIDED>(mx, i), xv);
+            load_vec<T, VEC, !STRIDED>(dp + seg_offset<STRIDED>(md, i), dv);
 #pragma unroll
             for (int j = 0; j < VEC; ++j)
                 accumulate(xv[j], dv[j]);
@@ -416,12 +441,12 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop1_kernel(
 // Replaces backprop2_opt_kernel, batchnorm.cu:1371-1418.  x and dx may alias:
 // each thread reads its elements before it writes them, so neither is
 // restrict-qualified.
-template <typename T, int VEC>
+template <typename T, int VEC, bool STRIDED>
 __global__ __launch_bounds__(kBlockSize) void bn_backprop2_kernel(
     const T* x, const T* __restrict__ dy, const T* __restrict__ mean,
     const T* __restrict__ var, const T* __restrict__ scale, const T* __restrict__ dmean,
     const T* __restrict__ dvar, T* dx, T epsilon, size_t num_per_sum, int num_channels,
-    size_t spatial, size_t x_real, size_t dy_real, size_t dx_real, size_t chunk,
+    size_t spatial, const TensorMap mx, const TensorMap md, const TensorMap mo, size_t chunk,
     int chunks_per_seg)
 {
     const size_t seg = blockIdx.x / chunks_per_seg;
@@ -434,9 +459,10 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop2_kernel(
     const T dvar_term = dvar[c] * T(2) / static_cast<T>(num_per_sum - 1);
     const size_t begin = static_cast<size_t>(k) * chunk;
     const size_t end = begin + chunk < spatial ? begin + chunk : spatial;
-    const T* xp = x + seg * x_real;
-    const T* dp = dy + seg * dy_real;
-    T* op = dx + seg * dx_real;
+    const size_t n = seg / num_channels;
+    const T* xp = x + n * mx.stride_n + c * mx.stride_c;
+    const T* dp = dy + n * md.stride_n + c * md.stride_c;
+    T* op = dx + n * mo.stride_n + c * mo.stride_c;
 
     constexpr size_t kStride = static_cast<size_t>(kBlockSize) * VEC;
     constexpr int kUnroll2 = kUnroll / 2;
@@ -448,8 +474,9 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop2_kernel(
 #pragma unroll
         for (int u = 0; u < kUnroll2; ++u)
         {
-            load_vec<T, VEC>(xp + tile + u * kStride + threadIdx.x * VEC, xv[u]);
-            load_vec<T, VEC>(dp + tile + u * kStride + threadIdx.x * VEC, dv[u]);
+            const size_t i = tile + u * kStride + threadIdx.x * VEC;
+            load_vec<T, VEC, !STRIDED>(xp + seg_offset<STRIDED>(mx, i), xv[u]);
+            load_vec<T, VEC, !STRIDED>(dp + seg_offset<STRIDED>(md, i), dv[u]);
         }
 #pragma unroll
         for (int u = 0; u < kUnroll2; ++u)
@@ -460,21 +487,22 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop2_kernel(
                 T r = fma_t(dv[u][j] * sc, inv_stdev, dmean_term);
                 xv[u][j] = fma_t(xv[u][j] - m, dvar_term, r);
             }
-            store_vec<T, VEC>(op + tile + u * kStride + threadIdx.x * VEC, xv[u]);
+            store_vec<T, VEC, !STRIDED>(
+                op + seg_offset<STRIDED>(mo, tile + u * kStride + threadIdx.x * VEC), xv[u]);
         }
     }
     for (size_t i = tile + threadIdx.x * VEC; i < end; i += kStride)
     {
         T xv[VEC], dv[VEC];
-        load_vec<T, VEC>(xp + i, xv);
-        load_vec<T, VEC>(dp + i, dv);
+        load_vec<T, VEC, !STRIDED>(xp + seg_offset<STRIDED>(mx, i), xv);
+        load_vec<T, VEC, !STRIDED>(dp + seg_offset<STRIDED>(md, i), dv);
 #pragma unroll
         for (int j = 0; j < VEC; ++j)
         {
             T r = fma_t(dv[j] * sc, inv_stdev, dmean_term);
             xv[j] = fma_t(xv[j] - m, dvar_term, r);
         }
-        store_vec<T, VEC>(op + i, xv);
+        store_vec<T, VEC, !STRIDED>(op + seg_offset<STRIDED>(mo, i), xv);
     }
 }
 
@@ -486,34 +514,161 @@ constexpr int full_vec()
     return 16 / sizeof(T);
 }
 
-// 16-byte accesses need every segment start and the base on a 16-byte boundary.
-template <typename T>
-bool can_vectorize(const void* p, size_t spatial, size_t real)
-{
-    constexpr size_t v = full_vec<T>();
-    return aligned16(p) && spatial % v == 0 && real % v == 0;
-}
-
 bool grid_ok(size_t blocks)
 {
     return blocks <= 0x7fffffffull;
 }
 
+// One tensor as the kernels see it, plus what decides the vector width.
+struct HostTensor
+{
+    TensorMap map;
+    bool strided = false; // needs index splitting
+    size_t row = 0;       // contiguous interior elements per row (strided) or `spatial` (dense)
+    bool aligned = false; // dense: every segment starts on a 16-byte boundary
+};
+
+// Index splitting that is the identity (x = i, y = z = 0), for a dense tensor
+// that takes part in a launch of the strided kernels: every index is below the
+// divisor 2^31 - 1.
+void set_dense_map(TensorMap* m)
+{
+    m->w = make_fastdiv(0x7fffffffu);
+    m->h = make_fastdiv(1);
+    m->sy = m->sz = 0;
+}
+
 template <typename T>
-int sums_impl(int num_samples, int num_channels, size_t spatial, size_t real, const void* x,
+HostTensor dense_tensor(const void* p, int num_channels, size_t spatial, size_t real)
+{
+    HostTensor t;
+    t.map.stride_c = static_cast<int64_t>(real);
+    t.map.stride_n = static_cast<int64_t>(real) * num_channels;
+    set_dense_map(&t.map);
+    t.row = spatial;
+    t.aligned = aligned16(p) && real % full_vec<T>() == 0;
+    return t;
+}
+
+// A tensor given by local shape and strides (innermost first; channel and
+// sample are the last two dimensions).  Falls back to the dense description
+// when the inner spatial dimensions carry no halo.
+template <typename T>
+int strided_tensor(const h2x_tensor_geometry* g, const void* p, int num_samples, HostTensor* out,
+                   int* num_channels, size_t* spatial)
+{
+    if (!g || g->num_dims < 3 || g->num_dims > 5)
+        return H2X_ERR_INVALID_ARGUMENT;
+    const int nd = g->num_dims, ns = nd - 2;
+    size_t sp = 1;
+    for (int i = 0; i < nd; ++i)
+        if (g->local_shape[i] < 0 || g->strides[i] < 0)
+            return H2X_ERR_INVALID_ARGUMENT;
+    if (g->strides[0] != 1 && g->local_shape[0] > 1)
+        return H2X_ERR_UNSUPPORTED;
+    for (int i = 0; i < ns; ++i)
+        sp *= static_cast<size_t>(g->local_shape[i]);
+    if (g->local_shape[nd - 1] != num_samples && num_samples != 0)
+        return H2X_ERR_INVALID_ARGUMENT;
+    *num_channels = static_cast<int>(g->local_shape[nd - 2]);
+    *spatial = sp;
+    HostTensor t;
+    t.map.stride_c = g->strides[nd - 2];
+    t.map.stride_n = g->strides[nd - 1];
+    // dense inside a segment?  (stride of each spatial dimension = product of the extents below it)
+    bool dense = true;
+    int64_t expect = 1;
+    for (int i = 0; i < ns; ++i)
+    {
+        if (g->local_shape[i] > 1 && g->strides[i] != expect)
+            dense = false;
+        expect *= g->local_shape[i];
+    }
+    if (dense)
+    {
+        set_dense_map(&t.map);
+        t.row = sp;
+        t.aligned = aligned16(p) && t.map.stride_c % full_vec<T>() == 0
+                    && t.map.stride_n % full_vec<T>() == 0;
+    }
+    else
+    {
+        if (sp >= (1ull << 31))
+            return H2X_ERR_TOO_LARGE;
+        t.strided = true;
+        t.row = static_cast<size_t>(g->local_shape[0]);
+        t.map.w = make_fastdiv(static_cast<uint32_t>(g->local_shape[0]));
+        t.map.h = make_fastdiv(ns > 1 ? static_cast<uint32_t>(g->local_shape[1]) : 1u);
+        t.map.sy = ns > 1 ? g->strides[1] : 0;
+        t.map.sz = ns > 2 ? g->strides[2] : 0;
+        t.aligned = false;
+    }
+    *out = t;
+    return H2X_SUCCESS;
+}
+
+// Vector width all tensors of a launch allow, and whether the strided kernels are needed.
+template <typename T>
+int common_vector(std::initializer_list<const HostTensor*> ts, bool* strided)
+{
+    int v = full_vec<T>();
+    *strided = false;
+    for (const HostTensor* t : ts)
+        *strided = *strided || t->strided;
+    for (const HostTensor* t : ts)
+    {
+        // dense tensors in a strided launch are addressed with i itself, so rows do not matter for them
+        const bool ok = t->strided ? t->row % v == 0 : (t->row % v == 0 && (t->aligned || *strided));
+        if (!ok)
+            v = 1;
+    }
+    // unaligned vectors are only generated by the strided kernels
+    if (*strided == false)
+        for (const HostTensor* t : ts)
+            if (!t->aligned)
+                v = 1;
+    return v;
+}
+
+// Launches kernel<T, V, STRIDED> for the width and layout chosen at run time.
+#define H2X_DISPATCH(KERNEL, GRID, ...)                                                            \
+    do                                                                                             \
+    {                                                                                              \
+        if (strided)                                                                               \
+        {                                                                                          \
+            if (vw > 1)                                                                            \
+                KERNEL<T, full_vec<T>(), true><<<GRID, kBlockSize, 0, stream>>>(__VA_ARGS__);      \
+            else                                                                                   \
+                KERNEL<T, 1, true><<<GRID, kBlockSize, 0, stream>>>(__VA_ARGS__);                  \
+        }                                                                                          \
+        else                                                                                       \
+        {                                                                                          \
+            if (vw > 1)                                                                            \
+                KERNEL<T, full_vec<T>(), false><<<GRID, kBlockSize, 0, stream>>>(__VA_ARGS__);     \
+            else                                                                                   \
+                KERNEL<T, 1, false><<<GRID, kBlockSize, 0, stream>>>(__VA_ARGS__);                 \
+        }                                                                                          \
+    } while (0)
+
+template <typename T>
+int zero_outputs(std::initializer_list<void*> outs, int num_channels, hipStream_t stream)
+{
+    const int blocks = (num_channels + kBlockSize - 1) / kBlockSize;
+    for (void* p : outs)
+        fill_kernel<T><<<blocks, kBlockSize, 0, stream>>>(static_cast<T*>(p), num_channels, T(0));
+    return launch_status();
+}
+
+template <typename T>
+int sums_impl(int num_samples, int num_channels, size_t spatial, const HostTensor& tx, const void* x,
               void* sums, void* sqsums, void* workspace, hipStream_t stream)
 {
     if (num_channels == 0)
         return H2X_SUCCESS;
     if (num_samples == 0 || spatial == 0)
-    {
-        const int blocks = (num_channels + kBlockSize - 1) / kBlockSize;
-        fill_kernel<T><<<blocks, kBlockSize, 0, stream>>>(static_cast<T*>(sums), num_channels, T(0));
-        fill_kernel<T><<<blocks, kBlockSize, 0, stream>>>(static_cast<T*>(sqsums), num_channels, T(0));
-        return launch_status();
-    }
-    const bool vec = can_vectorize<T>(x, spatial, real);
-    const int vw = vec ? full_vec<T>() : 1;
+        return zero_outputs<T>({sums, sqsums}, num_channels, stream);
+    bool strided;
+    const int vw = common_vector<T>({&tx}, &strided);
     const int gmax = max_groups_per_channel(num_channels);
     const size_t tile = static_cast<size_t>(kBlockSize) * vw * kUnroll;
     const Chunking ch = make_chunking(spatial, num_samples, gmax, tile, tile);
@@ -523,16 +678,9 @@ int sums_impl(int num_samples, int num_channels, size_t spatial, size_t real, co
     const size_t groups = std::min<size_t>(units, gmax);
     double* partials = static_cast<double*>(workspace);
     const dim3 grid(static_cast<unsigned int>(groups), num_channels);
-    if (vec)
-        bn_sums_kernel<T, full_vec<T>()><<<grid, kBlockSize, 0, stream>>>(
-            static_cast<const T*>(x), static_cast<T*>(sums), static_cast<T*>(sqsums), partials,
-            num_channels, spatial, real, ch.chunk, ch.chunks_per_seg,
-            static_cast<unsigned int>(units), gmax);
-    else
-        bn_sums_kernel<T, 1><<<grid, kBlockSize, 0, stream>>>(
-            static_cast<const T*>(x), static_cast<T*>(sums), static_cast<T*>(sqsums), partials,
-            num_channels, spatial, real, ch.chunk, ch.chunks_per_seg,
-            static_cast<unsigned int>(units), gmax);
+    H2X_DISPATCH(bn_sums_kernel, grid, static_cast<const T*>(x), static_cast<T*>(sums),
+                 static_cast<T*>(sqsums), partials, tx.map, spatial, ch.chunk, ch.chunks_per_seg,
+                 static_cast<unsigned int>(units), gmax);
     if (groups > 1)
         bn_finish_kernel<T, 2><<<num_channels, kBlockSize, 0, stream>>>(
             partials, static_cast<int>(groups), gmax, static_cast<T*>(sums),
@@ -553,63 +701,50 @@ int statistics_impl(int num_channels, size_t num_per_sum, double decay, void* me
     return launch_status();
 }
 
-// Chunking of an elementwise pass over N*C segments.
-template <typename T>
+// Chunking of an elementwise pass over N*C segments: at least one full vector
+// per thread, about kElementwiseBlocks workgroups.
 Chunking elementwise_chunking(size_t spatial, size_t segments, int vw, int unroll)
 {
     const size_t tile = static_cast<size_t>(kBlockSize) * vw * unroll;
     const size_t one_pass = static_cast<size_t>(kBlockSize) * vw;
-    // aim at >= 4096 workgroups, but at least one full vector per thread
     return make_chunking(spatial, segments, kElementwiseBlocks, one_pass,
                          one_pass * 2 > tile ? one_pass : one_pass * 2);
 }
 
 template <typename T>
-int apply_impl(int num_samples, int num_channels, size_t spatial, size_t x_real, size_t y_real,
-               const void* x, const void* mean, const void* var, const void* scale,
-               const void* bias, void* y, double epsilon, hipStream_t stream)
+int apply_impl(int num_samples, int num_channels, size_t spatial, const HostTensor& tx,
+               const HostTensor& ty, const void* x, const void* mean, const void* var,
+               const void* scale, const void* bias, void* y, double epsilon, hipStream_t stream)
 {
     const size_t segments = static_cast<size_t>(num_samples) * num_channels;
     if (segments == 0 || spatial == 0)
         return H2X_SUCCESS;
-    const bool vec = can_vectorize<T>(x, spatial, x_real) && can_vectorize<T>(y, spatial, y_real);
-    const int vw = vec ? full_vec<T>() : 1;
-    const Chunking ch = elementwise_chunking<T>(spatial, segments, vw, kUnroll);
+    bool strided;
+    const int vw = common_vector<T>({&tx, &ty}, &strided);
+    const Chunking ch = elementwise_chunking(spatial, segments, vw, kUnroll);
     const size_t blocks = segments * ch.chunks_per_seg;
     if (!grid_ok(blocks))
         return H2X_ERR_TOO_LARGE;
     const unsigned int grid = static_cast<unsigned int>(blocks);
-#define H2X_LAUNCH(V)                                                                              \
-    bn_apply_kernel<T, V><<<grid, kBlockSize, 0, stream>>>(                                        \
-        static_cast<const T*>(x), static_cast<const T*>(mean), static_cast<const T*>(var),         \
-        static_cast<const T*>(scale), static_cast<const T*>(bias), static_cast<T*>(y),             \
-        static_cast<T>(epsilon), num_channels, spatial, x_real, y_real, ch.chunk,                  \
-        ch.chunks_per_seg)
-    if (vec)
-        H2X_LAUNCH(full_vec<T>());
-    else
-        H2X_LAUNCH(1);
-#undef H2X_LAUNCH
+    H2X_DISPATCH(bn_apply_kernel, grid, static_cast<const T*>(x), static_cast<const T*>(mean),
+                 static_cast<const T*>(var), static_cast<const T*>(scale),
+                 static_cast<const T*>(bias), static_cast<T*>(y), static_cast<T>(epsilon),
+                 num_channels, spatial, tx.map, ty.map, ch.chunk, ch.chunks_per_seg);
     return launch_status();
 }
 
 template <typename T>
-int backprop1_impl(int num_samples, int num_channels, size_t spatial, size_t x_real,
-                   size_t dy_real, const void* x, const void* dy, const void* mean,
+int backprop1_impl(int num_samples, int num_channels, size_t spatial, const HostTensor& tx,
+                   const HostTensor& td, const void* x, const void* dy, const void* mean,
                    const void* var, const void* scale, void* dscale, void* dbias, void* dmean,
                    void* dvar, double epsilon, void* workspace, hipStream_t stream)
 {
     if (num_channels == 0)
         return H2X_SUCCESS;
     if (num_samples == 0 || spatial == 0)
-    {
-        const int blocks = (num_channels + kBlockSize - 1) / kBlockSize;
-        for (void* p : {dscale, dbias, dmean, dvar})
-            fill_kernel<T><<<blocks, kBlockSize, 0, stream>>>(static_cast<T*>(p), num_channels, T(0));
-        return launch_status();
-    }
-    const bool vec = can_vectorize<T>(x, spatial, x_real) && can_vectorize<T>(dy, spatial, dy_real);
-    const int vw = vec ? full_vec<T>() : 1;
+        return zero_outputs<T>({dscale, dbias, dmean, dvar}, num_channels, stream);
+    bool strided;
+    const int vw = common_vector<T>({&tx, &td}, &strided);
     const int gmax = max_groups_per_channel(num_channels);
     const size_t tile = static_cast<size_t>(kBlockSize) * vw * (kUnroll / 2);
     const Chunking ch = make_chunking(spatial, num_samples, gmax, tile, tile);
@@ -619,18 +754,12 @@ int backprop1_impl(int num_samples, int num_channels, size_t spatial, size_t x_r
     const size_t groups = std::min<size_t>(units, gmax);
     double* partials = static_cast<double*>(workspace);
     const dim3 grid(static_cast<unsigned int>(groups), num_channels);
-#define H2X_LAUNCH(V)                                                                              \
-    bn_backprop1_kernel<T, V><<<grid, kBlockSize, 0, stream>>>(                                    \
-        static_cast<const T*>(x), static_cast<const T*>(dy), static_cast<const T*>(mean),          \
-        static_cast<const T*>(var), static_cast<const T*>(scale), static_cast<T*>(dscale),         \
-        static_cast<T*>(dbias), static_cast<T*>(dmean), static_cast<T*>(dvar),                     \
-        static_cast<T>(epsilon), partials, num_channels, spatial, x_real, dy_real, ch.chunk,       \
-        ch.chunks_per_seg, static_cast<unsigned int>(units), gmax)
-    if (vec)
-        H2X_LAUNCH(full_vec<T>());
-    else
-        H2X_LAUNCH(1);
-#undef H2X_LAUNCH
+    H2X_DISPATCH(bn_backprop1_kernel, grid, static_cast<const T*>(x), static_cast<const T*>(dy),
+                 static_cast<const T*>(mean), static_cast<const T*>(var),
+                 static_cast<const T*>(scale), static_cast<T*>(dscale), static_cast<T*>(dbias),
+                 static_cast<T*>(dmean), static_cast<T*>(dvar), static_cast<T>(epsilon), partials,
+                 spatial, tx.map, td.map, ch.chunk, ch.chunks_per_seg,
+                 static_cast<unsigned int>(units), gmax);
     if (groups > 1)
         bn_finish_kernel<T, 4><<<num_channels, kBlockSize, 0, stream>>>(
             partials, static_cast<int>(groups), gmax, static_cast<T*>(dscale),
@@ -639,8 +768,8 @@ int backprop1_impl(int num_samples, int num_channels, size_t spatial, size_t x_r
 }
 
 template <typename T>
-int backprop2_impl(int num_samples, int num_channels, size_t spatial, size_t x_real,
-                   size_t dy_real, size_t dx_real, size_t num_per_sum, const void* x,
+int backprop2_impl(int num_samples, int num_channels, size_t spatial, size_t num_per_sum,
+                   const HostTensor& tx, const HostTensor& td, const HostTensor& to, const void* x,
                    const void* dy, const void* mean, const void* var, const void* scale,
                    const void* dmean, const void* dvar, void* dx, double epsilon,
                    hipStream_t stream)
@@ -648,25 +777,19 @@ int backprop2_impl(int num_samples, int num_channels, size_t spatial, size_t x_r
     const size_t segments = static_cast<size_t>(num_samples) * num_channels;
     if (segments == 0 || spatial == 0)
         return H2X_SUCCESS;
-    const bool vec = can_vectorize<T>(x, spatial, x_real) && can_vectorize<T>(dy, spatial, dy_real)
-                     && can_vectorize<T>(dx, spatial, dx_real);
-    const int vw = vec ? full_vec<T>() : 1;
-    const Chunking ch = elementwise_chunking<T>(spatial, segments, vw, kUnroll / 2);
+    bool strided;
+    const int vw = common_vector<T>({&tx, &td, &to}, &strided);
+    const Chunking ch = elementwise_chunking(spatial, segments, vw, kUnroll / 2);
     const size_t blocks = segments * ch.chunks_per_seg;
     if (!grid_ok(blocks))
         return H2X_ERR_TOO_LARGE;
     const unsigned int grid = static_cast<unsigned int>(blocks);
-#define H2X_LAUNCH(V)                                                                              \
-    bn_backprop2_kernel<T, V><<<grid, kBlockSize, 0, stream>>>(                                    \
-        static_cast<const T*>(x), static_cast<const T*>(dy), static_cast<const T*>(mean),          \
-        static_cast<const T*>(var), static_cast<const T*>(scale), static_cast<const T*>(dmean),    \
-        static_cast<const T*>(dvar), static_cast<T*>(dx), static_cast<T>(epsilon), num_per_sum,    \
-        num_channels, spatial, x_real, dy_real, dx_real, ch.chunk, ch.chunks_per_seg)
-    if (vec)
-        H2X_LAUNCH(full_vec<T>());
-    else
-        H2X_LAUNCH(1);
-#undef H2X_LAUNCH
+    H2X_DISPATCH(bn_backprop2_kernel, grid, static_cast<const T*>(x), static_cast<const T*>(dy),
+                 static_cast<const T*>(mean), static_cast<const T*>(var),
+                 static_cast<const T*>(scale), static_cast<const T*>(dmean),
+                 static_cast<const T*>(dvar), static_cast<T*>(dx), static_cast<T>(epsilon),
+                 num_per_sum, num_channels, spatial, tx.map, td.map, to.map, ch.chunk,
+                 ch.chunks_per_seg);
     return launch_status();
 }
 
@@ -675,10 +798,94 @@ bool bad_geometry(int num_samples, int num_channels, size_t spatial, size_t real
     return num_samples < 0 || num_channels < 0 || real < spatial;
 }
 
+// ---- typed bodies of the C entry points ----------------------------------------
+
+template <typename T>
+int sums_dense(int n, int c, size_t s, size_t sr, const void* x, void* sums, void* sqsums, void* ws,
+               hipStream_t st)
+{
+    return sums_impl<T>(n, c, s, dense_tensor<T>(x, c, s, sr), x, sums, sqsums, ws, st);
+}
+
+template <typename T>
+int sums_strided(int n, const h2x_tensor_geometry* g, const void* x, void* sums, void* sqsums,
+                 void* ws, hipStream_t st)
+{
+    HostTensor tx;
+    int c;
+    size_t s;
+    const int err = strided_tensor<T>(g, x, n, &tx, &c, &s);
+    return err ? err : sums_impl<T>(n, c, s, tx, x, sums, sqsums, ws, st);
+}
+
+template <typename T>
+int apply_strided(int n, const h2x_tensor_geometry* gx, const h2x_tensor_geometry* gy, const void* x,
+                  const void* mean, const void* var, const void* scale, const void* bias, void* y,
+                  double eps, hipStream_t st)
+{
+    HostTensor tx, ty;
+    int c, c2;
+    size_t s, s2;
+    int err = strided_tensor<T>(gx, x, n, &tx, &c, &s);
+    if (!err)
+        err = strided_tensor<T>(gy, y, n, &ty, &c2, &s2);
+    if (!err && (c != c2 || s != s2))
+        err = H2X_ERR_INVALID_ARGUMENT;
+    return err ? err : apply_impl<T>(n, c, s, tx, ty, x, mean, var, scale, bias, y, eps, st);
+}
+
+template <typename T>
+int backprop1_strided(int n, const h2x_tensor_geometry* gx, const h2x_tensor_geometry* gd,
+                      const void* x, const void* dy, const void* mean, const void* var,
+                      const void* scale, void* dscale, void* dbias, void* dmean, void* dvar,
+                      double eps, void* ws, hipStream_t st)
+{
+    HostTensor tx, td;
+    int c, c2;
+    size_t s, s2;
+    int err = strided_tensor<T>(gx, x, n, &tx, &c, &s);
+    if (!err)
+        err = strided_tensor<T>(gd, dy, n, &td, &c2, &s2);
+    if (!err && (c != c2 || s != s2))
+        err = H2X_ERR_INVALID_ARGUMENT;
+    return err ? err
+               : backprop1_impl<T>(n, c, s, tx, td, x, dy, mean, var, scale, dscale, dbias, dmean,
+                                   dvar, eps, ws, st);
+}
+
+template <typename T>
+int backprop2_strided(int n, size_t num_per_sum, const h2x_tensor_geometry* gx,
+                      const h2x_tensor_geometry* gd, const h2x_tensor_geometry* go, const void* x,
+                      const void* dy, const void* mean, const void* var, const void* scale,
+                      const void* dmean, const void* dvar, void* dx, double eps, hipStream_t st)
+{
+    HostTensor tx, td, to;
+    int c, c2, c3;
+    size_t s, s2, s3;
+    int err = strided_tensor<T>(gx, x, n, &tx, &c, &s);
+    if (!err)
+        err = strided_tensor<T>(gd, dy, n, &td, &c2, &s2);
+    if (!err)
+        err = strided_tensor<T>(go, dx, n, &to, &c3, &s3);
+    if (!err && (c != c2 || s != s2 || c != c3 || s != s3))
+        err = H2X_ERR_INVALID_ARGUMENT;
+    return err ? err
+               : backprop2_impl<T>(n, c, s, num_per_sum, tx, td, to, x, dy, mean, var, scale, dmean,
+                                   dvar, dx, eps, st);
+}
+
 } // namespace
 } // namespace h2x
 
 using namespace h2x;
+
+#define H2X_BY_DTYPE(dtype, CALL_F32, CALL_F64)                                                    \
+    switch (dtype)                                                                                 \
+    {                                                                                              \
+    case H2X_F32: return CALL_F32;                                                                 \
+    case H2X_F64: return CALL_F64;                                                                 \
+    }                                                                                              \
+    return H2X_ERR_UNSUPPORTED
 
 extern "C" size_t h2x_bn_workspace_bytes(int num_channels)
 {
@@ -695,16 +902,25 @@ extern "C" int h2x_bn_channel_sums_and_sqsums(h2x_dtype dtype, int num_samples, 
     if (bad_geometry(num_samples, num_channels, spatial_size, spatial_real_size) || !sums || !sqsums
         || !workspace || (!x && num_samples > 0 && spatial_size > 0 && num_channels > 0))
         return H2X_ERR_INVALID_ARGUMENT;
-    switch (dtype)
-    {
-    case H2X_F32:
-        return sums_impl<float>(num_samples, num_channels, spatial_size, spatial_real_size, x, sums,
-                                sqsums, workspace, as_stream(stream));
-    case H2X_F64:
-        return sums_impl<double>(num_samples, num_channels, spatial_size, spatial_real_size, x,
-                                 sums, sqsums, workspace, as_stream(stream));
-    }
-    return H2X_ERR_UNSUPPORTED;
+    H2X_BY_DTYPE(dtype,
+                 sums_dense<float>(num_samples, num_channels, spatial_size, spatial_real_size, x, sums,
+                                   sqsums, workspace, as_stream(stream)),
+                 sums_dense<double>(num_samples, num_channels, spatial_size, spatial_real_size, x,
+                                    sums, sqsums, workspace, as_stream(stream)));
+}
+
+extern "C" int h2x_bn_channel_sums_and_sqsums_strided(h2x_dtype dtype, int num_samples,
+                                                      const h2x_tensor_geometry* x_geometry,
+                                                      const void* x, void* sums, void* sqsums,
+                                                      void* workspace, h2x_stream_t stream)
+{
+    if (num_samples < 0 || !x_geometry || !sums || !sqsums || !workspace)
+        return H2X_ERR_INVALID_ARGUMENT;
+    H2X_BY_DTYPE(dtype,
+                 sums_strided<float>(num_samples, x_geometry, x, sums, sqsums, workspace,
+                                     as_stream(stream)),
+                 sums_strided<double>(num_samples, x_geometry, x, sums, sqsums, workspace,
+                                      as_stream(stream)));
 }
 
 extern "C" int h2x_bn_sums_to_statistics(h2x_dtype dtype, int num_channels, size_t num_per_sum,
@@ -714,16 +930,11 @@ extern "C" int h2x_bn_sums_to_statistics(h2x_dtype dtype, int num_channels, size
 {
     if (num_channels < 0 || !mean_inout || !var_inout || !running_mean || !running_var)
         return H2X_ERR_INVALID_ARGUMENT;
-    switch (dtype)
-    {
-    case H2X_F32:
-        return statistics_impl<float>(num_channels, num_per_sum, decay, mean_inout, var_inout,
-                                      running_mean, running_var, as_stream(stream));
-    case H2X_F64:
-        return statistics_impl<double>(num_channels, num_per_sum, decay, mean_inout, var_inout,
-                                       running_mean, running_var, as_stream(stream));
-    }
-    return H2X_ERR_UNSUPPORTED;
+    H2X_BY_DTYPE(dtype,
+                 statistics_impl<float>(num_channels, num_per_sum, decay, mean_inout, var_inout,
+                                        running_mean, running_var, as_stream(stream)),
+                 statistics_impl<double>(num_channels, num_per_sum, decay, mean_inout, var_inout,
+                                         running_mean, running_var, as_stream(stream)));
 }
 
 extern "C" int h2x_bn_batch_normalization(h2x_dtype dtype, int num_samples, int num_channels,
@@ -738,18 +949,31 @@ extern "C" int h2x_bn_batch_normalization(h2x_dtype dtype, int num_samples, int 
         return H2X_ERR_INVALID_ARGUMENT;
     if ((!x || !y) && static_cast<size_t>(num_samples) * num_channels * spatial_size > 0)
         return H2X_ERR_INVALID_ARGUMENT;
-    switch (dtype)
-    {
-    case H2X_F32:
-        return apply_impl<float>(num_samples, num_channels, spatial_size, x_spatial_real_size,
-                                 y_spatial_real_size, x, mean, var, scale, bias, y, epsilon,
-                                 as_stream(stream));
-    case H2X_F64:
-        return apply_impl<double>(num_samples, num_channels, spatial_size, x_spatial_real_size,
-                                  y_spatial_real_size, x, mean, var, scale, bias, y, epsilon,
-                                  as_stream(stream));
-    }
-    return H2X_ERR_UNSUPPORTED;
+    const int n = num_samples, c = num_channels;
+    const size_t s = spatial_size;
+    H2X_BY_DTYPE(dtype,
+                 apply_impl<float>(n, c, s, dense_tensor<float>(x, c, s, x_spatial_real_size),
+                                   dense_tensor<float>(y, c, s, y_spatial_real_size), x, mean, var,
+                                   scale, bias, y, epsilon, as_stream(stream)),
+                 apply_impl<double>(n, c, s, dense_tensor<double>(x, c, s, x_spatial_real_size),
+                                    dense_tensor<double>(y, c, s, y_spatial_real_size), x, mean, var,
+                                    scale, bias, y, epsilon, as_stream(stream)));
+}
+
+extern "C" int h2x_bn_batch_normalization_strided(h2x_dtype dtype, int num_samples,
+                                                  const h2x_tensor_geometry* x_geometry,
+                                                  const h2x_tensor_geometry* y_geometry,
+                                                  const void* x, const void* mean, const void* var,
+                                                  const void* scale, const void* bias, void* y,
+                                                  double epsilon, h2x_stream_t stream)
+{
+    if (num_samples < 0 || !x_geometry || !y_geometry || !mean || !var || !scale || !bias)
+        return H2X_ERR_INVALID_ARGUMENT;
+    H2X_BY_DTYPE(dtype,
+                 apply_strided<float>(num_samples, x_geometry, y_geometry, x, mean, var, scale, bias,
+                                      y, epsilon, as_stream(stream)),
+                 apply_strided<double>(num_samples, x_geometry, y_geometry, x, mean, var, scale,
+                                       bias, y, epsilon, as_stream(stream)));
 }
 
 extern "C" int h2x_bn_backprop1(h2x_dtype dtype, int num_samples, int num_channels,
@@ -765,18 +989,37 @@ extern "C" int h2x_bn_backprop1(h2x_dtype dtype, int num_samples, int num_channe
         return H2X_ERR_INVALID_ARGUMENT;
     if ((!x || !dy) && static_cast<size_t>(num_samples) * num_channels * spatial_size > 0)
         return H2X_ERR_INVALID_ARGUMENT;
-    switch (dtype)
-    {
-    case H2X_F32:
-        return backprop1_impl<float>(num_samples, num_channels, spatial_size, x_spatial_real_size,
-                                     dy_spatial_real_size, x, dy, mean, var, scale, dscale, dbias,
-                                     dmean, dvar, epsilon, workspace, as_stream(stream));
-    case H2X_F64:
-        return backprop1_impl<double>(num_samples, num_channels, spatial_size, x_spatial_real_size,
-                                      dy_spatial_real_size, x, dy, mean, var, scale, dscale, dbias,
-                                      dmean, dvar, epsilon, workspace, as_stream(stream));
-    }
-    return H2X_ERR_UNSUPPORTED;
+    const int n = num_samples, c = num_channels;
+    const size_t s = spatial_size;
+    H2X_BY_DTYPE(dtype,
+                 backprop1_impl<float>(n, c, s, dense_tensor<float>(x, c, s, x_spatial_real_size),
+                                       dense_tensor<float>(dy, c, s, dy_spatial_real_size), x, dy,
+                                       mean, var, scale, dscale, dbias, dmean, dvar, epsilon,
+                                       workspace, as_stream(stream)),
+                 backprop1_impl<double>(n, c, s, dense_tensor<double>(x, c, s, x_spatial_real_size),
+                                        dense_tensor<double>(dy, c, s, dy_spatial_real_size), x, dy,
+                                        mean, var, scale, dscale, dbias, dmean, dvar, epsilon,
+                                        workspace, as_stream(stream)));
+}
+
+extern "C" int h2x_bn_backprop1_strided(h2x_dtype dtype, int num_samples,
+                                        const h2x_tensor_geometry* x_geometry,
+                                        const h2x_tensor_geometry* dy_geometry, const void* x,
+                                        const void* dy, const void* mean, const void* var,
+                                        const void* scale, void* dscale, void* dbias, void* dmean,
+                                        void* dvar, double epsilon, void* workspace,
+                                        h2x_stream_t stream)
+{
+    if (num_samples < 0 || !x_geometry || !dy_geometry || !mean || !var || !scale || !dscale
+        || !dbias || !dmean || !dvar || !workspace)
+        return H2X_ERR_INVALID_ARGUMENT;
+    H2X_BY_DTYPE(dtype,
+                 backprop1_strided<float>(num_samples, x_geometry, dy_geometry, x, dy, mean, var,
+                                          scale, dscale, dbias, dmean, dvar, epsilon, workspace,
+                                          as_stream(stream)),
+                 backprop1_strided<double>(num_samples, x_geometry, dy_geometry, x, dy, mean, var,
+                                           scale, dscale, dbias, dmean, dvar, epsilon, workspace,
+                                           as_stream(stream)));
 }
 
 extern "C" int h2x_bn_backprop2(h2x_dtype dtype, int num_samples, int num_channels,
@@ -793,17 +1036,38 @@ extern "C" int h2x_bn_backprop2(h2x_dtype dtype, int num_samples, int num_channe
         return H2X_ERR_INVALID_ARGUMENT;
     if ((!x || !dy || !dx) && static_cast<size_t>(num_samples) * num_channels * spatial_size > 0)
         return H2X_ERR_INVALID_ARGUMENT;
-    switch (dtype)
-    {
-    case H2X_F32:
-        return backprop2_impl<float>(num_samples, num_channels, spatial_size, x_spatial_real_size,
-                                     dy_spatial_real_size, dx_spatial_real_size, num_per_sum, x, dy,
-                                     mean, var, scale, dmean, dvar, dx, epsilon, as_stream(stream));
-    case H2X_F64:
-        return backprop2_impl<double>(num_samples, num_channels, spatial_size, x_spatial_real_size,
-                                      dy_spatial_real_size, dx_spatial_real_size, num_per_sum, x,
-                                      dy, mean, var, scale, dmean, dvar, dx, epsilon,
-                                      as_stream(stream));
-    }
-    return H2X_ERR_UNSUPPORTED;
+    const int n = num_samples, c = num_channels;
+    const size_t s = spatial_size;
+    H2X_BY_DTYPE(dtype,
+                 backprop2_impl<float>(n, c, s, num_per_sum,
+                                       dense_tensor<float>(x, c, s, x_spatial_real_size),
+                                       dense_tensor<float>(dy, c, s, dy_spatial_real_size),
+                                       dense_tensor<float>(dx, c, s, dx_spatial_real_size), x, dy,
+                                       mean, var, scale, dmean, dvar, dx, epsilon, as_stream(stream)),
+                 backprop2_impl<double>(n, c, s, num_per_sum,
+                                        dense_tensor<double>(x, c, s, x_spatial_real_size),
+                                        dense_tensor<double>(dy, c, s, dy_spatial_real_size),
+                                        dense_tensor<double>(dx, c, s, dx_spatial_real_size), x, dy,
+                                        mean, var, scale, dmean, dvar, dx, epsilon,
+                                        as_stream(stream)));
+}
+
+extern "C" int h2x_bn_backprop2_strided(h2x_dtype dtype, int num_samples, size_t num_per_sum,
+                                        const h2x_tensor_geometry* x_geometry,
+                                        const h2x_tensor_geometry* dy_geometry,
+                                        const h2x_tensor_geometry* dx_geometry, const void* x,
+                                        const void* dy, const void* mean, const void* var,
+                                        const void* scale, const void* dmean, const void* dvar,
+                                        void* dx, double epsilon, h2x_stream_t stream)
+{
+    if (num_samples < 0 || !x_geometry || !dy_geometry || !dx_geometry || !mean || !var || !scale
+        || !dmean || !dvar)
+        return H2X_ERR_INVALID_ARGUMENT;
+    H2X_BY_DTYPE(dtype,
+                 backprop2_strided<float>(num_samples, num_per_sum, x_geometry, dy_geometry,
+                                          dx_geometry, x, dy, mean, var, scale, dmean, dvar, dx,
+                                          epsilon, as_stream(stream)),
+                 backprop2_strided<double>(num_samples, num_per_sum, x_geometry, dy_geometry,
+                                           dx_geometry, x, dy, mean, var, scale, dmean, dvar, dx,
+                                           epsilon, as_stream(stream)));
 }

@@ -32,6 +32,41 @@ inline bool aligned16(const void* p)
     return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
 }
 
+// ---- division by a launch-time constant ------------------------------------
+// n / d for n < 2^31 by multiply-high and shift.
+struct FastDiv
+{
+    uint32_t divisor;
+    uint32_t multiplier;
+    uint32_t shift;
+};
+
+inline FastDiv make_fastdiv(uint32_t d)
+{
+    FastDiv f{d, 0u, 0u};
+    if (d > 1)
+    {
+        uint32_t log2 = 0;
+        while ((1ull << log2) < d)
+            ++log2;
+        const uint32_t p = 31 + log2;
+        f.multiplier = static_cast<uint32_t>(((1ull << p) + d - 1) / d);
+        f.shift = p - 32;
+    }
+    return f;
+}
+
+__host__ __device__ inline uint32_t fastdiv(uint32_t n, const FastDiv& f)
+{
+#ifdef __HIP_DEVICE_COMPILE__
+    return f.divisor == 1 ? n : __umulhi(n, f.multiplier) >> f.shift;
+#else
+    return f.divisor == 1
+               ? n
+               : static_cast<uint32_t>((static_cast<uint64_t>(n) * f.multiplier) >> 32) >> f.shift;
+#endif
+}
+
 #ifdef __HIPCC__
 
 // ---- lane permutes --------------------------------------------------------

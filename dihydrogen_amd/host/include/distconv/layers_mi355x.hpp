@@ -27,9 +27,18 @@ private:
 namespace batchnorm
 {
 
-// (num_samples, num_channels, spatial, spatial_real) of a tensor the
-// optimised layout covers: no halo in the inner spatial dimensions
-// (legacy/src/dnn_backend/batchnorm.cu:210-219).
+// True when the inner spatial dimensions carry no halo: the layout of the
+// reference's optimised kernels (legacy/src/dnn_backend/batchnorm.cu:210-219).
+template <typename Tensor>
+bool is_dense(const Tensor& t)
+{
+    for (int i = 0; i < t.get_num_dims() - 3; ++i)
+        if (t.get_halo_width(i) != 0)
+            return false;
+    return true;
+}
+
+// (num_channels, spatial, spatial_real) of a dense tensor.
 template <typename Tensor>
 struct ChannelGeometry
 {
@@ -38,8 +47,6 @@ struct ChannelGeometry
     explicit ChannelGeometry(const Tensor& t)
     {
         const int nd = t.get_num_dims();
-        for (int i = 0; i < nd - 3; ++i)
-            assert_always(t.get_halo_width(i) == 0);
         assert_always(t.get_halo_width(nd - 2) == 0 && t.get_halo_width(nd - 1) == 0);
         num_channels = static_cast<int>(t.get_local_shape()[-2]);
         spatial = spatial_real = 1;
@@ -50,6 +57,25 @@ struct ChannelGeometry
         }
     }
 };
+
+// Local shape + strides for the strided entry points (tensors with a halo on
+// an inner spatial dimension: the reference's generic kernels).
+template <typename Tensor>
+h2x_tensor_geometry tensor_geometry(const Tensor& t, int num_samples)
+{
+    const int nd = t.get_num_dims();
+    assert_always(t.get_halo_width(nd - 2) == 0 && t.get_halo_width(nd - 1) == 0);
+    h2x_tensor_geometry g = {};
+    g.num_dims = nd;
+    const auto strides = t.get_strides();
+    for (int i = 0; i < nd; ++i)
+    {
+        g.local_shape[i] = static_cast<int64_t>(t.get_local_shape()[i]);
+        g.strides[i] = static_cast<int64_t>(strides[i]);
+    }
+    g.local_shape[nd - 1] = num_samples;
+    return g;
+}
 
 // Workspace of fp64 partial sums, owned by the caller (one per layer object).
 class Workspace
@@ -86,10 +112,21 @@ void channel_sums_and_sqsums(int num_dims, int num_samples, const Tensor& input,
     // a rank that is not a split root, or holds nothing, only zeroes the sums
     // (batchnorm.cu:201-208)
     const bool active = input.get_local_size() > 0 && input.is_split_root();
-    DISTCONV_CHECK_H2X(h2x_bn_channel_sums_and_sqsums(
-        Tensor::h2x_type(), active ? num_samples : 0, g.num_channels, g.spatial, g.spatial_real,
-        input.get_const_base_ptr(), sums.get_base_ptr(), sqsums.get_base_ptr(),
-        ws.get(g.num_channels), stream));
+    const int ns = active ? num_samples : 0;
+    if (is_dense(input))
+    {
+        DISTCONV_CHECK_H2X(h2x_bn_channel_sums_and_sqsums(
+            Tensor::h2x_type(), ns, g.num_channels, g.spatial, g.spatial_real,
+            input.get_const_base_ptr(), sums.get_base_ptr(), sqsums.get_base_ptr(),
+            ws.get(g.num_channels), stream));
+    }
+    else // batchnorm.cu:232-248
+    {
+        const h2x_tensor_geometry gx = tensor_geometry(input, ns);
+        DISTCONV_CHECK_H2X(h2x_bn_channel_sums_and_sqsums_strided(
+            Tensor::h2x_type(), ns, &gx, input.get_const_base_ptr(), sums.get_base_ptr(),
+            sqsums.get_base_ptr(), ws.get(g.num_channels), stream));
+    }
 }
 
 template <typename Tensor>
@@ -122,11 +159,23 @@ void batch_normalization(int num_dims, int num_samples, const Tensor& input, con
     if (input.get_local_size() == 0)
         return;
     const ChannelGeometry<Tensor> gi(input), go(output);
-    DISTCONV_CHECK_H2X(h2x_bn_batch_normalization(
-        Tensor::h2x_type(), num_samples, gi.num_channels, gi.spatial, gi.spatial_real,
-        go.spatial_real, input.get_const_base_ptr(), mean.get_const_base_ptr(),
-        var.get_const_base_ptr(), scale.get_const_base_ptr(), bias.get_const_base_ptr(),
-        output.get_base_ptr(), epsilon, stream));
+    if (is_dense(input) && is_dense(output))
+    {
+        DISTCONV_CHECK_H2X(h2x_bn_batch_normalization(
+            Tensor::h2x_type(), num_samples, gi.num_channels, gi.spatial, gi.spatial_real,
+            go.spatial_real, input.get_const_base_ptr(), mean.get_const_base_ptr(),
+            var.get_const_base_ptr(), scale.get_const_base_ptr(), bias.get_const_base_ptr(),
+            output.get_base_ptr(), epsilon, stream));
+    }
+    else
+    {
+        const h2x_tensor_geometry gx = tensor_geometry(input, num_samples),
+                                  gy = tensor_geometry(output, num_samples);
+        DISTCONV_CHECK_H2X(h2x_bn_batch_normalization_strided(
+            Tensor::h2x_type(), num_samples, &gx, &gy, input.get_const_base_ptr(),
+            mean.get_const_base_ptr(), var.get_const_base_ptr(), scale.get_const_base_ptr(),
+            bias.get_const_base_ptr(), output.get_base_ptr(), epsilon, stream));
+    }
 }
 
 // batchnorm.hpp:68-81
@@ -139,12 +188,26 @@ void backprop1(int num_dims, int num_samples, const Tensor& input, const Tensor&
     assert_always(num_dims == 4 || num_dims == 5);
     const ChannelGeometry<Tensor> gi(input), go(d_output);
     const bool active = input.get_local_size() > 0 && input.is_split_root();
-    DISTCONV_CHECK_H2X(h2x_bn_backprop1(
-        Tensor::h2x_type(), active ? num_samples : 0, gi.num_channels, gi.spatial, gi.spatial_real,
-        go.spatial_real, input.get_const_base_ptr(), d_output.get_const_base_ptr(),
-        mean.get_const_base_ptr(), var.get_const_base_ptr(), scale.get_const_base_ptr(),
-        scale_gradient.get_base_ptr(), bias_gradient.get_base_ptr(), mean_gradient.get_base_ptr(),
-        var_gradient.get_base_ptr(), epsilon, ws.get(gi.num_channels), stream));
+    const int ns = active ? num_samples : 0;
+    if (is_dense(input) && is_dense(d_output))
+    {
+        DISTCONV_CHECK_H2X(h2x_bn_backprop1(
+            Tensor::h2x_type(), ns, gi.num_channels, gi.spatial, gi.spatial_real, go.spatial_real,
+            input.get_const_base_ptr(), d_output.get_const_base_ptr(), mean.get_const_base_ptr(),
+            var.get_const_base_ptr(), scale.get_const_base_ptr(), scale_gradient.get_base_ptr(),
+            bias_gradient.get_base_ptr(), mean_gradient.get_base_ptr(),
+            var_gradient.get_base_ptr(), epsilon, ws.get(gi.num_channels), stream));
+    }
+    else
+    {
+        const h2x_tensor_geometry gx = tensor_geometry(input, ns), gd = tensor_geometry(d_output, ns);
+        DISTCONV_CHECK_H2X(h2x_bn_backprop1_strided(
+            Tensor::h2x_type(), ns, &gx, &gd, input.get_const_base_ptr(),
+            d_output.get_const_base_ptr(), mean.get_const_base_ptr(), var.get_const_base_ptr(),
+            scale.get_const_base_ptr(), scale_gradient.get_base_ptr(), bias_gradient.get_base_ptr(),
+            mean_gradient.get_base_ptr(), var_gradient.get_base_ptr(), epsilon,
+            ws.get(gi.num_channels), stream));
+    }
 }
 
 template <typename Tensor>
@@ -169,12 +232,27 @@ void backprop2(int num_dims, index_t num_samples, index_t num_per_sum, const Ten
     if (input.get_local_size() == 0)
         return;
     const ChannelGeometry<Tensor> gi(input), go(d_output), gd(d_input);
-    DISTCONV_CHECK_H2X(h2x_bn_backprop2(
-        Tensor::h2x_type(), static_cast<int>(num_samples), gi.num_channels, gi.spatial,
-        gi.spatial_real, go.spatial_real, gd.spatial_real, num_per_sum,
-        input.get_const_base_ptr(), d_output.get_const_base_ptr(), mean.get_const_base_ptr(),
-        var.get_const_base_ptr(), scale.get_const_base_ptr(), mean_gradient.get_const_base_ptr(),
-        var_gradient.get_const_base_ptr(), d_input.get_base_ptr(), epsilon, stream));
+    const int ns = static_cast<int>(num_samples);
+    // the fast path needs halo-free tensors, as in the reference (batchnorm.cu:1503-1506)
+    if (is_dense(input) && is_dense(d_output) && is_dense(d_input))
+    {
+        DISTCONV_CHECK_H2X(h2x_bn_backprop2(
+            Tensor::h2x_type(), ns, gi.num_channels, gi.spatial, gi.spatial_real, go.spatial_real,
+            gd.spatial_real, num_per_sum, input.get_const_base_ptr(),
+            d_output.get_const_base_ptr(), mean.get_const_base_ptr(), var.get_const_base_ptr(),
+            scale.get_const_base_ptr(), mean_gradient.get_const_base_ptr(),
+            var_gradient.get_const_base_ptr(), d_input.get_base_ptr(), epsilon, stream));
+    }
+    else
+    {
+        const h2x_tensor_geometry gx = tensor_geometry(input, ns), gy = tensor_geometry(d_output, ns),
+                                  gz = tensor_geometry(d_input, ns);
+        DISTCONV_CHECK_H2X(h2x_bn_backprop2_strided(
+            Tensor::h2x_type(), ns, num_per_sum, &gx, &gy, &gz, input.get_const_base_ptr(),
+            d_output.get_const_base_ptr(), mean.get_const_base_ptr(), var.get_const_base_ptr(),
+            scale.get_const_base_ptr(), mean_gradient.get_const_base_ptr(),
+            var_gradient.get_const_base_ptr(), d_input.get_base_ptr(), epsilon, stream));
+    }
 }
 
 } // namespace batchnorm

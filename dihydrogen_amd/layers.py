@@ -29,18 +29,35 @@ def _ptr(t) -> ctypes.c_void_p:
     return ctypes.c_void_p(int(t))
 
 
-def _channel_geometry(t: Tensor):
-    """(num_samples, num_channels, spatial, spatial_real) of a local tensor whose
-    inner spatial dimensions carry no halo -- the layout the batch-norm entry
-    points take (legacy/src/dnn_backend/batchnorm.cu:134-190,210-230)."""
+def _is_dense(t: Tensor) -> bool:
+    """No halo on the inner spatial dimensions: the layout the dense entry points
+    take (legacy/src/dnn_backend/batchnorm.cu:210-219)."""
     nd = t.get_num_dims()
-    for d in range(nd - 3):
-        if t.overlap[d] != 0:
-            raise NotImplementedError("halo on an inner spatial dimension is not supported")
+    return all(t.overlap[d] == 0 for d in range(nd - 3))
+
+
+def _channel_geometry(t: Tensor):
+    """(num_samples, num_channels, spatial, spatial_real) of a dense local tensor."""
+    nd = t.get_num_dims()
     if t.overlap[nd - 2] != 0 or t.overlap[nd - 1] != 0:
         raise NotImplementedError("halo on the channel or sample dimension is not supported")
     n, c = t.local_shape[nd - 1], t.local_shape[nd - 2]
     return n, c, _prod(t.local_shape[: nd - 2]), _prod(t.local_real_shape[: nd - 2])
+
+
+def _tensor_geometry(t: Tensor, num_samples: int) -> capi.TensorGeometry:
+    """h2x_tensor_geometry of a local tensor (local shape + get_strides())."""
+    nd = t.get_num_dims()
+    if t.overlap[nd - 2] != 0 or t.overlap[nd - 1] != 0:
+        raise NotImplementedError("halo on the channel or sample dimension is not supported")
+    g = capi.TensorGeometry()
+    g.num_dims = nd
+    strides = t.get_strides()
+    for i in range(nd):
+        g.local_shape[i] = t.local_shape[i]
+        g.strides[i] = strides[i]
+    g.local_shape[nd - 1] = num_samples
+    return g
 
 
 class BatchNormalization:
@@ -90,10 +107,17 @@ class BatchNormalization:
             return 0
         n, c, s, sr = _channel_geometry(input)
         active = input.is_split_root() and input.get_local_size() > 0
-        capi.check(self._lib.h2x_bn_channel_sums_and_sqsums(
-            input.h2x_dtype, self.num_current_samples if active else 0, c, s, sr,
-            _ptr(input.get_base_ptr()), _ptr(mean), _ptr(var), _ptr(self._ws(c)),
-            _stream_handle(self.stream)), "channel_sums_and_sqsums")
+        ns = self.num_current_samples if active else 0
+        if _is_dense(input):
+            capi.check(self._lib.h2x_bn_channel_sums_and_sqsums(
+                input.h2x_dtype, ns, c, s, sr, _ptr(input.get_base_ptr()), _ptr(mean), _ptr(var),
+                _ptr(self._ws(c)), _stream_handle(self.stream)), "channel_sums_and_sqsums")
+        else:  # halo on an inner spatial dimension: the generic path of batchnorm.cu:232-248
+            g = _tensor_geometry(input, ns)
+            capi.check(self._lib.h2x_bn_channel_sums_and_sqsums_strided(
+                input.h2x_dtype, ns, ctypes.byref(g), _ptr(input.get_base_ptr()), _ptr(mean),
+                _ptr(var), _ptr(self._ws(c)), _stream_handle(self.stream)),
+                "channel_sums_and_sqsums (strided)")
         return 0
 
     def forward_allreduce(self, mean: torch.Tensor, var: torch.Tensor, is_training: bool = True) -> int:
@@ -112,10 +136,18 @@ class BatchNormalization:
         """batchnorm.hpp:505-517."""
         n, c, s, sr = _channel_geometry(input)
         _, _, so, sro = _channel_geometry(output)
-        capi.check(self._lib.h2x_bn_batch_normalization(
-            input.h2x_dtype, self.num_current_samples, c, s, sr, sro, _ptr(input.get_base_ptr()),
-            _ptr(mean), _ptr(var), _ptr(scale), _ptr(bias), _ptr(output.get_base_ptr()), self.epsilon,
-            _stream_handle(self.stream)), "batch_normalization")
+        ns = self.num_current_samples
+        if _is_dense(input) and _is_dense(output):
+            capi.check(self._lib.h2x_bn_batch_normalization(
+                input.h2x_dtype, ns, c, s, sr, sro, _ptr(input.get_base_ptr()), _ptr(mean), _ptr(var),
+                _ptr(scale), _ptr(bias), _ptr(output.get_base_ptr()), self.epsilon,
+                _stream_handle(self.stream)), "batch_normalization")
+        else:
+            gx, gy = _tensor_geometry(input, ns), _tensor_geometry(output, ns)
+            capi.check(self._lib.h2x_bn_batch_normalization_strided(
+                input.h2x_dtype, ns, ctypes.byref(gx), ctypes.byref(gy), _ptr(input.get_base_ptr()),
+                _ptr(mean), _ptr(var), _ptr(scale), _ptr(bias), _ptr(output.get_base_ptr()),
+                self.epsilon, _stream_handle(self.stream)), "batch_normalization (strided)")
 
     def forward_stage2(self, input: Tensor, mean, var, running_mean, running_var, scale, bias,
                        output: Tensor, is_training: bool = True) -> int:
@@ -141,12 +173,19 @@ class BatchNormalization:
         n, c, s, sr = _channel_geometry(input)
         _, _, _, sro = _channel_geometry(d_output)
         active = input.is_split_root() and input.get_local_size() > 0
-        capi.check(self._lib.h2x_bn_backprop1(
-            input.h2x_dtype, self.num_current_samples if active else 0, c, s, sr, sro,
-            _ptr(input.get_base_ptr()), _ptr(d_output.get_base_ptr()), _ptr(mean), _ptr(var),
-            _ptr(scale), _ptr(scale_gradient), _ptr(bias_gradient), _ptr(mean_gradient),
-            _ptr(var_gradient), self.epsilon, _ptr(self._ws(c)), _stream_handle(self.stream)),
-            "backprop1")
+        ns = self.num_current_samples if active else 0
+        tail = (_ptr(mean), _ptr(var), _ptr(scale), _ptr(scale_gradient), _ptr(bias_gradient),
+                _ptr(mean_gradient), _ptr(var_gradient), self.epsilon, _ptr(self._ws(c)),
+                _stream_handle(self.stream))
+        if _is_dense(input) and _is_dense(d_output):
+            capi.check(self._lib.h2x_bn_backprop1(
+                input.h2x_dtype, ns, c, s, sr, sro, _ptr(input.get_base_ptr()),
+                _ptr(d_output.get_base_ptr()), *tail), "backprop1")
+        else:
+            gx, gd = _tensor_geometry(input, ns), _tensor_geometry(d_output, ns)
+            capi.check(self._lib.h2x_bn_backprop1_strided(
+                input.h2x_dtype, ns, ctypes.byref(gx), ctypes.byref(gd), _ptr(input.get_base_ptr()),
+                _ptr(d_output.get_base_ptr()), *tail), "backprop1 (strided)")
         return 0
 
     def backward_allreduce(self, scale_gradient, bias_gradient, mean_gradient, var_gradient,
@@ -164,11 +203,19 @@ class BatchNormalization:
         n, c, s, sr = _channel_geometry(input)
         _, _, _, sro = _channel_geometry(d_output)
         _, _, _, sri = _channel_geometry(d_input)
-        capi.check(self._lib.h2x_bn_backprop2(
-            input.h2x_dtype, self.num_current_samples, c, s, sr, sro, sri, self._num_per_sum(input),
-            _ptr(input.get_base_ptr()), _ptr(d_output.get_base_ptr()), _ptr(mean), _ptr(var),
-            _ptr(scale), _ptr(mean_gradient), _ptr(var_gradient), _ptr(d_input.get_base_ptr()),
-            self.epsilon, _stream_handle(self.stream)), "backprop2")
+        ns = self.num_current_samples
+        tail = (_ptr(input.get_base_ptr()), _ptr(d_output.get_base_ptr()), _ptr(mean), _ptr(var),
+                _ptr(scale), _ptr(mean_gradient), _ptr(var_gradient), _ptr(d_input.get_base_ptr()),
+                self.epsilon, _stream_handle(self.stream))
+        # the reference takes its fast path only for halo-free tensors (batchnorm.cu:1503-1506)
+        if _is_dense(input) and _is_dense(d_output) and _is_dense(d_input):
+            capi.check(self._lib.h2x_bn_backprop2(
+                input.h2x_dtype, ns, c, s, sr, sro, sri, self._num_per_sum(input), *tail), "backprop2")
+        else:
+            gx, gd, gi = (_tensor_geometry(t, ns) for t in (input, d_output, d_input))
+            capi.check(self._lib.h2x_bn_backprop2_strided(
+                input.h2x_dtype, ns, self._num_per_sum(input), ctypes.byref(gx), ctypes.byref(gd),
+                ctypes.byref(gi), *tail), "backprop2 (strided)")
         return 0
 
     def backward(self, input, d_output, mean, var, scale, scale_gradient, bias_gradient,

@@ -206,6 +206,86 @@ int h2x_bn_backprop2(h2x_dtype dtype,
                      double epsilon,
                      h2x_stream_t stream);
 
+/**
+ * Local part of a tensor given by shape and strides, for tensors that carry a
+ * halo on an inner spatial dimension.  Innermost first; the last two
+ * dimensions are channel and sample; num_dims is 3, 4 or 5.  strides are in
+ * elements of the real (haloed) allocation (Tensor::get_strides(),
+ * legacy/include/distconv/tensor/tensor.hpp:291-298) and strides[0] must be 1;
+ * the data pointer that goes with it is the tensor's get_base_ptr().
+ */
+typedef struct h2x_tensor_geometry
+{
+    int32_t num_dims;
+    int32_t reserved;
+    int64_t local_shape[H2X_MAX_DIMS];
+    int64_t strides[H2X_MAX_DIMS];
+} h2x_tensor_geometry;
+
+/**
+ * The four tensor passes for arbitrarily haloed tensors: what the reference's
+ * generic kernels cover (legacy/src/dnn_backend/batchnorm.cu:39-90, 369-418,
+ * 899-980, 1303-1369, chosen by its drivers at :210-248, 514-573, 1168-1230,
+ * 1503-1559).  Same results as the dense entry points on the same elements;
+ * a geometry that is dense inside its segments is forwarded to them.
+ * local_shape[num_dims - 1] must equal num_samples.
+ */
+int h2x_bn_channel_sums_and_sqsums_strided(h2x_dtype dtype,
+                                           int num_samples,
+                                           const h2x_tensor_geometry* x_geometry,
+                                           const void* x,
+                                           void* sums,
+                                           void* sqsums,
+                                           void* workspace,
+                                           h2x_stream_t stream);
+
+int h2x_bn_batch_normalization_strided(h2x_dtype dtype,
+                                       int num_samples,
+                                       const h2x_tensor_geometry* x_geometry,
+                                       const h2x_tensor_geometry* y_geometry,
+                                       const void* x,
+                                       const void* mean,
+                                       const void* var,
+                                       const void* scale,
+                                       const void* bias,
+                                       void* y,
+                                       double epsilon,
+                                       h2x_stream_t stream);
+
+int h2x_bn_backprop1_strided(h2x_dtype dtype,
+                             int num_samples,
+                             const h2x_tensor_geometry* x_geometry,
+                             const h2x_tensor_geometry* dy_geometry,
+                             const void* x,
+                             const void* dy,
+                             const void* mean,
+                             const void* var,
+                             const void* scale,
+                             void* dscale,
+                             void* dbias,
+                             void* dmean,
+                             void* dvar,
+                             double epsilon,
+                             void* workspace,
+                             h2x_stream_t stream);
+
+int h2x_bn_backprop2_strided(h2x_dtype dtype,
+                             int num_samples,
+                             size_t num_per_sum,
+                             const h2x_tensor_geometry* x_geometry,
+                             const h2x_tensor_geometry* dy_geometry,
+                             const h2x_tensor_geometry* dx_geometry,
+                             const void* x,
+                             const void* dy,
+                             const void* mean,
+                             const void* var,
+                             const void* scale,
+                             const void* dmean,
+                             const void* dvar,
+                             void* dx,
+                             double epsilon,
+                             h2x_stream_t stream);
+
 /* ------------------------------------------------------------------------ */
 /* Channel softmax: dense [num_samples][num_channels][spatial_size] tensors,  */
 /* softmax taken over the channel dimension.                                  */

@@ -55,6 +55,10 @@ def _ptr(a: np.ndarray):
     return ctypes.c_void_p(a.ctypes.data)
 
 
+def _i64(seq):
+    return (ctypes.c_int64 * len(seq))(*[int(v) for v in seq])
+
+
 def _scalar(dtype, v):
     return ctypes.c_float(v) if np.dtype(dtype) == np.float32 else ctypes.c_double(v)
 
@@ -144,6 +148,45 @@ def bn_backward(x, dy, mean, var, scale, eps=1e-5):
     return dx, dscale, dbias, dmean, dvar
 
 
+# -- strided variants: `x` is the flat real buffer starting at the first interior
+#    element, shape/strides innermost first (channel = nd-2, sample = nd-1)
+
+def _geom(shape, *strides_list):
+    nd = len(shape)
+    return [ctypes.c_int(nd), _i64(shape)] + [_i64(st) for st in strides_list]
+
+
+def bn_channel_sums_and_sqsums_strided(x, shape, strides):
+    c = int(shape[-2])
+    sums, sqsums = np.empty(c, x.dtype), np.empty(c, x.dtype)
+    fn = getattr(lib(), "orc_bn_channel_sums_and_sqsums_strided_" + _sfx(x.dtype))
+    fn(*_geom(shape, strides), _ptr(x), _ptr(sums), _ptr(sqsums))
+    return sums, sqsums
+
+
+def bn_batch_normalization_strided(x, shape, x_strides, y, y_strides, mean, var, scale, bias, eps):
+    fn = getattr(lib(), "orc_bn_batch_normalization_strided_" + _sfx(x.dtype))
+    fn(*_geom(shape, x_strides, y_strides), _ptr(x), _ptr(mean), _ptr(var), _ptr(scale), _ptr(bias),
+       _ptr(y), _scalar(x.dtype, eps))
+
+
+def bn_backprop1_strided(x, shape, x_strides, dy, dy_strides, mean, var, scale, eps):
+    c = int(shape[-2])
+    outs = [np.empty(c, x.dtype) for _ in range(4)]
+    fn = getattr(lib(), "orc_bn_backprop1_strided_" + _sfx(x.dtype))
+    fn(*_geom(shape, x_strides, dy_strides), _ptr(x), _ptr(dy), _ptr(mean), _ptr(var), _ptr(scale),
+       _ptr(outs[0]), _ptr(outs[1]), _ptr(outs[2]), _ptr(outs[3]), _scalar(x.dtype, eps))
+    return tuple(outs)
+
+
+def bn_backprop2_strided(x, shape, x_strides, dy, dy_strides, dx, dx_strides, num_per_sum, mean, var,
+                         scale, dmean, dvar, eps):
+    fn = getattr(lib(), "orc_bn_backprop2_strided_" + _sfx(x.dtype))
+    fn(*_geom(shape, x_strides, dy_strides, dx_strides), ctypes.c_size_t(num_per_sum), _ptr(x),
+       _ptr(dy), _ptr(mean), _ptr(var), _ptr(scale), _ptr(dmean), _ptr(dvar), _ptr(dx),
+       _scalar(x.dtype, eps))
+
+
 # --------------------------------------------------------------------------
 # Channel softmax
 # --------------------------------------------------------------------------
@@ -203,10 +246,6 @@ def halo_pack_or_unpack(tensor: np.ndarray, dim: int, side: int, width: int, buf
 # --------------------------------------------------------------------------
 # Shuffler pack / unpack
 # --------------------------------------------------------------------------
-
-def _i64(seq):
-    return (ctypes.c_int64 * len(seq))(*[int(v) for v in seq])
-
 
 def _i32arr(a):
     a = np.ascontiguousarray(a, dtype=np.int32)

@@ -133,9 +133,82 @@ static int test_softmax(const Shape& shape)
     return (max_rel(hy, oy) > 1e-5) + (max_rel(to_host(dx), odx) > 1e-5);
 }
 
+// A spatially decomposed tensor with halos on the inner spatial dimensions must
+// give, rank by rank, what a halo-free tensor with the same interior gives
+// (generic vs optimised kernels, the reference's own validation idea:
+// legacy/tests/dnn_backend/test_cudnn_util.sh.in:339-410).
+static int test_bn_haloed()
+{
+    const Shape shape({16, 12, 6, 2});
+    const Shape locale({2, 2, 1, 1});
+    const Distribution dh = Distribution::make_overlapped_distribution(locale, IntVector({1, 2, 0, 0}));
+    const Distribution dp = Distribution::make_distribution(locale);
+    Shape pshape({1, 1, 6, 1});
+    const Distribution dl = Distribution::make_localized_distribution(4);
+    int errors = 0;
+    for (int r = 0; r < 4; ++r)
+    {
+        const LocaleVirtual loc(r, 4), one(0, 1);
+        DevTensor<float> xh(shape, loc, dh), yh(shape, loc, dh), dyh(shape, loc, dp), dxh(shape, loc, dh);
+        DevTensor<float> xp(shape, loc, dp), yp(shape, loc, dp), dxp(shape, loc, dp);
+        std::vector<DevTensor<float>> pv;
+        for (int i = 0; i < 20; ++i)
+        {
+            pv.emplace_back(pshape, one, dl);
+            pv.back().allocate();
+        }
+        for (auto* t : {&xh, &yh, &dyh, &dxh, &xp, &yp, &dxp})
+            t->allocate();
+        // same interior in the haloed and the plain tensor
+        const auto vals = randn(xp.get_local_size(), 100 + r), dvals = randn(xp.get_local_size(), 200 + r);
+        std::vector<float> hx(xh.get_local_real_size(), NAN);
+        const Shape& ls = xh.get_local_shape();
+        for (index_t o = 0; o < xh.get_local_size(); ++o)
+            hx[xh.get_local_offset(ls.get_index(o))] = vals[o];
+        to_device(xh, hx);
+        to_device(xp, vals);
+        to_device(dyh, dvals);
+        to_device(pv[4], randn(6, 3, 0.25f, 1.0f)); // scale
+        to_device(pv[5], randn(6, 4, 0.1f));         // bias
+        to_device(pv[14], to_host(pv[4]));
+        to_device(pv[15], to_host(pv[5]));
+        to_device(pv[3], std::vector<float>(6, 1.0f));
+        to_device(pv[13], std::vector<float>(6, 1.0f));
+        BackendMI355X backend;
+        BatchNormalization<BackendMI355X, float> bh(backend, 4, 0.9f, 1e-5f, false), bp(backend, 4, 0.9f, 1e-5f, false);
+        bh.forward(xh, pv[0], pv[1], pv[2], pv[3], pv[4], pv[5], yh, true);
+        bh.backward(xh, dyh, pv[0], pv[1], pv[4], pv[6], pv[7], pv[8], pv[9], dxh);
+        bp.forward(xp, pv[10], pv[11], pv[12], pv[13], pv[14], pv[15], yp, true);
+        bp.backward(xp, dyh, pv[10], pv[11], pv[14], pv[16], pv[17], pv[18], pv[19], dxp);
+        // the two paths add the same fp64 terms in different orders: equal to rounding
+        for (int k : {0, 1, 2, 3, 6, 7, 8, 9})
+            errors += max_rel(to_host(pv[k]), to_host(pv[k + 10])) > 1e-6;
+        const auto hy = to_host(yh), py = to_host(yp), hdx = to_host(dxh), pdx = to_host(dxp);
+        std::vector<float> iy(py.size()), idx(py.size());
+        for (index_t o = 0; o < xh.get_local_size(); ++o)
+        {
+            const index_t off = xh.get_local_offset(ls.get_index(o));
+            iy[o] = hy[off];
+            idx[o] = hdx[off];
+        }
+        errors += max_rel(iy, py) > 1e-5;
+        errors += max_rel(idx, pdx) > 1e-5;
+        // halo cells of the outputs keep the allocator's zeros
+        double halo_sum = 0;
+        for (float v : hy)
+            halo_sum += std::fabs(v);
+        double inner_sum = 0;
+        for (float v : iy)
+            inner_sum += std::fabs(v);
+        errors += std::fabs(halo_sum - inner_sum) > 1e-3 * inner_sum;
+    }
+    return errors;
+}
+
 int main()
 {
     int errors = 0;
+    errors += test_bn_haloed();
     errors += test_bn(Shape({56, 56, 64, 8}));   // BASELINE config 1
     errors += test_bn(Shape({5, 7, 3, 2}));
     errors += test_bn(Shape({16, 16, 16, 8, 4})); // 5-D

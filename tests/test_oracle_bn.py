@@ -228,3 +228,56 @@ def test_float64_variant():
     ax = _axes(x)
     assert max_rel(mean, x.mean(axis=ax)) < 1e-12
     assert max_rel(var, x.var(axis=ax, ddof=1)) < 1e-12
+
+
+def _haloed(shape_np, halo_np, seed, dtype=np.float32):
+    """A real (haloed) array with random interior and NaN halo; returns the real
+    array, the interior view, innermost-first local shape and strides."""
+    rng = np.random.default_rng(seed)
+    real_np = tuple(s + 2 * h for s, h in zip(shape_np, halo_np))
+    real = np.full(real_np, np.nan, dtype)
+    inner = tuple(slice(h, h + s) for s, h in zip(shape_np, halo_np))
+    real[inner] = rng.standard_normal(shape_np).astype(dtype)
+    strides, s = [], 1
+    for e in real_np[::-1]:
+        strides.append(s)
+        s *= e
+    base = sum(h * st for h, st in zip(halo_np[::-1], strides))
+    return real, inner, list(shape_np[::-1]), strides, base
+
+
+@pytest.mark.parametrize("shape,halo", [((2, 3, 6, 8), (0, 0, 1, 2)), ((2, 3, 4, 5, 6), (0, 0, 1, 0, 2)),
+                                        ((1, 2, 3, 4, 5), (0, 0, 2, 1, 1))])
+def test_strided_equals_dense_on_the_interior(shape, halo):
+    """The strided (generic-kernel) functions on a haloed tensor give exactly the
+    dense functions' results on a contiguous copy of its interior."""
+    x_real, inner, lshape, xs, xb = _haloed(shape, halo, 71)
+    d_real, _, _, ds, db = _haloed(shape, tuple(h + 1 if h else 0 for h in halo), 72)
+    d_inner = tuple(slice(h + 1 if h else 0, (h + 1 if h else 0) + s) for s, h in zip(shape, halo))
+    x, dy = np.ascontiguousarray(x_real[inner]), np.ascontiguousarray(d_real[d_inner])
+    c = shape[1]
+    rng = np.random.default_rng(73)
+    scale = rng.uniform(0.5, 1.5, c).astype(np.float32)
+    bias = rng.standard_normal(c).astype(np.float32)
+    xf, df = x_real.reshape(-1)[xb:], d_real.reshape(-1)[db:]
+    s1, q1 = oracle.bn_channel_sums_and_sqsums_strided(xf, lshape, xs)
+    s0, q0 = oracle.bn_channel_sums_and_sqsums(x)
+    assert np.array_equal(s0, s1) and np.array_equal(q0, q1)
+    n = x.size // c
+    rm, rv = np.zeros(c, np.float32), np.ones(c, np.float32)
+    oracle.bn_sums_to_statistics(n, 0.9, s0, q0, rm, rv)
+    mean, var = s0, q0
+    y0 = oracle.bn_batch_normalization(x, mean, var, scale, bias, EPS)
+    y_real = np.full_like(x_real, np.nan)
+    oracle.bn_batch_normalization_strided(xf, lshape, xs, y_real.reshape(-1)[xb:], xs, mean, var, scale, bias, EPS)
+    assert np.array_equal(y_real[inner], y0)
+    assert np.isnan(y_real).sum() == y_real.size - x.size          # halo cells untouched
+    g0 = oracle.bn_backprop1(x, dy, mean, var, scale, EPS)
+    g1 = oracle.bn_backprop1_strided(xf, lshape, xs, df, ds, mean, var, scale, EPS)
+    for a, b in zip(g0, g1):
+        assert np.array_equal(a, b)
+    dx0 = oracle.bn_backprop2(x, dy, mean, var, scale, g0[2], g0[3], EPS, n)
+    dx_real = np.full_like(x_real, np.nan)
+    oracle.bn_backprop2_strided(xf, lshape, xs, df, ds, dx_real.reshape(-1)[xb:], xs, n, mean, var, scale,
+                                g0[2], g0[3], EPS)
+    assert np.array_equal(dx_real[inner], dx0)
