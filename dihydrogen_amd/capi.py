@@ -99,6 +99,15 @@ SIGNATURES = {
                                             c_void_p]),
     "h2x_softmax_channel_backward": (c_int, [c_int, c_int, c_int, c_size_t, c_void_p, c_void_p,
                                              c_void_p, c_void_p]),
+    "h2x_softmax_instance_workspace_bytes": (c_size_t, [c_int]),
+    "h2x_softmax_instance_max": (c_int, [c_int, c_int, c_size_t, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "h2x_softmax_instance_exp": (c_int, [c_int, c_int, c_size_t, c_void_p, c_void_p, c_void_p, c_void_p,
+                                         c_void_p, c_void_p]),
+    "h2x_softmax_instance_normalize": (c_int, [c_int, c_int, c_size_t, c_void_p, c_void_p, c_void_p]),
+    "h2x_softmax_instance_dot": (c_int, [c_int, c_int, c_size_t, c_void_p, c_void_p, c_void_p, c_void_p,
+                                         c_void_p]),
+    "h2x_softmax_instance_gradient": (c_int, [c_int, c_int, c_size_t, c_void_p, c_void_p, c_void_p,
+                                              c_void_p, c_void_p]),
     "h2x_halo_size": (c_size_t, [c_int, POINTER(c_int64), c_int, c_int]),
     "h2x_halo_pack_or_unpack": (c_int, [c_int, c_void_p, c_int, POINTER(c_int64), c_int, c_int,
                                         c_int, c_void_p, c_int, c_int, c_int, c_void_p]),

@@ -12,6 +12,7 @@
 #include "h2x_device.hpp"
 
 #include <cfloat>
+#include <cmath>
 
 namespace h2x
 {
@@ -394,6 +395,266 @@ int backward_impl(int n, int c, size_t s, const void* yv, const void* dyv, void*
     return launch_status();
 }
 
+// ---- instance mode -----------------------------------------------------------
+// Softmax over all elements of a sample (legacy/src/dnn_backend/softmax.cu:179-536,
+// 705-784): per-sample maximum, exp(x - max) with per-sample sum, y / sum clamped
+// to sqrt(min_normal); backward: per-sample dot product, then the gradient.  The
+// reference finishes its per-sample reductions with atomics; here every
+// workgroup stores a partial (fp64 for sums) and a second small kernel combines
+// them in index order.  A sample is a contiguous block of `sample_size`
+// elements (dense tensor), so every pass is a plain 16-byte stream.
+
+constexpr int kInstUnroll = 4;
+constexpr int kInstTargetGroups = 4096;
+constexpr int kInstMaxGroupsPerSample = 2048;
+
+int inst_groups_per_sample_max(int num_samples)
+{
+    const int g = (kInstTargetGroups + num_samples - 1) / (num_samples > 0 ? num_samples : 1);
+    return g < 8 ? 8 : (g > kInstMaxGroupsPerSample ? kInstMaxGroupsPerSample : g);
+}
+
+template <typename T>
+__device__ __forceinline__ T wave_max(T v)
+{
+#pragma unroll
+    for (int d = 1; d < kWaveSize; d *= 2)
+    {
+        const T o = __shfl_xor(v, d, kWaveSize);
+        v = o > v ? o : v;
+    }
+    return v;
+}
+
+enum InstReduce : int
+{
+    kInstMax = 0,   // max x                       -> T partial
+    kInstExpSum = 1, // y = exp(x - max); sum y     -> double partial
+    kInstDot = 2     // sum y * dy                  -> double partial
+};
+
+// One pass over the chunk [begin, end) of sample n.  a: x (max, exp) or y (dot);
+// b: dy (dot); out: y (exp).  Partials are stored as doubles in all modes.
+template <typename T, int VEC, int MODE>
+__global__ __launch_bounds__(kBlockSize) void softmax_inst_reduce_kernel(
+    const T* __restrict__ a, const T* __restrict__ b, T* __restrict__ out,
+    const T* __restrict__ sample_param, double* partials, size_t sample_size, size_t chunk,
+    int groups_max)
+{
+    using P = Pack<T, VEC>;
+    __shared__ double lds[kWavesPerBlock];
+    const int n = blockIdx.y;
+    const size_t begin = static_cast<size_t>(blockIdx.x) * chunk;
+    const size_t end = begin + chunk < sample_size ? begin + chunk : sample_size;
+    const T* ap = a + static_cast<size_t>(n) * sample_size;
+    const T* bp = MODE == kInstDot ? b + static_cast<size_t>(n) * sample_size : nullptr;
+    T* op = MODE == kInstExpSum ? out + static_cast<size_t>(n) * sample_size : nullptr;
+    const T shift = MODE == kInstExpSum ? sample_param[n] : T(0);
+    constexpr size_t kStride = static_cast<size_t>(kBlockSize) * VEC;
+
+    T mx = Limits<T>::min_normal; // softmax.cu:88-99: the maximum starts at min_normal
+    double acc = 0.0;
+    for (size_t i = begin + threadIdx.x * VEC; i < end; i += kStride * kInstUnroll)
+    {
+        P va[kInstUnroll], vb[kInstUnroll];
+#pragma unroll
+        for (int u = 0; u < kInstUnroll; ++u)
+            if (i + u * kStride < end)
+            {
+                va[u] = P::load(ap + i + u * kStride);
+                if constexpr (MODE == kInstDot)
+                    vb[u] = P::load(bp + i + u * kStride);
+            }
+#pragma unroll
+        for (int u = 0; u < kInstUnroll; ++u)
+            if (i + u * kStride < end)
+            {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+                {
+                    if constexpr (MODE == kInstMax)
+                    {
+                        mx = va[u][j] >= mx ? va[u][j] : mx;
+                    }
+                    else if constexpr (MODE == kInstExpSum)
+                    {
+                        const T e = exp_t(va[u][j] - shift);
+                        va[u][j] = e;
+                        acc += static_cast<double>(e);
+                    }
+                    else
+                    {
+                        acc = __builtin_fma(static_cast<double>(va[u][j]),
+                                            static_cast<double>(vb[u][j]), acc);
+                    }
+                }
+                if constexpr (MODE == kInstExpSum)
+                    P::store(op + i + u * kStride, va[u]);
+            }
+    }
+    double part;
+    if constexpr (MODE == kInstMax)
+    {
+        mx = wave_max(mx);
+        if ((threadIdx.x & (kWaveSize - 1)) == 0)
+            lds[threadIdx.x / kWaveSize] = static_cast<double>(mx);
+        __syncthreads();
+        part = lds[0];
+#pragma unroll
+        for (int w = 1; w < kWavesPerBlock; ++w)
+            part = lds[w] > part ? lds[w] : part;
+    }
+    else
+    {
+        double v[1] = {acc};
+        block_sum<1>(v, lds);
+        part = v[0];
+    }
+    if (threadIdx.x == 0)
+        partials[static_cast<size_t>(n) * groups_max + blockIdx.x] = part;
+}
+
+// Combines the partials of every sample in index order.
+template <typename T, bool IS_MAX>
+__global__ __launch_bounds__(kBlockSize) void softmax_inst_finish_kernel(
+    const double* __restrict__ partials, int groups, int groups_max, T* __restrict__ out)
+{
+    __shared__ double lds[kWavesPerBlock];
+    const int n = blockIdx.x;
+    const double* mine = partials + static_cast<size_t>(n) * groups_max;
+    if constexpr (IS_MAX)
+    {
+        double m = static_cast<double>(Limits<T>::min_normal);
+        for (int g = threadIdx.x; g < groups; g += kBlockSize)
+            m = mine[g] > m ? mine[g] : m;
+        m = wave_max(m);
+        if ((threadIdx.x & (kWaveSize - 1)) == 0)
+            lds[threadIdx.x / kWaveSize] = m;
+        __syncthreads();
+        if (threadIdx.x == 0)
+        {
+            double r = lds[0];
+            for (int w = 1; w < kWavesPerBlock; ++w)
+                r = lds[w] > r ? lds[w] : r;
+            out[n] = static_cast<T>(r);
+        }
+    }
+    else
+    {
+        double t[1] = {0.0};
+        for (int g = threadIdx.x; g < groups; g += kBlockSize)
+            t[0] += mine[g];
+        block_sum<1>(t, lds);
+        if (threadIdx.x == 0)
+            out[n] = static_cast<T>(t[0]);
+    }
+}
+
+// y = max(y / sum, sqrt(min_normal))  (SoftmaxOp, softmax.cu:424-435) or
+// dx = y > sqrt(min_normal) ? y * (dy - dp) : 0  (bp_compute_func, :483-500)
+template <typename T, int VEC, bool BACKWARD>
+__global__ __launch_bounds__(kBlockSize) void softmax_inst_map_kernel(
+    const T* y_in, const T* __restrict__ dy, const T* __restrict__ sample_param, T* out,
+    size_t sample_size, T min_output)
+{
+    using P = Pack<T, VEC>;
+    const int n = blockIdx.y;
+    const size_t i = (static_cast<size_t>(blockIdx.x) * kBlockSize + threadIdx.x) * VEC;
+    if (i >= sample_size)
+        return;
+    const size_t off = static_cast<size_t>(n) * sample_size + i;
+    const T p = sample_param[n];
+    P v = P::load(y_in + off);
+    if constexpr (BACKWARD)
+    {
+        const P g = P::load(dy + off);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j)
+            v[j] = v[j] > min_output ? v[j] * (g[j] - p) : T(0);
+    }
+    else
+    {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j)
+        {
+            const T r = v[j] / p;
+            v[j] = r > min_output ? r : min_output;
+        }
+    }
+    P::store(out + off, v);
+}
+
+template <typename T>
+T inst_min_output()
+{
+    return static_cast<T>(std::sqrt(static_cast<double>(Limits<T>::min_normal))); // softmax.cu:156-160
+}
+
+struct InstChunking
+{
+    size_t chunk;
+    int groups;
+};
+
+InstChunking inst_chunking(size_t sample_size, int num_samples, int vec)
+{
+    const int gmax = inst_groups_per_sample_max(num_samples);
+    const size_t tile = static_cast<size_t>(kBlockSize) * vec * kInstUnroll;
+    size_t chunk = (sample_size + gmax - 1) / gmax;
+    chunk = (chunk + tile - 1) / tile * tile;
+    InstChunking c;
+    c.chunk = chunk;
+    c.groups = static_cast<int>((sample_size + chunk - 1) / chunk);
+    return c;
+}
+
+template <typename T, int MODE>
+int inst_reduce(int n, size_t sample_size, const void* a, const void* b, void* out,
+                const void* param, void* result, void* workspace, hipStream_t st)
+{
+    constexpr int kFull = 16 / sizeof(T);
+    const int v = vector_width<T>(sample_size, kFull, {a, b ? b : a, out ? out : a});
+    const InstChunking ch = inst_chunking(sample_size, n, v);
+    const int gmax = inst_groups_per_sample_max(n);
+    const dim3 grid(ch.groups, n);
+    double* partials = static_cast<double*>(workspace);
+    if (v == kFull)
+        softmax_inst_reduce_kernel<T, kFull, MODE><<<grid, kBlockSize, 0, st>>>(
+            static_cast<const T*>(a), static_cast<const T*>(b), static_cast<T*>(out),
+            static_cast<const T*>(param), partials, sample_size, ch.chunk, gmax);
+    else
+        softmax_inst_reduce_kernel<T, 1, MODE><<<grid, kBlockSize, 0, st>>>(
+            static_cast<const T*>(a), static_cast<const T*>(b), static_cast<T*>(out),
+            static_cast<const T*>(param), partials, sample_size, ch.chunk, gmax);
+    softmax_inst_finish_kernel<T, MODE == kInstMax><<<n, kBlockSize, 0, st>>>(
+        partials, ch.groups, gmax, static_cast<T*>(result));
+    return launch_status();
+}
+
+template <typename T, bool BACKWARD>
+int inst_map(int n, size_t sample_size, const void* y, const void* dy, const void* param, void* out,
+             hipStream_t st)
+{
+    constexpr int kFull = 16 / sizeof(T);
+    const int v = vector_width<T>(sample_size, kFull, {y, dy ? dy : y, out});
+    const T min_output = inst_min_output<T>();
+    if (v == kFull)
+        softmax_inst_map_kernel<T, kFull, BACKWARD><<<pixel_grid(sample_size, kFull, n), kBlockSize, 0, st>>>(
+            static_cast<const T*>(y), static_cast<const T*>(dy), static_cast<const T*>(param),
+            static_cast<T*>(out), sample_size, min_output);
+    else
+        softmax_inst_map_kernel<T, 1, BACKWARD><<<pixel_grid(sample_size, 1, n), kBlockSize, 0, st>>>(
+            static_cast<const T*>(y), static_cast<const T*>(dy), static_cast<const T*>(param),
+            static_cast<T*>(out), sample_size, min_output);
+    return launch_status();
+}
+
+bool inst_bad(int num_samples, size_t sample_size)
+{
+    return num_samples < 0 || num_samples > 65535
+           || (sample_size + kBlockSize - 1) / kBlockSize > 0x7fffffffull;
+}
+
 } // namespace
 } // namespace h2x
 
@@ -441,4 +702,84 @@ extern "C" int h2x_softmax_channel_backward(h2x_dtype dtype, int num_samples, in
         return backward_impl<double>(num_samples, num_channels, spatial_size, y, dy, dx, as_stream(stream));
     }
     return H2X_ERR_UNSUPPORTED;
+}
+
+// ---- instance mode -------------------------------------------------------------
+
+extern "C" size_t h2x_softmax_instance_workspace_bytes(int num_samples)
+{
+    const size_t n = num_samples > 0 ? num_samples : 1;
+    return (n * inst_groups_per_sample_max(num_samples) * sizeof(double) + 255) / 256 * 256;
+}
+
+#define H2X_INST_ENTRY(CALL_F32, CALL_F64)                                                         \
+    if (inst_bad(num_samples, sample_size))                                                        \
+        return num_samples < 0 ? H2X_ERR_INVALID_ARGUMENT : H2X_ERR_TOO_LARGE;                     \
+    if (num_samples == 0 || sample_size == 0)                                                      \
+        return H2X_SUCCESS;                                                                        \
+    switch (dtype)                                                                                 \
+    {                                                                                              \
+    case H2X_F32: return CALL_F32;                                                                 \
+    case H2X_F64: return CALL_F64;                                                                 \
+    }                                                                                              \
+    return H2X_ERR_UNSUPPORTED
+
+extern "C" int h2x_softmax_instance_max(h2x_dtype dtype, int num_samples, size_t sample_size,
+                                        const void* x, void* sample_max, void* workspace,
+                                        h2x_stream_t stream)
+{
+    if (!x || !sample_max || !workspace)
+        return num_samples == 0 || sample_size == 0 ? H2X_SUCCESS : H2X_ERR_INVALID_ARGUMENT;
+    H2X_INST_ENTRY((inst_reduce<float, kInstMax>(num_samples, sample_size, x, nullptr, nullptr, nullptr,
+                                                 sample_max, workspace, as_stream(stream))),
+                   (inst_reduce<double, kInstMax>(num_samples, sample_size, x, nullptr, nullptr,
+                                                  nullptr, sample_max, workspace, as_stream(stream))));
+}
+
+extern "C" int h2x_softmax_instance_exp(h2x_dtype dtype, int num_samples, size_t sample_size,
+                                        const void* x, const void* sample_max, void* y,
+                                        void* sample_exp, void* workspace, h2x_stream_t stream)
+{
+    if (!x || !sample_max || !y || !sample_exp || !workspace)
+        return num_samples == 0 || sample_size == 0 ? H2X_SUCCESS : H2X_ERR_INVALID_ARGUMENT;
+    H2X_INST_ENTRY((inst_reduce<float, kInstExpSum>(num_samples, sample_size, x, nullptr, y, sample_max,
+                                                    sample_exp, workspace, as_stream(stream))),
+                   (inst_reduce<double, kInstExpSum>(num_samples, sample_size, x, nullptr, y,
+                                                     sample_max, sample_exp, workspace,
+                                                     as_stream(stream))));
+}
+
+extern "C" int h2x_softmax_instance_normalize(h2x_dtype dtype, int num_samples, size_t sample_size,
+                                              const void* sample_exp, void* y, h2x_stream_t stream)
+{
+    if (!sample_exp || !y)
+        return num_samples == 0 || sample_size == 0 ? H2X_SUCCESS : H2X_ERR_INVALID_ARGUMENT;
+    H2X_INST_ENTRY((inst_map<float, false>(num_samples, sample_size, y, nullptr, sample_exp, y,
+                                           as_stream(stream))),
+                   (inst_map<double, false>(num_samples, sample_size, y, nullptr, sample_exp, y,
+                                            as_stream(stream))));
+}
+
+extern "C" int h2x_softmax_instance_dot(h2x_dtype dtype, int num_samples, size_t sample_size,
+                                        const void* y, const void* dy, void* sample_dp,
+                                        void* workspace, h2x_stream_t stream)
+{
+    if (!y || !dy || !sample_dp || !workspace)
+        return num_samples == 0 || sample_size == 0 ? H2X_SUCCESS : H2X_ERR_INVALID_ARGUMENT;
+    H2X_INST_ENTRY((inst_reduce<float, kInstDot>(num_samples, sample_size, y, dy, nullptr, nullptr,
+                                                 sample_dp, workspace, as_stream(stream))),
+                   (inst_reduce<double, kInstDot>(num_samples, sample_size, y, dy, nullptr, nullptr,
+                                                  sample_dp, workspace, as_stream(stream))));
+}
+
+extern "C" int h2x_softmax_instance_gradient(h2x_dtype dtype, int num_samples, size_t sample_size,
+                                             const void* y, const void* dy, const void* sample_dp,
+                                             void* dx, h2x_stream_t stream)
+{
+    if (!y || !dy || !sample_dp || !dx)
+        return num_samples == 0 || sample_size == 0 ? H2X_SUCCESS : H2X_ERR_INVALID_ARGUMENT;
+    H2X_INST_ENTRY((inst_map<float, true>(num_samples, sample_size, y, dy, sample_dp, dx,
+                                          as_stream(stream))),
+                   (inst_map<double, true>(num_samples, sample_size, y, dy, sample_dp, dx,
+                                           as_stream(stream))));
 }

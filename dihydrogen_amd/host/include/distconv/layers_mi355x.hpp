@@ -424,19 +424,26 @@ private:
 template <typename Backend>
 class Softmax;
 
-// softmax.hpp:14-63, channel mode.
+// softmax.hpp:14-63.  Channel mode is one launch; instance mode runs the
+// reference's stages (legacy/src/dnn_backend/softmax.cu:705-784) with an
+// optional all-reduce of the per-sample scalars between them.
 template <>
 class Softmax<BackendMI355X>
 {
 public:
+    // allreduce(values, count, is_max): sums (or maximises) `count` per-sample
+    // scalars of type T over the ranks that share a sample (softmax.hpp:52-62)
+    using Allreduce = std::function<void(void*, size_t, bool)>;
+
     explicit Softmax(BackendMI355X const& backend) : m_stream(backend.get_stream()) {}
     explicit Softmax(hipStream_t stream) : m_stream(stream) {}
+
+    void set_allreducer(Allreduce fn) { m_allreducer = std::move(fn); }
 
     template <typename Tensor>
     void setup(const Tensor& input, SoftmaxMode mode)
     {
         (void) input;
-        assert_always(mode == SoftmaxMode::CHANNEL); // instance mode is not part of this path
         m_mode = mode;
     }
 
@@ -444,13 +451,31 @@ public:
     int forward(const Tensor& x, Tensor& y)
     {
         if (x.get_local_size() == 0)
-            return 0; // softmax.cu:600-603
+            return 0; // softmax.cu:600-603,717-720
         size_t spatial;
         int n, c;
         geometry(x, n, c, spatial);
-        DISTCONV_CHECK_H2X(h2x_softmax_channel_forward(Tensor::h2x_type(), n, c, spatial,
-                                                       x.get_const_base_ptr(), y.get_base_ptr(),
-                                                       m_stream));
+        const h2x_dtype dt = Tensor::h2x_type();
+        if (m_mode == SoftmaxMode::CHANNEL)
+        {
+            DISTCONV_CHECK_H2X(h2x_softmax_channel_forward(dt, n, c, spatial, x.get_const_base_ptr(),
+                                                           y.get_base_ptr(), m_stream));
+            return 0;
+        }
+        using T = typename Tensor::data_type;
+        const size_t size = spatial * c;
+        T* scalars = per_sample<T>(n);
+        T *smax = scalars, *sexp = scalars + n;
+        DISTCONV_CHECK_H2X(h2x_softmax_instance_max(dt, n, size, x.get_const_base_ptr(), smax,
+                                                    workspace(n), m_stream));
+        if (m_allreducer)
+            m_allreducer(smax, n, true);
+        DISTCONV_CHECK_H2X(h2x_softmax_instance_exp(dt, n, size, x.get_const_base_ptr(), smax,
+                                                    y.get_base_ptr(), sexp, workspace(n), m_stream));
+        if (m_allreducer)
+            m_allreducer(sexp, n, false);
+        DISTCONV_CHECK_H2X(h2x_softmax_instance_normalize(dt, n, size, sexp, y.get_base_ptr(),
+                                                          m_stream));
         return 0;
     }
 
@@ -462,10 +487,26 @@ public:
         size_t spatial;
         int n, c;
         geometry(dx, n, c, spatial);
-        DISTCONV_CHECK_H2X(h2x_softmax_channel_backward(Tensor::h2x_type(), n, c, spatial,
-                                                        y.get_const_base_ptr(),
-                                                        dy.get_const_base_ptr(), dx.get_base_ptr(),
-                                                        m_stream));
+        const h2x_dtype dt = Tensor::h2x_type();
+        if (m_mode == SoftmaxMode::CHANNEL)
+        {
+            DISTCONV_CHECK_H2X(h2x_softmax_channel_backward(dt, n, c, spatial,
+                                                            y.get_const_base_ptr(),
+                                                            dy.get_const_base_ptr(),
+                                                            dx.get_base_ptr(), m_stream));
+            return 0;
+        }
+        using T = typename Tensor::data_type;
+        const size_t size = spatial * c;
+        T* sdp = per_sample<T>(n);
+        DISTCONV_CHECK_H2X(h2x_softmax_instance_dot(dt, n, size, y.get_const_base_ptr(),
+                                                    dy.get_const_base_ptr(), sdp, workspace(n),
+                                                    m_stream));
+        if (m_allreducer)
+            m_allreducer(sdp, n, false);
+        DISTCONV_CHECK_H2X(h2x_softmax_instance_gradient(dt, n, size, y.get_const_base_ptr(),
+                                                         dy.get_const_base_ptr(), sdp,
+                                                         dx.get_base_ptr(), m_stream));
         return 0;
     }
 
@@ -481,8 +522,28 @@ private:
         spatial = t.get_local_size() / n / c;
     }
 
+    // The reference takes these from its device memory pool per call
+    // (softmax.cu:723-731); here they live with the layer object.
+    void* workspace(int n)
+    {
+        const size_t need = h2x_softmax_instance_workspace_bytes(n);
+        if (m_ws.is_null() || m_ws.get_size() < need)
+            m_ws.allocate(need);
+        return m_ws.get();
+    }
+    template <typename T>
+    T* per_sample(int n)
+    {
+        const size_t need = 2 * static_cast<size_t>(n) * sizeof(T);
+        if (m_scalars.is_null() || m_scalars.get_size() < need)
+            m_scalars.allocate(need);
+        return static_cast<T*>(m_scalars.get());
+    }
+
     hipStream_t m_stream;
     SoftmaxMode m_mode = SoftmaxMode::CHANNEL;
+    Allreduce m_allreducer;
+    tensor::Memory<tensor::CUDAAllocator> m_ws, m_scalars;
 };
 
 } // namespace distconv

@@ -234,38 +234,84 @@ class SoftmaxMode(Enum):
 
 
 class Softmax:
-    """Softmax<Backend> (legacy/include/distconv/dnn_backend/softmax.hpp:14-63);
-    channel mode only."""
+    """Softmax<Backend> (legacy/include/distconv/dnn_backend/softmax.hpp:14-63).
 
-    def __init__(self, stream: Optional[torch.cuda.Stream] = None):
-        self.stream = stream
+    ``allreduce(values, is_max)``, if given, is called on the per-sample scalars of
+    instance mode where the reference all-reduces them over the ranks that share
+    a sample (softmax.hpp:52-62); ``None`` means every sample is whole on this rank.
+    """
+
+    def __init__(self, stream: Optional[torch.cuda.Stream] = None,
+                 allreduce: Optional[Callable[[torch.Tensor, bool], None]] = None):
+        self.stream, self.allreduce = stream, allreduce
         self.mode = SoftmaxMode.CHANNEL
         self._lib = capi.load()
+        self._ws: Optional[torch.Tensor] = None
 
     def setup(self, input: Tensor, mode: SoftmaxMode) -> None:
-        if mode != SoftmaxMode.CHANNEL:
-            raise NotImplementedError("only SoftmaxMode.CHANNEL is implemented")
         self.mode = mode
 
     @staticmethod
     def _geometry(t: Tensor):
         if any(t.overlap):
-            raise NotImplementedError("channel softmax assumes a dense local tensor")  # softmax.cu:562-563
+            raise NotImplementedError("softmax assumes a dense local tensor")  # softmax.cu:562-563
         nd = t.get_num_dims()
         return t.local_shape[nd - 1], t.local_shape[nd - 2], _prod(t.local_shape[: nd - 2])
 
+    def _workspace(self, n: int) -> torch.Tensor:
+        need = self._lib.h2x_softmax_instance_workspace_bytes(n)
+        if self._ws is None or self._ws.numel() < need:
+            self._ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+        return self._ws
+
     def forward(self, x: Tensor, y: Tensor) -> int:
         n, c, s = self._geometry(x)
-        capi.check(self._lib.h2x_softmax_channel_forward(
-            x.h2x_dtype, n, c, s, _ptr(x.get_base_ptr()), _ptr(y.get_base_ptr()),
-            _stream_handle(self.stream)), "softmax forward")
+        if n == 0:
+            return 0
+        st = _stream_handle(self.stream)
+        if self.mode == SoftmaxMode.CHANNEL:
+            capi.check(self._lib.h2x_softmax_channel_forward(
+                x.h2x_dtype, n, c, s, _ptr(x.get_base_ptr()), _ptr(y.get_base_ptr()), st), "softmax forward")
+            return 0
+        # instance mode: softmax.cu:723-746
+        dt, size, ws = x.h2x_dtype, c * s, self._workspace(n)
+        smax = torch.empty(n, dtype=x.dtype, device=x.device)
+        sexp = torch.empty(n, dtype=x.dtype, device=x.device)
+        capi.check(self._lib.h2x_softmax_instance_max(dt, n, size, _ptr(x.get_base_ptr()), _ptr(smax),
+                                                      _ptr(ws), st), "softmax instance max")
+        if self.allreduce:
+            self.allreduce(smax, True)
+        capi.check(self._lib.h2x_softmax_instance_exp(dt, n, size, _ptr(x.get_base_ptr()), _ptr(smax),
+                                                      _ptr(y.get_base_ptr()), _ptr(sexp), _ptr(ws), st),
+                   "softmax instance exp")
+        if self.allreduce:
+            self.allreduce(sexp, False)
+        capi.check(self._lib.h2x_softmax_instance_normalize(dt, n, size, _ptr(sexp), _ptr(y.get_base_ptr()), st),
+                   "softmax instance normalize")
         return 0
 
     def backward(self, y: Tensor, dy: Tensor, dx: Tensor) -> int:
         n, c, s = self._geometry(dx)
-        capi.check(self._lib.h2x_softmax_channel_backward(
-            y.h2x_dtype, n, c, s, _ptr(y.get_base_ptr()), _ptr(dy.get_base_ptr()),
-            _ptr(dx.get_base_ptr()), _stream_handle(self.stream)), "softmax backward")
+        if n == 0:
+            return 0
+        st = _stream_handle(self.stream)
+        if self.mode == SoftmaxMode.CHANNEL:
+            capi.check(self._lib.h2x_softmax_channel_backward(
+                y.h2x_dtype, n, c, s, _ptr(y.get_base_ptr()), _ptr(dy.get_base_ptr()),
+                _ptr(dx.get_base_ptr()), st), "softmax backward")
+            return 0
+        # instance mode: softmax.cu:770-783
+        dt, size, ws = y.h2x_dtype, c * s, self._workspace(n)
+        sdp = torch.empty(n, dtype=y.dtype, device=y.device)
+        capi.check(self._lib.h2x_softmax_instance_dot(dt, n, size, _ptr(y.get_base_ptr()),
+                                                      _ptr(dy.get_base_ptr()), _ptr(sdp), _ptr(ws), st),
+                   "softmax instance dot")
+        if self.allreduce:
+            self.allreduce(sdp, False)
+        capi.check(self._lib.h2x_softmax_instance_gradient(dt, n, size, _ptr(y.get_base_ptr()),
+                                                           _ptr(dy.get_base_ptr()), _ptr(sdp),
+                                                           _ptr(dx.get_base_ptr()), st),
+                   "softmax instance gradient")
         return 0
 
 

@@ -318,6 +318,39 @@ int h2x_softmax_channel_backward(h2x_dtype dtype,
                                  void* dx,
                                  h2x_stream_t stream);
 
+/* Instance mode: softmax over all elements of a sample (dense tensors, a      */
+/* sample is `sample_size` contiguous elements).  The reference runs it as     */
+/* three forward and two backward stages with an all-reduce of the per-sample  */
+/* scalars between them when a sample is spread over ranks                     */
+/* (legacy/src/dnn_backend/softmax.cu:705-784,                                */
+/*  legacy/include/distconv/dnn_backend/softmax.hpp:52-62); the stages are    */
+/* the entry points.  Per-sample vectors hold num_samples elements.           */
+
+/** Workspace (fp64 partials) of the three reducing stages; no initialisation needed. */
+size_t h2x_softmax_instance_workspace_bytes(int num_samples);
+
+/** sample_max[n] = max(min_normal, max_i x): compute_max, softmax.cu:357-381. */
+int h2x_softmax_instance_max(h2x_dtype dtype, int num_samples, size_t sample_size, const void* x,
+                             void* sample_max, void* workspace, h2x_stream_t stream);
+
+/** y = exp(x - sample_max[n]); sample_exp[n] = sum_i y: compute_exp, softmax.cu:394-421. */
+int h2x_softmax_instance_exp(h2x_dtype dtype, int num_samples, size_t sample_size, const void* x,
+                             const void* sample_max, void* y, void* sample_exp, void* workspace,
+                             h2x_stream_t stream);
+
+/** y = max(y / sample_exp[n], sqrt(min_normal)) in place: compute_softmax, softmax.cu:424-456. */
+int h2x_softmax_instance_normalize(h2x_dtype dtype, int num_samples, size_t sample_size,
+                                   const void* sample_exp, void* y, h2x_stream_t stream);
+
+/** sample_dp[n] = sum_i y * dy: bp_dotproduct, softmax.cu:458-481. */
+int h2x_softmax_instance_dot(h2x_dtype dtype, int num_samples, size_t sample_size, const void* y,
+                             const void* dy, void* sample_dp, void* workspace, h2x_stream_t stream);
+
+/** dx = y > sqrt(min_normal) ? y * (dy - sample_dp[n]) : 0: bp_compute_gradient, softmax.cu:483-536. */
+int h2x_softmax_instance_gradient(h2x_dtype dtype, int num_samples, size_t sample_size,
+                                  const void* y, const void* dy, const void* sample_dp, void* dx,
+                                  h2x_stream_t stream);
+
 /* ------------------------------------------------------------------------ */
 /* Halo pack / unpack                                                        */
 /* ------------------------------------------------------------------------ */

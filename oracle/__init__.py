@@ -207,6 +207,39 @@ def softmax_channel_backward(y: np.ndarray, dy: np.ndarray) -> np.ndarray:
     return dx
 
 
+def softmax_instance_forward(x: np.ndarray, allreduce=None):
+    """Softmax::forward in instance mode (legacy/src/dnn_backend/softmax.cu:705-747):
+    returns y.  `allreduce(values, is_max)` stands where the reference all-reduces
+    the per-sample scalars over the ranks that share a sample."""
+    n = x.shape[0]
+    size = x.size // n if n else 0
+    sfx = _sfx(x.dtype)
+    mx, ex, y = np.empty(n, x.dtype), np.empty(n, x.dtype), np.empty_like(x)
+    getattr(lib(), "orc_softmax_instance_max_" + sfx)(ctypes.c_int(n), ctypes.c_size_t(size), _ptr(x), _ptr(mx))
+    if allreduce:
+        allreduce(mx, True)
+    getattr(lib(), "orc_softmax_instance_exp_" + sfx)(ctypes.c_int(n), ctypes.c_size_t(size), _ptr(x), _ptr(mx),
+                                                      _ptr(y), _ptr(ex))
+    if allreduce:
+        allreduce(ex, False)
+    getattr(lib(), "orc_softmax_instance_normalize_" + sfx)(ctypes.c_int(n), ctypes.c_size_t(size), _ptr(ex), _ptr(y))
+    return y
+
+
+def softmax_instance_backward(y: np.ndarray, dy: np.ndarray, allreduce=None):
+    """Softmax::backward in instance mode (softmax.cu:749-784)."""
+    n = y.shape[0]
+    size = y.size // n if n else 0
+    sfx = _sfx(y.dtype)
+    dp, dx = np.empty(n, y.dtype), np.empty_like(y)
+    getattr(lib(), "orc_softmax_instance_dot_" + sfx)(ctypes.c_int(n), ctypes.c_size_t(size), _ptr(y), _ptr(dy), _ptr(dp))
+    if allreduce:
+        allreduce(dp, False)
+    getattr(lib(), "orc_softmax_instance_gradient_" + sfx)(ctypes.c_int(n), ctypes.c_size_t(size), _ptr(y), _ptr(dy),
+                                                           _ptr(dp), _ptr(dx))
+    return dx
+
+
 # --------------------------------------------------------------------------
 # Halo pack / unpack
 # --------------------------------------------------------------------------

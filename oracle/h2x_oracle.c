@@ -12,8 +12,9 @@
  * the reference checkout).  What pins each function besides reading the
  * reference is listed in oracle/README.md.  PARITY UNPINNED: the FLT_MIN
  * clamp, the y > FLT_MIN guard and the FLT_MIN initial maximum of channel
- * softmax -- the reference holds no softmax test or vector; everything else
- * of softmax is pinned by the textbook routine.
+ * softmax, and the sqrt(FLT_MIN) clamp and guard of instance softmax -- the
+ * reference holds no softmax test or vector; everything else of softmax is
+ * pinned by the textbook routine.
  *
  * Build: see oracle/Makefile (gcc -O3 -fopenmp, -ffp-contract=off so that the
  * only fused multiply-adds are the ones written explicitly).

@@ -18,6 +18,11 @@ void orc_bn_backprop2_f32(int, int, size_t, size_t, size_t, size_t, size_t, cons
                           float);
 void orc_softmax_channel_forward_f32(int, int, size_t, const float*, float*);
 void orc_softmax_channel_backward_f32(int, int, size_t, const float*, const float*, float*);
+void orc_softmax_instance_max_f32(int, size_t, const float*, float*);
+void orc_softmax_instance_exp_f32(int, size_t, const float*, const float*, float*, float*);
+void orc_softmax_instance_normalize_f32(int, size_t, const float*, float*);
+void orc_softmax_instance_dot_f32(int, size_t, const float*, const float*, float*);
+void orc_softmax_instance_gradient_f32(int, size_t, const float*, const float*, const float*, float*);
 }
 
 static double max_rel(const std::vector<float>& a, const std::vector<float>& b)
@@ -105,6 +110,45 @@ static int test_bn(const Shape& shape)
     orc_bn_batch_normalization_f32(N, C, S, S, S, hx.data(), hrm.data(), hrv.data(), hscale.data(),
                                    hbias.data(), oy.data(), 1e-5f);
     errors += max_rel(to_host(y), oy) > tol;
+    return errors;
+}
+
+static int test_softmax_instance(const Shape& shape)
+{
+    const int nd = shape.length();
+    const int N = static_cast<int>(shape[-1]);
+    const size_t size = shape.get_size() / N;
+    const Distribution dist = Distribution::make_localized_distribution(nd);
+    const LocaleVirtual loc(0, 1);
+    DevTensor<float> x(shape, loc, dist), y(shape, loc, dist), dy(shape, loc, dist), dx(shape, loc, dist);
+    for (auto* t : {&x, &y, &dy, &dx})
+        t->allocate();
+    const auto hx = randn(shape.get_size(), 7, 2.0f), hdy = randn(shape.get_size(), 8);
+    to_device(x, hx);
+    to_device(dy, hdy);
+    BackendMI355X backend;
+    Softmax<BackendMI355X> sm(backend);
+    sm.setup(x, SoftmaxMode::INSTANCE);
+    CHECK(sm.forward(x, y) == 0);
+    CHECK(sm.backward(y, dy, dx) == 0);
+    const auto hy = to_host(y), hdx = to_host(dx);
+    std::vector<float> mx(N), ex(N), dp(N), oy(hx.size()), odx(hx.size());
+    orc_softmax_instance_max_f32(N, size, hx.data(), mx.data());
+    orc_softmax_instance_exp_f32(N, size, hx.data(), mx.data(), oy.data(), ex.data());
+    orc_softmax_instance_normalize_f32(N, size, ex.data(), oy.data());
+    orc_softmax_instance_dot_f32(N, size, hy.data(), hdy.data(), dp.data());
+    orc_softmax_instance_gradient_f32(N, size, hy.data(), hdy.data(), dp.data(), odx.data());
+    int errors = max_rel(hy, oy) > 1e-5;
+    // dx = y * (dy - dp) cancels where dy ~ dp: bound relative to the operands
+    for (size_t i = 0; i < hdx.size(); ++i)
+    {
+        const double bound = 1e-5 * std::fabs(hy[i]) * (std::fabs(hdy[i]) + std::fabs(dp[i / size]) + 1e-3);
+        if (std::fabs((double) hdx[i] - (double) odx[i]) > bound + 1e-30)
+        {
+            ++errors;
+            break;
+        }
+    }
     return errors;
 }
 
@@ -214,6 +258,8 @@ int main()
     errors += test_bn(Shape({16, 16, 16, 8, 4})); // 5-D
     errors += test_softmax(Shape({64, 64, 21, 4}));
     errors += test_softmax(Shape({5, 3, 7, 2}));
+    errors += test_softmax_instance(Shape({32, 32, 21, 4}));
+    errors += test_softmax_instance(Shape({5, 3, 7, 2}));
     std::printf("test_batchnorm_softmax: %d errors\n", errors);
     return errors ? 1 : 0;
 }

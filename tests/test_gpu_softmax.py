@@ -126,3 +126,68 @@ def test_float64(oracle_mod):
     y = yt.real_view().cpu().numpy()
     assert max_rel(y, oracle_mod.softmax_channel_forward(x)) <= 1e-12
     assert max_rel(dxt.real_view().cpu().numpy(), oracle_mod.softmax_channel_backward(y, dy)) <= 1e-12
+
+
+INSTANCE_CASES = [(16, 21, 64, 64), (3, 4, 5, 6), (2, 7, 9), (1, 2, 3, 4, 5), (5, 1, 1, 1), (2, 64, 128, 128)]
+
+
+@pytest.mark.parametrize("shape", INSTANCE_CASES)
+def test_instance_mode(shape, oracle_mod):
+    """SoftmaxMode::INSTANCE (legacy/src/dnn_backend/softmax.cu:705-784) against the oracle."""
+    import torch
+    from dihydrogen_amd.layers import Softmax, SoftmaxMode
+    rng = np.random.default_rng(123)
+    x = (2.0 * rng.standard_normal(shape)).astype(np.float32)
+    dy = rng.standard_normal(shape).astype(np.float32)
+    mk = _tensors(shape)
+    xt, yt, dyt, dxt = mk(), mk(), mk(), mk()
+    xt.real_view().copy_(torch.from_numpy(x))
+    dyt.real_view().copy_(torch.from_numpy(dy))
+    sm = Softmax()
+    sm.setup(xt, SoftmaxMode.INSTANCE)
+    assert sm.forward(xt, yt) == 0
+    torch.cuda.synchronize()
+    y = yt.real_view().cpu().numpy()
+    assert max_rel(y, oracle_mod.softmax_instance_forward(x)) <= TOL
+    assert sm.backward(yt, dyt, dxt) == 0
+    torch.cuda.synchronize()
+    # dp is a sum of signed terms; dx = y * (dy - dp): compare relative to the operands
+    dx, dx_o = dxt.real_view().cpu().numpy(), oracle_mod.softmax_instance_backward(y, dy)
+    n = shape[0]
+    bound = 1e-5 * np.abs(y) * (np.abs(dy) + np.abs(y * dy).reshape(n, -1).sum(axis=1).reshape((n,) + (1,) * (len(shape) - 1)))
+    assert (np.abs(dx - dx_o) <= bound + 1e-30).all()
+
+
+def test_instance_mode_split_sample_allreduce(oracle_mod):
+    """Two virtual ranks each hold half of every sample; the per-sample scalars
+    are combined through the allreduce hook (softmax.hpp:52-62)."""
+    import torch
+    from dihydrogen_amd.layers import Softmax, SoftmaxMode
+    rng = np.random.default_rng(77)
+    full = (2.0 * rng.standard_normal((4, 6, 8, 16))).astype(np.float32)
+    halves = [np.ascontiguousarray(full[:, :, :4]), np.ascontiguousarray(full[:, :, 4:])]
+    want = oracle_mod.softmax_instance_forward(full)
+    shape = halves[0].shape
+    mk = _tensors(shape)
+    xs, ys = [mk(), mk()], [mk(), mk()]
+    for t, h in zip(xs, halves):
+        t.real_view().copy_(torch.from_numpy(h))
+    # lock-step emulation: run rank 0's stage, then rank 1's, exchanging scalars in between
+    lib = __import__("dihydrogen_amd.capi", fromlist=["x"]).load()
+    from dihydrogen_amd import capi
+    n, size = shape[0], int(np.prod(shape[1:]))
+    ws = torch.empty(lib.h2x_softmax_instance_workspace_bytes(n), dtype=torch.uint8, device="cuda")
+    mx = [torch.empty(n, device="cuda") for _ in range(2)]
+    ex = [torch.empty(n, device="cuda") for _ in range(2)]
+    for r in range(2):
+        capi.check(lib.h2x_softmax_instance_max(capi.F32, n, size, xs[r].get_base_ptr(), mx[r].data_ptr(), ws.data_ptr(), None))
+    m = torch.maximum(mx[0], mx[1])
+    for r in range(2):
+        capi.check(lib.h2x_softmax_instance_exp(capi.F32, n, size, xs[r].get_base_ptr(), m.data_ptr(),
+                                                ys[r].get_base_ptr(), ex[r].data_ptr(), ws.data_ptr(), None))
+    e = ex[0] + ex[1]
+    for r in range(2):
+        capi.check(lib.h2x_softmax_instance_normalize(capi.F32, n, size, e.data_ptr(), ys[r].get_base_ptr(), None))
+    torch.cuda.synchronize()
+    got = np.concatenate([ys[0].real_view().cpu().numpy(), ys[1].real_view().cpu().numpy()], axis=2)
+    assert max_rel(got, want) <= TOL

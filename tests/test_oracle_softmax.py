@@ -72,3 +72,61 @@ def test_float64_variant():
     x = rng.standard_normal((2, 5, 3, 3))
     e = np.exp(x - x.max(axis=1, keepdims=True))
     assert max_rel(oracle.softmax_channel_forward(x), e / e.sum(axis=1, keepdims=True)) < 1e-13
+
+
+@pytest.mark.parametrize("shape", [(3, 4, 5, 6), (2, 21, 8), (1, 2, 3, 4, 5)])
+def test_instance_mode_against_torch(shape):
+    """Instance mode = softmax over all elements of a sample: torch.softmax on the
+    flattened sample and its autograd in float64."""
+    import torch
+    rng = np.random.default_rng(8)
+    x = (2 * rng.standard_normal(shape)).astype(np.float32)
+    dy = rng.standard_normal(shape).astype(np.float32)
+    xt = torch.tensor(x, dtype=torch.float64, requires_grad=True)
+    yt = torch.softmax(xt.reshape(shape[0], -1), dim=1).reshape(shape)
+    yt.backward(torch.tensor(dy, dtype=torch.float64))
+    y = oracle.softmax_instance_forward(x)
+    assert max_rel(y, yt.detach().numpy()) < 2e-6
+    dx = oracle.softmax_instance_backward(y, dy)
+    assert np.abs(dx - xt.grad.numpy()).max() < 2e-6
+    assert np.abs(y.reshape(shape[0], -1).astype(np.float64).sum(axis=1) - 1).max() < 1e-6
+    assert np.abs(dx.reshape(shape[0], -1).astype(np.float64).sum(axis=1)).max() < 1e-6
+
+
+def test_instance_mode_clamp_and_split_sample():
+    """Clamp and guard at sqrt(FLT_MIN) (softmax.cu:156-160); a sample split over
+    two ranks with the per-sample scalars all-reduced gives the unsplit result."""
+    x = np.zeros((1, 2, 2, 2), np.float32)
+    x[0, 0, 0, 0] = 100.0
+    y = oracle.softmax_instance_forward(x)
+    lim = np.float32(np.sqrt(np.float32(FLT_MIN)))
+    assert y[0, 0, 0, 0] == 1 and (y.reshape(-1)[1:] == lim).all()
+    assert (oracle.softmax_instance_backward(y, np.ones_like(x)).reshape(-1)[1:] == 0).all()
+    # split every sample's elements over two "ranks": record each rank's local
+    # scalars, combine them as the all-reduce would, then rerun with the combined values
+    rng = np.random.default_rng(9)
+    full = (2 * rng.standard_normal((3, 4, 6, 8))).astype(np.float32)
+    halves = [np.ascontiguousarray(full[:, :, :3]), np.ascontiguousarray(full[:, :, 3:])]
+
+    def staged(inject=None):
+        """Runs both ranks stage by stage; returns y of both."""
+        import ctypes
+        lib = oracle.lib()
+        n, size = 3, halves[0].size // 3
+        mx = [np.empty(n, np.float32) for _ in range(2)]
+        ex = [np.empty(n, np.float32) for _ in range(2)]
+        ys = [np.empty_like(h) for h in halves]
+        P = lambda a: ctypes.c_void_p(a.ctypes.data)
+        for r in range(2):
+            lib.orc_softmax_instance_max_f32(ctypes.c_int(n), ctypes.c_size_t(size), P(halves[r]), P(mx[r]))
+        m = np.maximum(mx[0], mx[1])                      # allreduce(max)
+        for r in range(2):
+            lib.orc_softmax_instance_exp_f32(ctypes.c_int(n), ctypes.c_size_t(size), P(halves[r]), P(m), P(ys[r]), P(ex[r]))
+        e = ex[0] + ex[1]                                 # allreduce(sum)
+        for r in range(2):
+            lib.orc_softmax_instance_normalize_f32(ctypes.c_int(n), ctypes.c_size_t(size), P(e), P(ys[r]))
+        return ys
+
+    y0, y1 = staged()
+    want = oracle.softmax_instance_forward(full)
+    assert max_rel(np.concatenate([y0, y1], axis=2), want) < 1e-6
