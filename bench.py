@@ -274,12 +274,10 @@ def main() -> int:
     bn_bytes = 8 * S3 * 4
     step_bytes = bn_bytes + halo.bytes
     step_elems = S3 + halo.elems
-    launch_bytes = halo.bytes // 6  # one launch: pack or unpack of the 16 faces of one dimension (read + write)
+    face_bytes = halo.bytes // (6 * 16)  # one face of one rank, read + write (16 faces per dimension)
     algo_bytes = {"bn_sums": S3 * 4, "bn_statistics": 0, "bn_apply": 2 * S3 * 4, "bn_backprop1": 2 * S3 * 4,
                   "bn_backprop2": 3 * S3 * 4}
-    for d in range(3):
-        algo_bytes[f"halo_dim{d}_pack"] = launch_bytes
-        algo_bytes[f"halo_dim{d}_unpack"] = launch_bytes
+    faces_per_launch = {}  # halo label -> faces in one launch (the exchange may split a phase)
 
     # Every launch of the step is bracketed by a pair of events on the stream it is
     # launched on (torch's current stream, whose handle the C ABI receives).
@@ -287,7 +285,10 @@ def main() -> int:
     recording = [False]
     only = [None]  # labels to instrument; None = all
 
-    def timed(label, launch):
+    def timed(label, launch, num_faces=None):
+        if num_faces is not None:
+            faces_per_launch[label] = num_faces
+            algo_bytes[label] = num_faces * face_bytes
         if not recording[0] or (only[0] is not None and label not in only[0]):
             launch()
             return
@@ -310,10 +311,10 @@ def main() -> int:
         timed("bn_backprop2", bn3.backward_apply)
         halo.run()
 
-    def kernel_share(evs):
+    def kernel_share(evs, steps):
         tot = {}
         for label, pairs in evs.items():
-            ms = statistics.mean(e0.elapsed_time(e1) for e0, e1 in pairs)
+            ms = sum(e0.elapsed_time(e1) for e0, e1 in pairs) / steps  # per step, all launches
             tot[KERNEL_OF[label]] = tot.get(KERNEL_OF[label], 0.0) + ms
         return tot
 
@@ -322,7 +323,7 @@ def main() -> int:
     for _ in range(max(args.warmup, 1)):
         step()
     torch.cuda.synchronize()
-    share0 = kernel_share(events)
+    share0 = kernel_share(events, max(args.warmup, 1))
     dominant = max(share0, key=share0.get)
     events.clear()
 
@@ -357,6 +358,9 @@ def main() -> int:
             "GB/s": _gbs(algo_bytes[label], ms), "frac": _gbs(algo_bytes[label], ms) / HBM_PEAK_GBS,
             "traffic": int((fetch_kib * scale + write_kib) * 1024) if label in PMC_KIB else None,
         }
+        if label in faces_per_launch:
+            launches[label]["faces"] = faces_per_launch[label]
+            launches[label]["launches_per_step"] = 16 // faces_per_launch[label]
     # dominant kernel = the kernel with the largest share of the step's launch time
     share = {}
     for label, v in launches.items():
@@ -406,6 +410,13 @@ def main() -> int:
         shf = ShuffleWorkload((128, 128, 64, 32), SEED + 5)
         breakdown["C5_shuffle_fwd"] = entry(4 * shf.elems * 4, shf.elems, *_time_events(shf.forward, it, wu))
         breakdown["C5_shuffle_bwd"] = entry(4 * shf.elems * 4, shf.elems, *_time_events(shf.backward, it, wu))
+
+        def round_trip():
+            shf.forward()
+            shf.backward()
+
+        breakdown["C5_shuffle_round_trip"] = entry(8 * shf.elems * 4, 2 * shf.elems,
+                                                   *_time_events(round_trip, it, wu))
         del shf
         torch.cuda.empty_cache()
 

@@ -192,11 +192,15 @@ __global__ __launch_bounds__(kBlockSize) void box_copy_kernel(const BoxBatch bat
             }
             else
             {
+                // The tensor is read once and streams past the memory-side
+                // cache; the packed image is stored normally so that it is
+                // still there when the matching unpack reads it.
                 WU v[kCopyUnroll];
 #pragma unroll
                 for (int u = 0; u < kCopyUnroll; ++u)
                     if (g[u] < count)
-                        v[u] = *reinterpret_cast<const WU*>(tensor + toff[u]);
+                        v[u] = __builtin_nontemporal_load(
+                            reinterpret_cast<const WU*>(tensor + toff[u]));
 #pragma unroll
                 for (int u = 0; u < kCopyUnroll; ++u)
                     if (g[u] < count)
@@ -209,7 +213,8 @@ __global__ __launch_bounds__(kBlockSize) void box_copy_kernel(const BoxBatch bat
 #pragma unroll
             for (int u = 0; u < kCopyUnroll; ++u)
                 if (g[u] < count)
-                    v[u] = *reinterpret_cast<const WA*>(buffer + g[u]);
+                    v[u] = __builtin_nontemporal_load(
+                        reinterpret_cast<const WA*>(buffer + g[u])); // last use of the image
             if constexpr (std::is_same<Op, OpId>::value)
             {
 #pragma unroll
@@ -219,7 +224,8 @@ __global__ __launch_bounds__(kBlockSize) void box_copy_kernel(const BoxBatch bat
                         if constexpr (SPARSE && VEC == 1)
                             sparse_store_scalar(tensor + toff[u], v[u][0]);
                         else
-                            *reinterpret_cast<WU*>(tensor + toff[u]) = v[u];
+                            __builtin_nontemporal_store(
+                                static_cast<WU>(v[u]), reinterpret_cast<WU*>(tensor + toff[u]));
                     }
             }
             else

@@ -10,6 +10,7 @@
 // all of them with as few launches as possible.
 #pragma once
 
+#include <algorithm>
 #include <memory>
 #include <vector>
 
@@ -271,36 +272,94 @@ public:
     void exchange(int dim, int wrs, int wrr, int wls, int wlr, hipStream_t stream, bool is_reverse,
                   bool skip_unpack, HaloExchangeAccumOp op)
     {
-        std::vector<h2x_halo_face> packs, unpacks;
-        for (auto& r : m_ranks)
-        {
-            if (!r->is_exchange_required(dim, wrs, wrr, wls, wlr))
-                continue;
-            for (Side side : SIDES)
-            {
-                const int peer = r->get_peer(dim, side);
-                if (peer == kProcNull)
-                    continue;
-                const int w_send = side == RHS ? wrs : wls;
-                const int w_recv = side == RHS ? wrr : wlr;
-                if (w_send > 0) // my RHS strip lands in my RHS neighbour's LHS receive buffer
-                    packs.push_back(face(*r, dim, side, w_send,
-                                         m_ranks[peer]->get_recv_buffer(dim, ~side), true,
-                                         is_reverse, op));
-                if (w_recv > 0 && !skip_unpack)
-                    unpacks.push_back(face(*r, dim, side, w_recv, r->get_recv_buffer(dim, side),
-                                           false, is_reverse, op));
-            }
-        }
         const h2x_dtype dt = TensorType::h2x_type();
-        if (!packs.empty())
-            DISTCONV_CHECK_H2X(h2x_halo_pack_or_unpack_batched(dt, packs.data(),
-                                                               static_cast<int>(packs.size()),
-                                                               stream));
-        if (!unpacks.empty())
-            DISTCONV_CHECK_H2X(h2x_halo_pack_or_unpack_batched(dt, unpacks.data(),
-                                                               static_cast<int>(unpacks.size()),
-                                                               stream));
+        const int width = std::max(std::max(wrs, wrr), std::max(wls, wlr));
+        for (const std::vector<int>& group : rank_groups(dim, width))
+        {
+            std::vector<h2x_halo_face> packs, unpacks;
+            for (int member : group)
+            {
+                auto& r = m_ranks[member];
+                if (!r->is_exchange_required(dim, wrs, wrr, wls, wlr))
+                    continue;
+                for (Side side : SIDES)
+                {
+                    const int peer = r->get_peer(dim, side);
+                    if (peer == kProcNull)
+                        continue;
+                    const int w_send = side == RHS ? wrs : wls;
+                    const int w_recv = side == RHS ? wrr : wlr;
+                    if (w_send > 0) // my RHS strip lands in my RHS neighbour's LHS receive buffer
+                        packs.push_back(face(*r, dim, side, w_send,
+                                             m_ranks[peer]->get_recv_buffer(dim, ~side), true,
+                                             is_reverse, op));
+                    if (w_recv > 0 && !skip_unpack)
+                        unpacks.push_back(face(*r, dim, side, w_recv,
+                                               r->get_recv_buffer(dim, side), false, is_reverse,
+                                               op));
+                }
+            }
+            if (!packs.empty())
+                DISTCONV_CHECK_H2X(h2x_halo_pack_or_unpack_batched(
+                    dt, packs.data(), static_cast<int>(packs.size()), stream));
+            if (!unpacks.empty())
+                DISTCONV_CHECK_H2X(h2x_halo_pack_or_unpack_batched(
+                    dt, unpacks.data(), static_cast<int>(unpacks.size()), stream));
+        }
+    }
+
+    // Ranks that exchange dimension `dim` together, group after group.  Faces
+    // of the innermost dimension touch one short run per row, each costing a
+    // 128-byte line, and the unpack writes into the lines its rank's pack has
+    // just read: a group is kept small enough for those lines to stay in the
+    // 256 MB memory-side cache between the two launches.  Neighbours along
+    // `dim` always share a group.
+    std::vector<std::vector<int>> rank_groups(int dim, int width) const
+    {
+        constexpr size_t kLineBytes = 128;
+        constexpr size_t kGroupBytes = size_t(320) << 20;
+        std::vector<std::vector<int>> groups;
+        if (dim != 0 || width * sizeof(DataType) >= kLineBytes)
+        {
+            groups.emplace_back();
+            for (int r = 0; r < num_ranks(); ++r)
+                groups.back().push_back(r);
+            return groups;
+        }
+        std::vector<bool> placed(m_ranks.size(), false);
+        size_t group_bytes = 0;
+        for (int r = 0; r < num_ranks(); ++r)
+        {
+            if (placed[r])
+                continue;
+            // the line of ranks through r along `dim`
+            std::vector<int> line;
+            size_t line_bytes = 0;
+            const auto& pr = m_ranks[r]->get_tensor().get_proc_index();
+            for (int q = r; q < num_ranks(); ++q)
+            {
+                const auto& t = m_ranks[q]->get_tensor();
+                bool same = !placed[q];
+                for (int i = 0; same && i < t.get_num_dims(); ++i)
+                    same = i == dim || t.get_proc_index()[i] == pr[i];
+                if (!same)
+                    continue;
+                placed[q] = true;
+                line.push_back(q);
+                size_t rows = 1;
+                for (int i = 1; i < t.get_num_dims(); ++i)
+                    rows *= static_cast<size_t>(t.get_local_real_shape()[i]);
+                line_bytes += rows * kLineBytes;
+            }
+            if (groups.empty() || group_bytes + line_bytes > kGroupBytes)
+            {
+                groups.emplace_back();
+                group_bytes = 0;
+            }
+            groups.back().insert(groups.back().end(), line.begin(), line.end());
+            group_bytes += line_bytes;
+        }
+        return groups;
     }
 
 private:

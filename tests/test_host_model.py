@@ -73,3 +73,37 @@ def test_shuffler_tables_match_oracle(src, dst):
         shuffler = S.__new__(S)
         shuffler.num_ranks = n
         assert shuffler._counts(a, b) == sc and shuffler._counts(b, a) == rc
+
+
+def test_halo_exchange_rank_groups():
+    """The innermost-dimension phase of a large exchange is split into groups
+    of ranks: every group is closed under the neighbour relation along that
+    dimension, the groups partition the ranks, and small or dense phases stay
+    one group."""
+    from dihydrogen_amd.layers import HaloExchangeVirtual as H
+
+    def make(gshape, locale, overlap):
+        dist = Distribution.make_overlapped_distribution(locale, overlap)
+        n = int(np.prod(locale))
+        x = H.__new__(H)
+        x.tensors = [Tensor(gshape, LocaleVirtual(r, n), dist) for r in range(n)]
+        x.dist, x.periodic = dist, True
+        return x
+
+    big = make((256, 256, 256, 32, 1), (2, 2, 2, 1, 1), (1, 1, 1, 0, 0))
+    groups = big._rank_groups(0, 1)
+    assert sorted(sum(groups, [])) == list(range(8)) and len(groups) == 2
+    for g in groups:
+        for r in g:
+            idx = list(big.tensors[r].proc_index)
+            for p in range(2):  # every rank of the line along dimension 0 is in the group
+                idx[0] = p
+                assert big.dist.rank_of(idx) in g
+    assert big._rank_groups(1, 1) == [list(range(8))]
+    assert big._rank_groups(2, 1) == [list(range(8))]
+    assert big._rank_groups(0, 32) == [list(range(8))]  # 128-byte runs are not sparse
+    small = make((16, 16, 16, 4, 1), (2, 2, 2, 1, 1), (1, 1, 1, 0, 0))
+    assert small._rank_groups(0, 1) == [list(range(8))]
+    # a line of four ranks along dimension 0 is never split, whatever its size
+    line = make((1024, 512, 256, 32, 1), (4, 1, 1, 1, 1), (1, 0, 0, 0, 0))
+    assert line._rank_groups(0, 1) == [list(range(4))]
