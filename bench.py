@@ -394,6 +394,14 @@ def main() -> int:
             ov = [1 if k == d else 0 for k in range(5)]
             fn = lambda ov=ov: halo.xch.exchange(ov, ov, ov, ov)
             breakdown[f"C2_halo_{name}"] = entry(halo.bytes // 3, halo.elems // 3, *_time_events(fn, it, wu))
+        # the same exchange as tensor-to-tensor transfers (no buffers): half the bytes per strip
+        breakdown["C2_halo_8ranks_fused"] = entry(
+            halo.bytes // 2, halo.elems // 2, *_time_events(lambda: halo.xch.exchange(fused=True), it, wu))
+        for d, name in enumerate(("dim0_W", "dim1_H", "dim2_D")):
+            ov = [1 if k == d else 0 for k in range(5)]
+            fn = lambda ov=ov: halo.xch.exchange(ov, ov, ov, ov, fused=True)
+            breakdown[f"C2_halo_{name}_fused"] = entry(halo.bytes // 6, halo.elems // 6,
+                                                       *_time_events(fn, it, wu))
         yard_x, yard_y = bn3.x.data, bn3.y.data
         breakdown["yardstick_torch_copy_268MB"] = entry(
             2 * S3 * 4, S3, *_time_events(lambda: yard_y.copy_(yard_x), it, wu))

@@ -41,6 +41,22 @@ class HaloFace(ctypes.Structure):
     ]
 
 
+class HaloTransfer(ctypes.Structure):
+    """struct h2x_halo_transfer"""
+    _fields_ = [
+        ("src", c_void_p),
+        ("dst", c_void_p),
+        ("src_real_shape", c_int64 * H2X_MAX_DIMS),
+        ("dst_real_shape", c_int64 * H2X_MAX_DIMS),
+        ("num_dims", c_int32),
+        ("dim", c_int32),
+        ("src_side", c_int32),
+        ("width", c_int32),
+        ("is_reverse", c_int32),
+        ("op", c_int32),
+    ]
+
+
 class TensorGeometry(ctypes.Structure):
     """struct h2x_tensor_geometry"""
     _fields_ = [
@@ -113,6 +129,7 @@ SIGNATURES = {
                                         c_int, c_void_p, c_int, c_int, c_int, c_void_p]),
     "h2x_halo_pack_or_unpack_batched": (c_int, [c_int, POINTER(HaloFace), c_int, c_void_p]),
     "h2x_halo_clear": (c_int, [c_int, c_void_p, c_int, POINTER(c_int64), c_int, c_int, c_void_p]),
+    "h2x_halo_exchange_fused": (c_int, [c_int, POINTER(HaloTransfer), c_int, c_void_p]),
     "h2x_shuffle_plan_create": (c_int, [POINTER(ShuffleGeometry), POINTER(c_void_p)]),
     "h2x_shuffle_plan_destroy": (c_int, [c_void_p]),
     "h2x_shuffle_pack": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p]),

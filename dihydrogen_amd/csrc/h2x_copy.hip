@@ -19,6 +19,10 @@
 // sides of a dimension, all peers of a rank, several virtual ranks -- share a
 // launch; their descriptors travel in the kernel arguments, so nothing is
 // allocated or copied to set a launch up.
+//
+// A fourth mode moves a strip straight from one tensor into another (the
+// neighbour's interior strip into this rank's halo) when both live on the same
+// device: pack and unpack of a halo exchange without the buffer in between.
 #include "h2x_device.hpp"
 
 #include <algorithm>
@@ -40,7 +44,8 @@ enum Mode : int
 {
     kPack = 0,    // buffer <- tensor
     kUnpack = 1,  // tensor <- op(tensor, buffer)
-    kClear = 2    // tensor <- 0
+    kClear = 2,   // tensor <- 0
+    kTransfer = 3 // tensor <- op(tensor, source tensor)
 };
 
 // One reduced box.  Packed element g (natural order of extent[]) lives at
@@ -48,10 +53,11 @@ enum Mode : int
 struct Box
 {
     char* tensor;            // base the strides are relative to
-    char* buffer;            // start of this box's contiguous image
+    char* buffer;            // start of this box's contiguous image (kTransfer: source box origin)
     char* tensor2;           // second box of identical geometry (sparse pairs), or null
     char* buffer2;
     int64_t stride[kMaxBoxDims]; // elements
+    int64_t stride_src[kMaxBoxDims]; // kTransfer: strides of the source tensor
     FastDiv div[kMaxBoxDims];    // by extent[i]; the last used one is never divided by
     uint32_t count;          // elements in the box (< 2^31)
     uint32_t first_block;    // first workgroup of this box in the launch
@@ -133,25 +139,32 @@ __global__ __launch_bounds__(kBlockSize) void box_copy_kernel(const BoxBatch bat
     const uint32_t block_base = (blockIdx.x - box.first_block) * (kStride * kCopyUnroll);
 
     int64_t toff[kCopyUnroll];
+    int64_t soff[kCopyUnroll]; // kTransfer only: offset in the source tensor
     uint32_t g[kCopyUnroll];
 #pragma unroll
     for (int u = 0; u < kCopyUnroll; ++u)
     {
         g[u] = block_base + u * kStride + threadIdx.x * VEC;
         uint32_t rem = g[u];
-        int64_t off = 0;
+        int64_t off = 0, src = 0;
 #pragma unroll
         for (int i = 0; i < kMaxBoxDims - 1; ++i)
         {
             if (i < nd - 1)
             {
                 const uint32_t q = fastdiv(rem, box.div[i]);
-                off += static_cast<int64_t>(rem - q * box.div[i].divisor) * box.stride[i];
+                const int64_t idx = rem - q * box.div[i].divisor;
+                off += idx * box.stride[i];
+                if (mode == kTransfer)
+                    src += idx * box.stride_src[i];
                 rem = q;
             }
         }
         off += static_cast<int64_t>(rem) * box.stride[nd - 1];
+        if (mode == kTransfer)
+            src += static_cast<int64_t>(rem) * box.stride_src[nd - 1];
         toff[u] = off;
+        soff[u] = src;
     }
 
     constexpr int kSides = SPARSE ? 2 : 1;
@@ -242,6 +255,81 @@ __global__ __launch_bounds__(kBlockSize) void box_copy_kernel(const BoxBatch bat
                     }
             }
         }
+        else if (mode == kTransfer)
+        {
+            // `buffer` is the origin of the source box in the other tensor
+            WU v[kCopyUnroll];
+            if constexpr (SPARSE)
+            {
+                // both faces' loads before any store, as for sparse packs
+                if (side == 1)
+                    break;
+                T* const tensor_b = reinterpret_cast<T*>(box.tensor2);
+                const T* const source_b = reinterpret_cast<const T*>(box.buffer2);
+                WU w[kCopyUnroll];
+#pragma unroll
+                for (int u = 0; u < kCopyUnroll; ++u)
+                    if (g[u] < count)
+                    {
+                        v[u] = *reinterpret_cast<const WU*>(buffer + soff[u]);
+                        if (tensor_b != nullptr)
+                            w[u] = *reinterpret_cast<const WU*>(source_b + soff[u]);
+                    }
+#pragma unroll
+                for (int u = 0; u < kCopyUnroll; ++u)
+                    if (g[u] < count)
+                    {
+                        if constexpr (std::is_same<Op, OpId>::value && VEC == 1)
+                        {
+                            sparse_store_scalar(tensor + toff[u], v[u][0]);
+                            if (tensor_b != nullptr)
+                                sparse_store_scalar(tensor_b + toff[u], w[u][0]);
+                        }
+                        else
+                        {
+                            WU t = *reinterpret_cast<const WU*>(tensor + toff[u]);
+#pragma unroll
+                            for (int j = 0; j < VEC; ++j)
+                                t[j] = op(t[j], v[u][j]);
+                            *reinterpret_cast<WU*>(tensor + toff[u]) = t;
+                            if (tensor_b != nullptr)
+                            {
+                                WU tb = *reinterpret_cast<const WU*>(tensor_b + toff[u]);
+#pragma unroll
+                                for (int j = 0; j < VEC; ++j)
+                                    tb[j] = op(tb[j], w[u][j]);
+                                *reinterpret_cast<WU*>(tensor_b + toff[u]) = tb;
+                            }
+                        }
+                    }
+            }
+            else
+            {
+#pragma unroll
+                for (int u = 0; u < kCopyUnroll; ++u)
+                    if (g[u] < count)
+                        v[u] = __builtin_nontemporal_load(
+                            reinterpret_cast<const WU*>(buffer + soff[u]));
+#pragma unroll
+                for (int u = 0; u < kCopyUnroll; ++u)
+                    if (g[u] < count)
+                    {
+                        if constexpr (std::is_same<Op, OpId>::value)
+                        {
+                            __builtin_nontemporal_store(
+                                v[u], reinterpret_cast<WU*>(tensor + toff[u]));
+                        }
+                        else
+                        {
+                            WU t = *reinterpret_cast<const WU*>(tensor + toff[u]);
+#pragma unroll
+                            for (int j = 0; j < VEC; ++j)
+                                t[j] = op(t[j], v[u][j]);
+                            *reinterpret_cast<WU*>(tensor + toff[u]) = t;
+                        }
+                    }
+            }
+        }
         else
         {
 #pragma unroll
@@ -272,26 +360,32 @@ struct HostBox
     int nd = 0;
     int64_t extent[kMaxBoxDims];
     int64_t stride[kMaxBoxDims];
+    int64_t stride_src[kMaxBoxDims] = {}; // transfers: strides of the source tensor
     int64_t tensor_offset = 0; // elements from the tensor pointer to the box origin
-    int64_t buffer_offset = 0; // elements from the buffer pointer
+    int64_t buffer_offset = 0; // elements from the buffer (transfers: source tensor) pointer
     int64_t count = 1;
+    bool transfer = false;
 };
 
 // Drops extent-1 dimensions and merges neighbours that are contiguous in the
-// tensor; the natural order of the reduced box is the natural order of the
-// original one.
+// tensor (for a transfer: in both tensors); the natural order of the reduced
+// box is the natural order of the original one.
 HostBox reduce_box(int nd, const int64_t* extent, const int64_t* stride, int64_t tensor_offset,
-                   int64_t buffer_offset)
+                   int64_t buffer_offset, const int64_t* stride_src = nullptr)
 {
     HostBox h;
     h.tensor_offset = tensor_offset;
     h.buffer_offset = buffer_offset;
+    h.transfer = stride_src != nullptr;
     for (int i = 0; i < nd; ++i)
     {
         h.count *= extent[i];
         if (extent[i] == 1)
             continue;
-        if (h.nd > 0 && stride[i] == h.stride[h.nd - 1] * h.extent[h.nd - 1])
+        const bool merge =
+            h.nd > 0 && stride[i] == h.stride[h.nd - 1] * h.extent[h.nd - 1]
+            && (!stride_src || stride_src[i] == h.stride_src[h.nd - 1] * h.extent[h.nd - 1]);
+        if (merge)
         {
             h.extent[h.nd - 1] *= extent[i];
         }
@@ -299,6 +393,7 @@ HostBox reduce_box(int nd, const int64_t* extent, const int64_t* stride, int64_t
         {
             h.extent[h.nd] = extent[i];
             h.stride[h.nd] = stride[i];
+            h.stride_src[h.nd] = stride_src ? stride_src[i] : 0;
             ++h.nd;
         }
     }
@@ -307,6 +402,7 @@ HostBox reduce_box(int nd, const int64_t* extent, const int64_t* stride, int64_t
         h.nd = 1;
         h.extent[0] = 1;
         h.stride[0] = 1;
+        h.stride_src[0] = 1;
     }
     return h;
 }
@@ -316,12 +412,17 @@ HostBox reduce_box(int nd, const int64_t* extent, const int64_t* stride, int64_t
 int box_vector(const HostBox& h, int elem_size, const void* buffer)
 {
     int v = 16 / elem_size;
-    if (h.stride[0] != 1)
+    if (h.stride[0] != 1 || (h.transfer && h.stride_src[0] != 1))
         return 1;
     while (v > 1)
     {
-        const bool ok = h.extent[0] % v == 0 && h.buffer_offset % v == 0
-                        && reinterpret_cast<uintptr_t>(buffer) % (static_cast<size_t>(v) * elem_size) == 0;
+        // a transfer has no buffer side: both tensors take unaligned vectors
+        const bool ok = h.extent[0] % v == 0
+                        && (h.transfer
+                            || (h.buffer_offset % v == 0
+                                && reinterpret_cast<uintptr_t>(buffer)
+                                           % (static_cast<size_t>(v) * elem_size)
+                                       == 0));
         if (ok)
             break;
         v /= 2;
@@ -334,7 +435,8 @@ bool same_geometry(const HostBox& a, const HostBox& b)
     if (a.nd != b.nd || a.count != b.count)
         return false;
     for (int i = 0; i < a.nd; ++i)
-        if (a.extent[i] != b.extent[i] || a.stride[i] != b.stride[i])
+        if (a.extent[i] != b.extent[i] || a.stride[i] != b.stride[i]
+            || a.stride_src[i] != b.stride_src[i])
             return false;
     return true;
 }
@@ -491,6 +593,7 @@ struct Launcher
         for (int i = 0; i < kMaxBoxDims; ++i)
         {
             b.stride[i] = i < h.nd ? h.stride[i] : 0;
+            b.stride_src[i] = i < h.nd ? h.stride_src[i] : 0;
             b.div[i] = make_fastdiv(i < h.nd ? static_cast<uint32_t>(h.extent[i]) : 1u);
         }
         b.count = static_cast<uint32_t>(h.count);
@@ -513,7 +616,7 @@ int elem_size_of(h2x_dtype dtype)
 }
 
 // The strip of a halo face as a box over the real tensor.
-int halo_box(const h2x_halo_face& f, HostBox* out)
+int halo_box(const h2x_halo_face& f, HostBox* out, bool origin_only = false)
 {
     const int nd = f.num_dims;
     if (nd < 1 || nd > H2X_MAX_DIMS || f.dim < 0 || f.dim >= nd || f.width < 0
@@ -539,6 +642,12 @@ int halo_box(const h2x_halo_face& f, HostBox* out)
     if (w > 0 && (start < 0 || start + w > len))
         return H2X_ERR_INVALID_ARGUMENT;
     extent[f.dim] = w;
+    if (origin_only)
+    {
+        *out = HostBox();
+        out->tensor_offset = start * stride[f.dim];
+        return H2X_SUCCESS;
+    }
     *out = reduce_box(nd, extent, stride, start * stride[f.dim], 0);
     return H2X_SUCCESS;
 }
@@ -657,6 +766,85 @@ extern "C" int h2x_halo_clear(h2x_dtype dtype, void* tensor, int num_dims,
             return err;
     }
     return l.flush();
+}
+
+extern "C" int h2x_halo_exchange_fused(h2x_dtype dtype, const h2x_halo_transfer* transfers,
+                                       int num_transfers, h2x_stream_t stream)
+{
+    const int es = elem_size_of(dtype);
+    if (es == 0)
+        return H2X_ERR_UNSUPPORTED;
+    if (num_transfers < 0 || (num_transfers > 0 && !transfers))
+        return H2X_ERR_INVALID_ARGUMENT;
+    // validate everything before anything is launched
+    std::vector<HostBox> boxes(num_transfers);
+    for (int i = 0; i < num_transfers; ++i)
+    {
+        const h2x_halo_transfer& t = transfers[i];
+        if (t.op < H2X_HALO_ID || t.op > H2X_HALO_MIN
+            || (t.src_side != H2X_LHS && t.src_side != H2X_RHS))
+            return H2X_ERR_INVALID_ARGUMENT;
+        // the strip as pack sees it in src and as unpack sees it in dst
+        h2x_halo_face from, to;
+        std::memset(&from, 0, sizeof(from));
+        std::memset(&to, 0, sizeof(to));
+        from.num_dims = to.num_dims = t.num_dims;
+        from.dim = to.dim = t.dim;
+        from.width = to.width = t.width;
+        from.side = t.src_side;
+        to.side = t.src_side == H2X_LHS ? H2X_RHS : H2X_LHS;
+        from.inner = t.is_reverse ? 0 : 1;
+        to.inner = t.is_reverse ? 1 : 0;
+        if (t.num_dims < 1 || t.num_dims > H2X_MAX_DIMS)
+            return H2X_ERR_INVALID_ARGUMENT;
+        for (int d = 0; d < t.num_dims; ++d)
+        {
+            from.real_shape[d] = t.src_real_shape[d];
+            to.real_shape[d] = t.dst_real_shape[d];
+            if (d != t.dim && t.src_real_shape[d] != t.dst_real_shape[d])
+                return H2X_ERR_INVALID_ARGUMENT;
+        }
+        HostBox a, b;
+        int err = halo_box(from, &a, true);
+        if (err == 0)
+            err = halo_box(to, &b, true);
+        if (err != 0)
+            return err;
+        // same extents, two sets of strides
+        int64_t extent[kMaxBoxDims], stride_dst[kMaxBoxDims], stride_src[kMaxBoxDims];
+        int64_t sd = 1, ss = 1;
+        for (int d = 0; d < t.num_dims; ++d)
+        {
+            extent[d] = d == t.dim ? t.width : t.dst_real_shape[d];
+            stride_dst[d] = sd;
+            stride_src[d] = ss;
+            sd *= t.dst_real_shape[d];
+            ss *= t.src_real_shape[d];
+        }
+        boxes[i] = reduce_box(t.num_dims, extent, stride_dst, b.tensor_offset, a.tensor_offset,
+                              stride_src);
+        if (boxes[i].count > 0 && (!t.src || !t.dst))
+            return H2X_ERR_INVALID_ARGUMENT;
+        if (boxes[i].count >= (1ll << 31))
+            return H2X_ERR_TOO_LARGE;
+    }
+    for (int op = H2X_HALO_ID; op <= H2X_HALO_MIN; ++op)
+    {
+        Launcher l(as_stream(stream), es, dtype, op);
+        for (int i = 0; i < num_transfers; ++i)
+        {
+            if (transfers[i].op != op)
+                continue;
+            const int err = l.add(boxes[i], transfers[i].dst, const_cast<void*>(transfers[i].src),
+                                  kTransfer);
+            if (err != 0)
+                return err;
+        }
+        const int err = l.flush();
+        if (err != 0)
+            return err;
+    }
+    return H2X_SUCCESS;
 }
 
 // ---- shuffle -------------------------------------------------------------------

@@ -308,6 +308,65 @@ public:
         }
     }
 
+    // The exchange of all dimensions with every strip moved straight from the
+    // neighbour's tensor into this rank's (one launch per dimension and group
+    // of ranks, no buffers).  The tensors end up as after exchange().
+    void exchange_fused(hipStream_t stream, bool is_reverse = false,
+                        HaloExchangeAccumOp op = HaloExchangeAccumOp::ID)
+    {
+        const IntVector& w = m_ranks[0]->get_tensor().get_halo_width();
+        const int nd = m_ranks[0]->get_tensor().get_num_dims();
+        for (int d = 0; d < nd; ++d)
+            exchange_fused(d, w[d], w[d], stream, is_reverse, op);
+    }
+
+    // width_rhs: strips that cross a rank's RHS face (sent from its RHS side and
+    // received on the neighbour's LHS side); width_lhs likewise.
+    void exchange_fused(int dim, int width_rhs, int width_lhs, hipStream_t stream, bool is_reverse,
+                        HaloExchangeAccumOp op)
+    {
+        const h2x_dtype dt = TensorType::h2x_type();
+        for (const std::vector<int>& group : rank_groups(dim, std::max(width_rhs, width_lhs)))
+        {
+            std::vector<h2x_halo_transfer> moves;
+            for (int member : group)
+            {
+                auto& r = m_ranks[member]; // the receiver
+                if (!r->is_exchange_required(dim, width_rhs, width_rhs, width_lhs, width_lhs))
+                    continue;
+                for (Side side : SIDES)
+                {
+                    const int peer = r->get_peer(dim, side);
+                    // my RHS halo holds what my RHS neighbour sends from its LHS side
+                    const int width = side == RHS ? width_lhs : width_rhs;
+                    if (peer == kProcNull || width == 0)
+                        continue;
+                    auto& src = m_ranks[peer]->get_tensor();
+                    auto& dst = r->get_tensor();
+                    assert_always(width <= dst.get_halo_width(dim));
+                    h2x_halo_transfer m = {};
+                    m.src = src.get_buffer();
+                    m.dst = dst.get_buffer();
+                    for (int i = 0; i < dst.get_num_dims(); ++i)
+                    {
+                        m.src_real_shape[i] = static_cast<int64_t>(src.get_local_real_shape()[i]);
+                        m.dst_real_shape[i] = static_cast<int64_t>(dst.get_local_real_shape()[i]);
+                    }
+                    m.num_dims = dst.get_num_dims();
+                    m.dim = dim;
+                    m.src_side = static_cast<int>(~side);
+                    m.width = width;
+                    m.is_reverse = is_reverse ? 1 : 0;
+                    m.op = static_cast<int>(op);
+                    moves.push_back(m);
+                }
+            }
+            if (!moves.empty())
+                DISTCONV_CHECK_H2X(h2x_halo_exchange_fused(dt, moves.data(),
+                                                           static_cast<int>(moves.size()), stream));
+        }
+    }
+
     // Ranks that exchange dimension `dim` together, group after group.  Faces
     // of the innermost dimension touch one short run per row, each costing a
     // 128-byte line, and the unpack writes into the lines its rank's pack has

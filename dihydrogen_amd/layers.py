@@ -406,11 +406,19 @@ class HaloExchangeVirtual:
 
     def exchange_dim(self, dim: int, width_rhs_send: int, width_rhs_recv: int, width_lhs_send: int,
                      width_lhs_recv: int, is_reverse: bool = False, skip_unpack: bool = False,
-                     op: HaloExchangeAccumOp = HaloExchangeAccumOp.ID) -> None:
+                     op: HaloExchangeAccumOp = HaloExchangeAccumOp.ID, fused: bool = False) -> None:
         """One dimension for all ranks; the order pack -> (transfer) -> unpack of
         halo_exchange_cuda_mpi.hpp:25-100.  A rank's RHS strip goes to its RHS
-        neighbour's LHS receive buffer and vice versa."""
+        neighbour's LHS receive buffer and vice versa.  With ``fused`` the strips
+        move straight from tensor to tensor in one launch per group of ranks;
+        the result is the same."""
         dtype = self.tensors[0].h2x_dtype
+        if fused:
+            if skip_unpack:
+                raise ValueError("a fused exchange has no separate unpack to skip")
+            self._exchange_dim_fused(dim, width_rhs_send, width_rhs_recv, width_lhs_send,
+                                     width_lhs_recv, is_reverse, op)
+            return
         key = (dim, width_rhs_send, width_rhs_recv, width_lhs_send, width_lhs_recv, is_reverse,
                skip_unpack, op)
         cached = self._faces.get(key)
@@ -450,6 +458,53 @@ class HaloExchangeVirtual:
                 else:
                     self.launch_hook(f"halo_dim{dim}_{what}", launch, len(arr))
 
+    def _exchange_dim_fused(self, dim, width_rhs_send, width_rhs_recv, width_lhs_send,
+                            width_lhs_recv, is_reverse, op) -> None:
+        dtype = self.tensors[0].h2x_dtype
+        widths = (width_rhs_send, width_rhs_recv, width_lhs_send, width_lhs_recv)
+        key = ("fused", dim) + widths + (is_reverse, op)
+        cached = self._faces.get(key)
+        if cached is None:
+            cached = []
+            for group in self._rank_groups(dim, max(widths)):
+                moves = []
+                for r in group:  # r receives; both of its halos are neighbours in the table
+                    if not self.is_exchange_required(r, dim, widths):
+                        continue
+                    for side in (capi.LHS, capi.RHS):
+                        peer = self.find_peer_rank(r, dim, side)
+                        if peer is None:
+                            continue
+                        # what the peer sends towards r leaves the peer on the opposite side
+                        w_send = width_lhs_send if side == capi.RHS else width_rhs_send
+                        w_recv = width_rhs_recv if side == capi.RHS else width_lhs_recv
+                        if w_send != w_recv:
+                            raise ValueError("a fused exchange needs equal send and receive widths")
+                        if w_recv == 0:
+                            continue
+                        src, dst = self.tensors[peer], self.tensors[r]
+                        m = capi.HaloTransfer()
+                        m.src, m.dst = src.get_buffer(), dst.get_buffer()
+                        for i in range(self.nd):
+                            m.src_real_shape[i] = src.local_real_shape[i]
+                            m.dst_real_shape[i] = dst.local_real_shape[i]
+                        m.num_dims, m.dim, m.width = self.nd, dim, w_recv
+                        m.src_side = capi.LHS if side == capi.RHS else capi.RHS
+                        m.is_reverse, m.op = int(is_reverse), op.value
+                        moves.append(m)
+                cached.append((capi.HaloTransfer * len(moves))(*moves) if moves else None)
+            self._faces[key] = cached
+        st = _stream_handle(self.stream)
+        for arr in cached:
+            if arr is None:
+                continue
+            launch = lambda arr=arr: capi.check(
+                self._lib.h2x_halo_exchange_fused(dtype, arr, len(arr), st), "fused halo exchange")
+            if self.launch_hook is None:
+                launch()
+            else:
+                self.launch_hook(f"halo_dim{dim}_fused", launch, len(arr))
+
     # Faces of the innermost dimension touch one short run per row, and every
     # run costs a whole 128-byte line of memory traffic; the unpack writes into
     # the lines its rank's pack has just read.  Exchanging a few ranks at a time
@@ -486,7 +541,7 @@ class HaloExchangeVirtual:
 
     def exchange(self, widths_rhs_send=None, widths_rhs_recv=None, widths_lhs_send=None,
                  widths_lhs_recv=None, is_reverse: bool = False, skip_unpack: bool = False,
-                 op: HaloExchangeAccumOp = HaloExchangeAccumOp.ID) -> None:
+                 op: HaloExchangeAccumOp = HaloExchangeAccumOp.ID, fused: bool = False) -> None:
         """All dimensions, innermost first, each seeing the halo cells the previous
         ones filled (halo_exchange_cuda.hpp:56-106)."""
         ov = self.tensors[0].overlap
@@ -495,7 +550,7 @@ class HaloExchangeVirtual:
         wls = ov if widths_lhs_send is None else widths_lhs_send
         wlr = ov if widths_lhs_recv is None else widths_lhs_recv
         for d in range(self.nd):
-            self.exchange_dim(d, wrs[d], wrr[d], wls[d], wlr[d], is_reverse, skip_unpack, op)
+            self.exchange_dim(d, wrs[d], wrr[d], wls[d], wlr[d], is_reverse, skip_unpack, op, fused)
 
     def clear_halo(self, dim: int) -> None:
         """Tensor::clear_halo (legacy/src/tensor/tensor_mpi_cuda.cu:14-84) on every rank."""

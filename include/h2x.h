@@ -430,6 +430,45 @@ int h2x_halo_clear(h2x_dtype dtype,
                    int width,
                    h2x_stream_t stream);
 
+/**
+ * One strip moved straight from the tensor of one rank into the tensor of its
+ * neighbour on the same device: what
+ *   h2x_halo_pack_or_unpack(src, ..., dim, src_side, width, buf, is_pack=1, is_reverse, ...)
+ * followed by
+ *   h2x_halo_pack_or_unpack(dst, ..., dim, opposite side, width, buf, is_pack=0, is_reverse, op)
+ * leaves in `dst`, without the buffer.  Forward (is_reverse = 0): the interior
+ * strip of `src` at `src_side` lands in the halo of `dst` on the opposite side;
+ * reverse: the halo of `src` at `src_side` is combined with `op` into the
+ * interior strip of `dst` on the opposite side.  The two real shapes must agree
+ * in every dimension but `dim`.  The reference always stages strips through
+ * buffers (legacy/include/distconv/tensor/halo_exchange_cuda_mpi.hpp:25-100,
+ * halo_packing_cuda.hpp:143-167); this entry point is for neighbours that
+ * share a device.
+ */
+typedef struct h2x_halo_transfer
+{
+    const void* src;  /* start of the source rank's real allocation */
+    void* dst;        /* start of the destination rank's real allocation */
+    int64_t src_real_shape[H2X_MAX_DIMS];
+    int64_t dst_real_shape[H2X_MAX_DIMS];
+    int32_t num_dims;
+    int32_t dim;
+    int32_t src_side;   /* h2x_side: the side of `src` that faces `dst` */
+    int32_t width;
+    int32_t is_reverse;
+    int32_t op;         /* h2x_halo_op */
+} h2x_halo_transfer;
+
+/**
+ * `num_transfers` strips in as few launches as possible.  No transfer of a
+ * call may write what another one reads or writes (true for all strips of one
+ * dimension of an exchange).  `transfers` is host memory, read before return.
+ */
+int h2x_halo_exchange_fused(h2x_dtype dtype,
+                            const h2x_halo_transfer* transfers,
+                            int num_transfers,
+                            h2x_stream_t stream);
+
 /* ------------------------------------------------------------------------ */
 /* Tensor shuffler pack / unpack                                             */
 /* ------------------------------------------------------------------------ */

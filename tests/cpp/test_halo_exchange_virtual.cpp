@@ -4,7 +4,8 @@
 // global offset of its source.
 #include "test_common.hpp"
 
-static int run_case(const Shape& shape, const Shape& locale, const IntVector& overlap, bool periodic)
+static int run_case(const Shape& shape, const Shape& locale, const IntVector& overlap, bool periodic,
+                    bool fused = false)
 {
     const int nd = shape.length();
     const int n = static_cast<int>(locale.get_size());
@@ -22,7 +23,10 @@ static int run_case(const Shape& shape, const Shape& locale, const IntVector& ov
     for (int d = 0; d < nd; ++d) // Convolution clears the halo before every exchange
         for (auto* t : ptrs)
             t->clear_halo(d, nullptr);
-    xch.exchange(nullptr);
+    if (fused)
+        xch.exchange_fused(nullptr);
+    else
+        xch.exchange(nullptr);
     int errors = 0;
     for (int r = 0; r < n; ++r)
     {
@@ -66,6 +70,9 @@ int main()
         errors += run_case(Shape({13, 11, 3, 2}), Shape({3, 2, 1, 1}), IntVector({1, 2, 0, 0}), periodic);
         errors += run_case(Shape({8, 10, 12, 3, 2}), Shape({2, 2, 2, 1, 1}), IntVector({1, 1, 1, 0, 0}), periodic);
         errors += run_case(Shape({8, 9, 10, 2, 1}), Shape({1, 2, 2, 1, 1}), IntVector({0, 2, 1, 0, 0}), periodic);
+        // tensor-to-tensor transfers instead of pack + unpack
+        errors += run_case(Shape({13, 11, 3, 2}), Shape({3, 2, 1, 1}), IntVector({1, 2, 0, 0}), periodic, true);
+        errors += run_case(Shape({8, 10, 12, 3, 2}), Shape({2, 2, 2, 1, 1}), IntVector({1, 1, 1, 0, 0}), periodic, true);
     }
     // per-rank interface: pack one strip, unpack it on the neighbour
     {

@@ -61,7 +61,8 @@ def test_accumulate_ops(op, dtype, oracle_mod):
             _single_face((4, 4, 8, 12), dim, side, 1, False, False, op, dtype, oracle_mod)
 
 
-def _exchange_case(shape, locale, overlap, periodic, oracle_mod, widths=None, dtype=np.float32):
+def _exchange_case(shape, locale, overlap, periodic, oracle_mod, widths=None, dtype=np.float32,
+                   fused=False):
     """Runs the exchange on the GPU and on the CPU oracle; returns both."""
     import torch
     from oracle import geometry as G
@@ -85,9 +86,9 @@ def _exchange_case(shape, locale, overlap, periodic, oracle_mod, widths=None, dt
         tensors.append(t)
     xch = HaloExchangeVirtual(tensors, periodic=periodic)
     if widths is None:
-        xch.exchange()
+        xch.exchange(fused=fused)
     else:
-        xch.exchange(widths, widths, widths, widths)
+        xch.exchange(widths, widths, widths, widths, fused=fused)
     torch.cuda.synchronize()
     oracle_halo_exchange(oracle_mod, geoms, fields, periodic, widths)
     return geoms, fields, [t.real_view().cpu().numpy() for t in tensors]
@@ -143,6 +144,72 @@ def test_exchange_closed_form_and_oracle(case, periodic, oracle_mod):
     _closed_form_check(geoms, got, periodic)
     for w, g in zip(want, got):
         assert np.array_equal(w, g, equal_nan=True)
+
+
+@pytest.mark.parametrize("periodic", [False, True])
+@pytest.mark.parametrize("case", EXCHANGE_CASES)
+def test_fused_exchange_closed_form_and_oracle(case, periodic, oracle_mod):
+    """Tensor-to-tensor transfers leave what pack + unpack through buffers leave."""
+    shape, locale, overlap = case
+    geoms, want, got = _exchange_case(shape, locale, overlap, periodic, oracle_mod, fused=True)
+    _closed_form_check(geoms, got, periodic)
+    for w, g in zip(want, got):
+        assert np.array_equal(w, g, equal_nan=True)
+
+
+def test_fused_exchange_narrower_than_halo_f64(oracle_mod):
+    shape, locale, overlap = (12, 10, 3, 2), (2, 2, 1, 1), (2, 2, 0, 0)
+    geoms, want, got = _exchange_case(shape, locale, overlap, True, oracle_mod, widths=[1, 1, 0, 0],
+                                      dtype=np.float64, fused=True)
+    for w, g in zip(want, got):
+        assert np.array_equal(w, g, equal_nan=True)
+
+
+@pytest.mark.parametrize("op", [1, 2, 3])
+def test_fused_reverse_exchange_ops(op, oracle_mod):
+    """Reverse transfers combine the neighbour's halo into the boundary cells
+    with SUM / MAX / MIN, as the unpack of halo_packing_cuda.hpp:36-58 does."""
+    import torch
+    from oracle import geometry as G
+    from dihydrogen_amd.layers import HaloExchangeAccumOp, HaloExchangeVirtual
+    from dihydrogen_amd.tensor import Distribution, LocaleVirtual, Tensor
+    shape, locale, overlap = (10, 12, 6, 2, 1), (2, 3, 2, 1, 1), (1, 2, 1, 0, 0)
+    nranks = 12
+    rng = np.random.default_rng(80 + op)
+    geoms = [G.TensorGeom(shape, G.Dist(locale, locale, overlap), r) for r in range(nranks)]
+    fields = [rng.integers(-8, 8, g.real_shape[::-1]).astype(np.float32) for g in geoms]
+    dist = Distribution.make_overlapped_distribution(locale, overlap)
+    tensors = []
+    for r in range(nranks):
+        t = Tensor(shape, LocaleVirtual(r, nranks), dist).allocate()
+        t.real_view().copy_(torch.from_numpy(fields[r]))
+        tensors.append(t)
+    HaloExchangeVirtual(tensors, periodic=True).exchange(is_reverse=True, op=HaloExchangeAccumOp(op),
+                                                         fused=True)
+    torch.cuda.synchronize()
+    oracle_halo_exchange(oracle_mod, geoms, fields, True, None, True, op)
+    for f, t in zip(fields, tensors):
+        assert np.array_equal(f, t.real_view().cpu().numpy())
+
+
+def test_fused_transfer_rejects_mismatched_shapes():
+    import torch
+    from dihydrogen_amd import capi
+    lib = capi.load()
+    a, b = torch.zeros(4 * 6 * 8, device="cuda"), torch.ones(4 * 6 * 8, device="cuda")
+    m = capi.HaloTransfer()
+    m.src, m.dst = a.data_ptr(), b.data_ptr()
+    for i, (x, y) in enumerate(zip((8, 6, 4), (8, 5, 4))):
+        m.src_real_shape[i], m.dst_real_shape[i] = x, y
+    m.num_dims, m.dim, m.src_side, m.width, m.is_reverse, m.op = 3, 0, capi.RHS, 1, 0, 0
+    assert lib.h2x_halo_exchange_fused(capi.F32, m, 1, None) == -1  # extents differ off the exchanged dimension
+    m.dst_real_shape[1] = 6
+    m.width = 5  # two strips of 5 do not fit in 8
+    assert lib.h2x_halo_exchange_fused(capi.F32, m, 1, None) == -1
+    m.width = 0
+    assert lib.h2x_halo_exchange_fused(capi.F32, m, 1, None) == 0
+    torch.cuda.synchronize()
+    assert (b == 1).all()
 
 
 def test_exchange_narrower_than_halo(oracle_mod):
