@@ -219,17 +219,17 @@ def cpu_baseline(repeats: int = 3):
 # HBM traffic per launch measured with rocprofv3 --pmc (profiles/bench_pmc_traffic.txt):
 # FETCH_SIZE and WRITE_SIZE in KiB per dispatch; FETCH_SIZE reads 0.5x for full-line
 # streaming reads on this stack (calibrated there on a copy of known size), WRITE_SIZE 1.0x.
-PMC_KIB = {  # label -> (FETCH_SIZE KiB, fetch scale, WRITE_SIZE KiB)
-    "bn_sums": (131096, 2.0, 128),
-    "bn_apply": (131093, 2.0, 262144),
-    "bn_backprop1": (262185, 2.0, 128),
-    "bn_backprop2": (262174, 2.0, 262144),
-    "halo_dim0_pack": (314300, 2.0, 33800),
-    "halo_dim0_unpack": (16952, 2.0, 270400),
-    "halo_dim1_pack": (21104, 2.0, 33800),
-    "halo_dim1_unpack": (16960, 2.0, 35495),
-    "halo_dim2_pack": (17126, 2.0, 33800),
-    "halo_dim2_unpack": (16960, 2.0, 33909),
+PMC_KIB = {  # label -> (FETCH_SIZE KiB, fetch scale, WRITE_SIZE KiB) per launch
+    "bn_sums": (131095, 2.0, 128),
+    "bn_apply": (131102, 2.0, 262162),
+    "bn_backprop1": (262182, 2.0, 128),
+    "bn_backprop2": (262178, 2.0, 262144),
+    "halo_dim0_pack": (153250, 2.0, 16900),    # 8 faces per launch, two launches per step
+    "halo_dim0_unpack": (8512, 2.0, 135200),
+    "halo_dim1_pack": (21181, 2.0, 33800),
+    "halo_dim1_unpack": (16968, 2.0, 37138),
+    "halo_dim2_pack": (17171, 2.0, 33800),
+    "halo_dim2_unpack": (16975, 2.0, 34929),
 }
 
 KERNEL_OF = {
