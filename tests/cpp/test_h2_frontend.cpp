@@ -1,0 +1,325 @@
+// The h2 operator front-end (dihydrogen_amd/host/include/h2) over libh2x.so:
+// typed and type-erased calls against the CPU oracle (reference metric
+// max(|d/v1|, |d/v2|) <= 1e-5, legacy/tests/compare_binary_files.cpp:47-49),
+// strided views against contiguous tensors, halo pack/unpack bit-exact, and the
+// errors of the dispatch registry (tests of the same shape as
+// test/unit_test/core/unit_test_dispatch.cpp and tensor/unit_test_fill.cpp).
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <random>
+#include <vector>
+
+#include "h2/ops_mi355x.hpp"
+
+extern "C" {
+void orc_bn_channel_sums_and_sqsums_f32(int, int, size_t, size_t, const float*, float*, float*);
+void orc_bn_sums_to_statistics_f32(int, size_t, float, float*, float*, float*, float*);
+void orc_bn_batch_normalization_f32(int, int, size_t, size_t, size_t, const float*, const float*,
+                                    const float*, const float*, const float*, float*, float);
+void orc_bn_backprop1_f32(int, int, size_t, size_t, size_t, const float*, const float*, const float*,
+                          const float*, const float*, float*, float*, float*, float*, float);
+void orc_bn_backprop2_f32(int, int, size_t, size_t, size_t, size_t, size_t, const float*, const float*,
+                          const float*, const float*, const float*, const float*, const float*, float*,
+                          float);
+void orc_softmax_channel_forward_f32(int, int, size_t, const float*, float*);
+void orc_softmax_channel_backward_f32(int, int, size_t, const float*, const float*, float*);
+}
+
+using namespace h2;
+
+#define CHECK(cond)                                                                                \
+    do                                                                                             \
+    {                                                                                              \
+        if (!(cond))                                                                               \
+        {                                                                                          \
+            std::printf("FAILED %s at %s:%d\n", #cond, __FILE__, __LINE__);                        \
+            std::exit(1);                                                                          \
+        }                                                                                          \
+    } while (0)
+
+#define CHECK_THROWS(stmt)                                                                         \
+    do                                                                                             \
+    {                                                                                              \
+        bool thrown = false;                                                                       \
+        try                                                                                        \
+        {                                                                                          \
+            stmt;                                                                                  \
+        }                                                                                          \
+        catch (const H2FatalException&)                                                            \
+        {                                                                                          \
+            thrown = true;                                                                         \
+        }                                                                                          \
+        if (!thrown)                                                                               \
+        {                                                                                          \
+            std::printf("FAILED: no exception from %s at %s:%d\n", #stmt, __FILE__, __LINE__);     \
+            std::exit(1);                                                                          \
+        }                                                                                          \
+    } while (0)
+
+template <typename T>
+static void upload(Tensor<T>& t, const std::vector<T>& h)
+{
+    CHECK(t.is_contiguous() && static_cast<size_t>(t.numel()) == h.size());
+    check_hip(hipMemcpy(t.data(), h.data(), h.size() * sizeof(T), hipMemcpyHostToDevice), "upload");
+}
+
+template <typename T>
+static std::vector<T> download(const Tensor<T>& t)
+{
+    CHECK(t.is_contiguous());
+    std::vector<T> h(t.numel());
+    check_hip(hipDeviceSynchronize(), "sync");
+    check_hip(hipMemcpy(h.data(), t.const_data(), h.size() * sizeof(T), hipMemcpyDeviceToHost),
+              "download");
+    return h;
+}
+
+static double max_rel(const std::vector<float>& a, const std::vector<float>& b)
+{
+    CHECK(a.size() == b.size());
+    double m = 0;
+    for (size_t i = 0; i < a.size(); ++i)
+    {
+        const double d = std::fabs((double) a[i] - (double) b[i]);
+        if (d == 0)
+            continue;
+        m = std::max(m, std::max(d / std::fabs((double) a[i]), d / std::fabs((double) b[i])));
+    }
+    return m;
+}
+
+static std::vector<float> randn(size_t n, unsigned seed, float sigma = 1.0f, float mu = 0.0f)
+{
+    std::mt19937 gen(seed);
+    std::normal_distribution<float> d(mu, sigma);
+    std::vector<float> v(n);
+    for (auto& x : v)
+        x = d(gen);
+    return v;
+}
+
+static DTTuple channel_types(int nd)
+{
+    DTTuple t;
+    for (int i = 0; i < nd - 2; ++i)
+        t.append(DT::Spatial);
+    t.append(DT::Channel);
+    t.append(DT::Sample);
+    return t;
+}
+
+// Batch norm forward + backward through the type-erased operators.
+static void test_batchnorm(const ShapeTuple& shape)
+{
+    const int nd = shape.size();
+    const int C = shape[nd - 2], N = shape[nd - 1];
+    const size_t total = product<size_t>(shape), S = total / C / N;
+    const ComputeStream stream(Device::GPU);
+    const DTTuple types = channel_types(nd);
+    Tensor<float> x(Device::GPU, shape, types, stream), y(Device::GPU, shape, types, stream),
+        dy(Device::GPU, shape, types, stream), dx(Device::GPU, shape, types, stream);
+    const ShapeTuple cshape{C};
+    const DTTuple ctypes{DT::Channel};
+    auto cvec = [&] { return Tensor<float>(Device::GPU, cshape, ctypes, stream); };
+    Tensor<float> mean = cvec(), var = cvec(), rm = cvec(), rv = cvec(), scale = cvec(), bias = cvec(),
+                  dscale = cvec(), dbias = cvec(), dmean = cvec(), dvar = cvec();
+    const std::vector<float> hx = randn(total, 1, 1.0f, 0.3f), hdy = randn(total, 2);
+    std::vector<float> hscale(C), hbias(C);
+    for (int c = 0; c < C; ++c)
+    {
+        hscale[c] = 0.5f + 0.01f * c;
+        hbias[c] = 0.1f * std::sin((float) c);
+    }
+    upload(x, hx);
+    upload(dy, hdy);
+    upload(scale, hscale);
+    upload(bias, hbias);
+    upload(rm, std::vector<float>(C, 0.0f));
+    upload(rv, std::vector<float>(C, 1.0f));
+
+    BaseTensor &bx = x, &by = y, &bdy = dy, &bdx = dx, &bmean = mean, &bvar = var, &brm = rm, &brv = rv,
+               &bscale = scale, &bbias = bias, &bdscale = dscale, &bdbias = dbias, &bdmean = dmean,
+               &bdvar = dvar;
+    const size_t n = (size_t) N * S;
+    batchnorm_channel_sums(bx, bmean, bvar);
+    batchnorm_statistics(bmean, bvar, brm, brv, n, 0.9);
+    batchnorm_normalize(bx, bmean, bvar, bscale, bbias, by, 1e-5);
+    batchnorm_backprop1(bx, bdy, bmean, bvar, bscale, bdscale, bdbias, bdmean, bdvar, 1e-5);
+    batchnorm_backprop2(bx, bdy, bmean, bvar, bscale, bdmean, bdvar, bdx, n, 1e-5);
+
+    std::vector<float> om(C), ov(C), orm(C, 0.0f), orv(C, 1.0f), oy(total), ods(C), odb(C), odm(C),
+        odv(C), odx(total);
+    orc_bn_channel_sums_and_sqsums_f32(N, C, S, S, hx.data(), om.data(), ov.data());
+    orc_bn_sums_to_statistics_f32(C, n, 0.9f, om.data(), ov.data(), orm.data(), orv.data());
+    orc_bn_batch_normalization_f32(N, C, S, S, S, hx.data(), om.data(), ov.data(), hscale.data(),
+                                   hbias.data(), oy.data(), 1e-5f);
+    orc_bn_backprop1_f32(N, C, S, S, S, hx.data(), hdy.data(), om.data(), ov.data(), hscale.data(),
+                         ods.data(), odb.data(), odm.data(), odv.data(), 1e-5f);
+    orc_bn_backprop2_f32(N, C, S, S, S, S, n, hx.data(), hdy.data(), om.data(), ov.data(),
+                         hscale.data(), odm.data(), odv.data(), odx.data(), 1e-5f);
+    CHECK(max_rel(download(mean), om) <= 1e-5);
+    CHECK(max_rel(download(var), ov) <= 1e-5);
+    CHECK(max_rel(download(rm), orm) <= 1e-5);
+    CHECK(max_rel(download(rv), orv) <= 1e-5);
+    CHECK(max_rel(download(y), oy) <= 1e-5);
+    CHECK(max_rel(download(dscale), ods) <= 1e-5);
+    CHECK(max_rel(download(dbias), odb) <= 1e-5);
+    CHECK(max_rel(download(dmean), odm) <= 1e-5);
+    CHECK(max_rel(download(dvar), odv) <= 1e-5);
+    CHECK(max_rel(download(dx), odx) <= 1e-5);
+
+    // the typed front gives the same bits as the type-erased one
+    Tensor<float> y2(Device::GPU, shape, types, stream);
+    batchnorm_normalize(x, mean, var, scale, bias, y2, 1e-5);
+    CHECK(download(y2) == download(y));
+}
+
+// A view with padded rows (stride of dimension 1 larger than the extent of
+// dimension 0) gives what the contiguous tensor gives on the same elements.
+static void test_strided_view()
+{
+    const int W = 12, H = 5, C = 6, N = 3, pitch = 16;
+    const ShapeTuple shape{W, H, C, N};
+    const DTTuple types = channel_types(4);
+    const ComputeStream stream(Device::GPU);
+    const StrideTuple padded{1, pitch, (DataIndexType) pitch * H, (DataIndexType) pitch * H * C};
+    const size_t total = (size_t) W * H * C * N, padded_total = (size_t) pitch * H * C * N;
+    const std::vector<float> hx = randn(total, 7, 2.0f, -1.0f);
+    std::vector<float> hp(padded_total, 1e30f); // the padding must never be read
+    for (size_t i = 0; i < total; ++i)
+    {
+        const size_t w = i % W, rest = i / W;
+        hp[rest * pitch + w] = hx[i];
+    }
+    Tensor<float> x(Device::GPU, shape, types, stream);
+    upload(x, hx);
+    float* raw = nullptr;
+    check_hip(hipMalloc(&raw, padded_total * sizeof(float)), "hipMalloc");
+    check_hip(hipMemcpy(raw, hp.data(), padded_total * sizeof(float), hipMemcpyHostToDevice), "copy");
+    Tensor<float> view(Device::GPU, raw, shape, types, padded, stream);
+    CHECK(!view.is_contiguous() && view.is_view());
+    const ShapeTuple cshape{C};
+    const DTTuple ctypes{DT::Channel};
+    Tensor<float> s1(Device::GPU, cshape, ctypes, stream), q1(Device::GPU, cshape, ctypes, stream),
+        s2(Device::GPU, cshape, ctypes, stream), q2(Device::GPU, cshape, ctypes, stream);
+    batchnorm_channel_sums(x, s1, q1);
+    batchnorm_channel_sums(view, s2, q2);
+    CHECK(max_rel(download(s1), download(s2)) <= 1e-6);
+    CHECK(max_rel(download(q1), download(q2)) <= 1e-6);
+    check_hip(hipDeviceSynchronize(), "sync");
+    check_hip(hipFree(raw), "hipFree");
+}
+
+static void test_softmax()
+{
+    const ShapeTuple shape{16, 8, 21, 2};
+    const DTTuple types = channel_types(4);
+    const ComputeStream stream(Device::GPU);
+    const size_t total = product<size_t>(shape), S = 16 * 8;
+    Tensor<float> x(Device::GPU, shape, types, stream), y(Device::GPU, shape, types, stream),
+        dy(Device::GPU, shape, types, stream), dx(Device::GPU, shape, types, stream);
+    const std::vector<float> hx = randn(total, 3, 2.0f), hdy = randn(total, 4);
+    upload(x, hx);
+    upload(dy, hdy);
+    BaseTensor &bx = x, &by = y, &bdy = dy, &bdx = dx;
+    softmax_channel_forward(bx, by);
+    softmax_channel_backward(by, bdy, bdx);
+    std::vector<float> oy(total), odx(total);
+    orc_softmax_channel_forward_f32(2, 21, S, hx.data(), oy.data());
+    orc_softmax_channel_backward_f32(2, 21, S, oy.data(), hdy.data(), odx.data());
+    CHECK(max_rel(download(y), oy) <= 1e-5);
+    CHECK(max_rel(download(dx), odx) <= 1e-5);
+}
+
+// Pack the RHS interior strip of one tensor, unpack it into the LHS halo of
+// another: the halo then holds the neighbour's boundary values, bit for bit.
+static void test_halo()
+{
+    const ShapeTuple shape{10, 6, 3, 2}; // 8 interior columns + one halo column on each side
+    const DTTuple types = channel_types(4);
+    const ComputeStream stream(Device::GPU);
+    const size_t total = product<size_t>(shape);
+    std::vector<double> ha(total), hb(total, -1.0);
+    for (size_t i = 0; i < total; ++i)
+        ha[i] = 0.5 * (double) i;
+    Tensor<double> a(Device::GPU, shape, types, stream), b(Device::GPU, shape, types, stream);
+    upload(a, ha);
+    upload(b, hb);
+    Tensor<double> buf(Device::GPU, ShapeTuple{6 * 3 * 2}, DTTuple{DT::Any}, stream);
+    BaseTensor &ba = a, &bb = b, &bbuf = buf;
+    halo_pack(ba, 0, H2X_RHS, 1, bbuf);
+    halo_unpack(bb, 0, H2X_LHS, 1, bbuf);
+    const std::vector<double> got = download(b);
+    for (size_t row = 0; row < total / 10; ++row)
+        for (int w = 0; w < 10; ++w)
+            CHECK(got[row * 10 + w] == (w == 0 ? ha[row * 10 + 8] : -1.0));
+    // SUM unpack of the reverse direction adds the neighbour's halo onto the boundary cells
+    halo_pack(ba, 0, H2X_RHS, 1, bbuf, true);           // a's RHS halo column (w = 9)
+    halo_unpack(bb, 0, H2X_LHS, 1, bbuf, true, H2X_HALO_SUM); // onto b's first interior column (w = 1)
+    const std::vector<double> sum = download(b);
+    for (size_t row = 0; row < total / 10; ++row)
+        CHECK(sum[row * 10 + 1] == -1.0 + ha[row * 10 + 9]);
+}
+
+static void test_errors()
+{
+    const ComputeStream stream(Device::GPU);
+    const ShapeTuple shape{8, 4, 3, 2};
+    Tensor<float> x(Device::GPU, shape, channel_types(4), stream);
+    Tensor<float> s(Device::GPU, ShapeTuple{3}, DTTuple{DT::Channel}, stream),
+        q(Device::GPU, ShapeTuple{3}, DTTuple{DT::Channel}, stream);
+    // dimension tags decide the layout: a tensor tagged differently is rejected
+    Tensor<float> wrong(Device::GPU, shape, DTTuple{DT::Spatial, DT::Channel, DT::Spatial, DT::Sample},
+                        stream);
+    CHECK_THROWS(batchnorm_channel_sums(wrong, s, q));
+    // per-channel vectors of the wrong length
+    Tensor<float> s4(Device::GPU, ShapeTuple{4}, DTTuple{DT::Channel}, stream);
+    CHECK_THROWS(batchnorm_channel_sums(x, s4, q));
+    // no CPU implementation
+    Tensor<float> cx(Device::CPU, shape, channel_types(4)), cs(Device::CPU, ShapeTuple{3}, DTTuple{DT::Channel}),
+        cq(Device::CPU, ShapeTuple{3}, DTTuple{DT::Channel});
+    CHECK_THROWS(batchnorm_channel_sums(cx, cs, cq));
+    // an element type nobody registered
+    Tensor<std::int32_t> ix(Device::GPU, shape, channel_types(4), stream),
+        is(Device::GPU, ShapeTuple{3}, DTTuple{DT::Channel}, stream),
+        iq(Device::GPU, ShapeTuple{3}, DTTuple{DT::Channel}, stream);
+    BaseTensor &bix = ix, &bis = is, &biq = iq;
+    CHECK_THROWS(batchnorm_channel_sums(bix, bis, biq));
+    // mixed element types
+    Tensor<double> ds(Device::GPU, ShapeTuple{3}, DTTuple{DT::Channel}, stream);
+    BaseTensor &bx = x, &bds = ds, &bq = q;
+    CHECK_THROWS(batchnorm_channel_sums(bx, bds, bq));
+    // registry: register, call, unregister
+    static int calls = 0;
+    struct Probe
+    {
+        static void fn(const BaseTensor&, int v) { calls += v; }
+    };
+    const auto key = get_dispatch_key(x);
+    CHECK(key == get_dispatch_key(get_h2_type<float>()));
+    CHECK(key != get_dispatch_key(get_h2_type<double>()));
+    dispatch_register("probe_gpu", key, &Probe::fn);
+    CHECK(internal::has_dispatch_entry("probe_gpu", key));
+    const BaseTensor& cbx = x;
+    int five = 5;
+    internal::call_dispatch_entry("probe_gpu", key, cbx, five);
+    CHECK(calls == 5);
+    dispatch_unregister("probe_gpu", key);
+    CHECK(!internal::has_dispatch_entry("probe_gpu", key));
+    CHECK_THROWS(internal::call_dispatch_entry("probe_gpu", key, cbx, five));
+}
+
+int main()
+{
+    test_batchnorm(ShapeTuple{14, 14, 8, 4});
+    test_batchnorm(ShapeTuple{6, 5, 7, 3, 2});
+    test_batchnorm(ShapeTuple{33, 5, 2}); // one spatial dimension, odd length
+    test_strided_view();
+    test_softmax();
+    test_halo();
+    test_errors();
+    std::printf("test_h2_frontend: ok\n");
+    return 0;
+}
