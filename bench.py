@@ -166,7 +166,7 @@ class ShuffleWorkload:
         self.sh.shuffle_backward()
 
 
-def cpu_baseline(repeats: int = 3):
+def cpu_baseline(repeats: int = 9):
     """The CPU oracle (this repository's restatement of the reference kernels;
     the reference has no CPU implementation of batch-norm, softmax or halo
     packing) on the same step: config 3 batch-norm forward+backward plus the
