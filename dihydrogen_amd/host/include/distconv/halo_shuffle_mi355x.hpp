@@ -326,10 +326,11 @@ public:
                         HaloExchangeAccumOp op)
     {
         const h2x_dtype dt = TensorType::h2x_type();
-        for (const std::vector<int>& group : rank_groups(dim, std::max(width_rhs, width_lhs)))
+        // all ranks in one launch: nothing is read back between launches here,
+        // so rank groups would only add launches
         {
             std::vector<h2x_halo_transfer> moves;
-            for (int member : group)
+            for (int member = 0; member < num_ranks(); ++member)
             {
                 auto& r = m_ranks[member]; // the receiver
                 if (!r->is_exchange_required(dim, width_rhs, width_rhs, width_lhs, width_lhs))

@@ -82,10 +82,12 @@ def test_config4_softmax(oracle_mod):
     assert max_rel(dxt.real_view().cpu().numpy(), oracle_mod.softmax_channel_backward(y, dy)) <= TOL
 
 
-def test_config2_halo_closed_form():
+@pytest.mark.parametrize("fused", [False, True])
+def test_config2_halo_closed_form(fused):
     """8 virtual ranks, N1 C32 128^3 each, periodic 2x2x2, width 1: after the
     exchange every cell of every real tensor, halo faces, edges and corners
-    included, equals the value of its periodic source coordinate."""
+    included, equals the value of its periodic source coordinate.  Once through
+    pack + unpack, once as tensor-to-tensor transfers."""
     import torch
     from dihydrogen_amd.layers import HaloExchangeVirtual
     from dihydrogen_amd.tensor import Distribution, LocaleVirtual, Tensor
@@ -111,7 +113,7 @@ def test_config2_halo_closed_form():
     for t in ranks:
         t.real_view().fill_(float("nan"))
         t.interior_view().copy_(field(t, False))
-    HaloExchangeVirtual(ranks, periodic=True).exchange()
+    HaloExchangeVirtual(ranks, periodic=True).exchange(fused=fused)
     torch.cuda.synchronize()
     for t in ranks:
         assert torch.equal(t.real_view(), field(t, True))
