@@ -55,6 +55,25 @@ def _time_events(fn, iters: int, warmup: int, inner: int = 4):
     return statistics.median(times), min(times)
 
 
+def _time_events_cold(fn, flush, iters: int, warmup: int):
+    """As _time_events, but every timed call starts with caches that hold
+    nothing of its working set: `flush` (a read of a buffer larger than the
+    256 MB memory-side cache) runs before each one, outside the event pair."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    times = []
+    for _ in range(iters):
+        flush()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        fn()
+        e1.record()
+        e1.synchronize()
+        times.append(e0.elapsed_time(e1))
+    return statistics.median(times), min(times)
+
+
 class BatchNormWorkload:
     """BatchNormalization forward + backward on one rank."""
 
@@ -407,14 +426,23 @@ def main() -> int:
             2 * S3 * 4, S3, *_time_events(lambda: yard_y.copy_(yard_x), it, wu))
         del bn3, halo, b, yard_x, yard_y
         torch.cuda.empty_cache()
+        # configs 1 and 4 fit in the memory-side cache: warm = back to back, cold = after a 512 MB read
+        evict = torch.empty(1 << 27, device="cuda").fill_(1.0)
+        flush = lambda: evict.sum()
         bn1 = BatchNormWorkload((8, 64, 56, 56), SEED + 1)
         breakdown["C1_bn2d_fwd_warm"] = entry(3 * bn1.elems * 4, bn1.elems, *_time_events(bn1.forward, it, wu))
+        breakdown["C1_bn2d_fwd_cold"] = entry(3 * bn1.elems * 4, bn1.elems,
+                                              *_time_events_cold(bn1.forward, flush, it, wu))
         del bn1
         sm = SoftmaxWorkload((16, 21, 256, 256), SEED + 4)
         sm.forward()
         breakdown["C4_softmax_fwd"] = entry(2 * sm.elems * 4, sm.elems, *_time_events(sm.forward, it, wu))
         breakdown["C4_softmax_bwd"] = entry(3 * sm.elems * 4, sm.elems, *_time_events(sm.backward, it, wu))
-        del sm
+        breakdown["C4_softmax_fwd_cold"] = entry(2 * sm.elems * 4, sm.elems,
+                                                 *_time_events_cold(sm.forward, flush, it, wu))
+        breakdown["C4_softmax_bwd_cold"] = entry(3 * sm.elems * 4, sm.elems,
+                                                 *_time_events_cold(sm.backward, flush, it, wu))
+        del sm, evict
         shf = ShuffleWorkload((128, 128, 64, 32), SEED + 5)
         breakdown["C5_shuffle_fwd"] = entry(4 * shf.elems * 4, shf.elems, *_time_events(shf.forward, it, wu))
         breakdown["C5_shuffle_bwd"] = entry(4 * shf.elems * 4, shf.elems, *_time_events(shf.backward, it, wu))
