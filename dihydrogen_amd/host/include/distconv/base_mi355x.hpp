@@ -87,6 +87,27 @@ inline void check_hip(hipError_t e, const char* file, int line)
     }
 }
 
+// `later` continues only after the work queued on `earlier` so far
+// (util::wait_stream, legacy/include/distconv/util/util_rocm.hpp).  The event
+// is released as soon as the wait is queued; the runtime keeps it alive until
+// it has fired.
+inline void wait_stream(hipStream_t earlier, hipStream_t later)
+{
+    if (earlier == later)
+        return;
+    hipEvent_t ev;
+    check_hip(hipEventCreateWithFlags(&ev, hipEventDisableTiming), __FILE__, __LINE__);
+    check_hip(hipEventRecord(ev, earlier), __FILE__, __LINE__);
+    check_hip(hipStreamWaitEvent(later, ev, 0), __FILE__, __LINE__);
+    check_hip(hipEventDestroy(ev), __FILE__, __LINE__);
+}
+
+inline void wait_stream(hipStream_t earlier, const hipStream_t* later, int num_streams)
+{
+    for (int i = 0; i < num_streams; ++i)
+        wait_stream(earlier, later[i]);
+}
+
 } // namespace util
 
 #define assert_always(cond)                                                                        \

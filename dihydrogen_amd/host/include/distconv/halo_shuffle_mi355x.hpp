@@ -111,6 +111,47 @@ public:
                           bool rendezvous, bool is_reverse, bool skip_unpack,
                           HaloExchangeAccumOp op = HaloExchangeAccumOp::ID) = 0;
 
+    // All dimensions, innermost first (halo_exchange_cuda.hpp:56-106): the two
+    // boundary streams of a dimension wait for the streams the previous
+    // exchanged dimension ran on (the main stream for the first), and with
+    // `sync_back` the main stream waits for the last ones.  `streams(dim, side)`
+    // stands for the stream of the reference's per-boundary communicator.
+    virtual void exchange(const IntVector& widths_rhs_send, const IntVector& widths_rhs_recv,
+                          const IntVector& widths_lhs_send, const IntVector& widths_lhs_recv,
+                          BoundaryAttributesV<hipStream_t>& streams, hipStream_t stream_main,
+                          bool rendezvous, bool sync_back, bool is_reverse, bool skip_unpack,
+                          HaloExchangeAccumOp op = HaloExchangeAccumOp::ID)
+    {
+        hipStream_t prev_streams[2] = {stream_main, stream_main};
+        for (int i = 0; i < m_tensor.get_num_dims(); ++i)
+        {
+            if (!is_exchange_required(i, widths_rhs_send[i], widths_rhs_recv[i], widths_lhs_send[i],
+                                      widths_lhs_recv[i]))
+                continue;
+            for (Side side : SIDES)
+            {
+                const hipStream_t cur_streams[2] = {streams(i, RHS), streams(i, LHS)};
+                util::wait_stream(prev_streams[side], cur_streams, 2);
+                prev_streams[side] = streams(i, side);
+            }
+            exchange(i, widths_rhs_send[i], widths_rhs_recv[i], widths_lhs_send[i],
+                     widths_lhs_recv[i], streams(i, RHS), streams(i, LHS), rendezvous, is_reverse,
+                     skip_unpack, op);
+        }
+        if (sync_back)
+            for (Side side : SIDES)
+                util::wait_stream(prev_streams[side], stream_main);
+    }
+
+    // halo_exchange_cuda.hpp:107-125: the tensor's own halo widths
+    virtual void exchange(BoundaryAttributesV<hipStream_t>& streams, hipStream_t stream_main,
+                          bool rendezvous, bool sync_back, bool is_reverse, bool skip_unpack,
+                          HaloExchangeAccumOp op = HaloExchangeAccumOp::ID)
+    {
+        const IntVector& w = m_tensor.get_halo_width();
+        exchange(w, w, w, w, streams, stream_main, rendezvous, sync_back, is_reverse, skip_unpack, op);
+    }
+
     TensorType& get_tensor() { return m_tensor; }
     int get_peer(int dim, Side side) const { return m_peers(dim, side); }
 
@@ -267,6 +308,41 @@ public:
     {
         const IntVector& w = m_ranks[0]->get_tensor().get_halo_width();
         exchange(w, w, w, w, stream, is_reverse, skip_unpack, op);
+    }
+
+    // The reference's driver signature (halo_exchange_cuda.hpp:56-82) for the
+    // whole group: boundary streams are fenced dimension after dimension as
+    // there; both sides of a dimension share launches here, which go to the
+    // RHS boundary stream.
+    void exchange(const IntVector& widths_rhs_send, const IntVector& widths_rhs_recv,
+                  const IntVector& widths_lhs_send, const IntVector& widths_lhs_recv,
+                  BoundaryAttributesV<hipStream_t>& streams, hipStream_t stream_main,
+                  bool /*rendezvous*/, bool sync_back, bool is_reverse, bool skip_unpack,
+                  HaloExchangeAccumOp op = HaloExchangeAccumOp::ID)
+    {
+        hipStream_t prev_streams[2] = {stream_main, stream_main};
+        const int nd = m_ranks[0]->get_tensor().get_num_dims();
+        for (int i = 0; i < nd; ++i)
+        {
+            bool required = false;
+            for (auto& r : m_ranks)
+                required = required
+                           || r->is_exchange_required(i, widths_rhs_send[i], widths_rhs_recv[i],
+                                                      widths_lhs_send[i], widths_lhs_recv[i]);
+            if (!required)
+                continue;
+            for (Side side : SIDES)
+            {
+                const hipStream_t cur_streams[2] = {streams(i, RHS), streams(i, LHS)};
+                util::wait_stream(prev_streams[side], cur_streams, 2);
+                prev_streams[side] = streams(i, side);
+            }
+            exchange(i, widths_rhs_send[i], widths_rhs_recv[i], widths_lhs_send[i],
+                     widths_lhs_recv[i], streams(i, RHS), is_reverse, skip_unpack, op);
+        }
+        if (sync_back)
+            for (Side side : SIDES)
+                util::wait_stream(prev_streams[side], stream_main);
     }
 
     void exchange(int dim, int wrs, int wrr, int wls, int wlr, hipStream_t stream, bool is_reverse,
@@ -428,6 +504,7 @@ private:
     struct Member : public Rank
     {
         using Rank::Rank;
+        using Rank::exchange;
         void exchange(int, int, int, int, int, hipStream_t, hipStream_t, bool, bool, bool,
                       HaloExchangeAccumOp) override
         {

@@ -4,8 +4,15 @@
 // global offset of its source.
 #include "test_common.hpp"
 
+enum Mode
+{
+    kBuffers,        // pack, unpack through receive buffers, one stream
+    kFused,          // tensor-to-tensor transfers
+    kBoundaryStreams // the reference's driver signature with two boundary streams per dimension
+};
+
 static int run_case(const Shape& shape, const Shape& locale, const IntVector& overlap, bool periodic,
-                    bool fused = false)
+                    Mode mode = kBuffers)
 {
     const int nd = shape.length();
     const int n = static_cast<int>(locale.get_size());
@@ -23,10 +30,31 @@ static int run_case(const Shape& shape, const Shape& locale, const IntVector& ov
     for (int d = 0; d < nd; ++d) // Convolution clears the halo before every exchange
         for (auto* t : ptrs)
             t->clear_halo(d, nullptr);
-    if (fused)
+    if (mode == kFused)
+    {
         xch.exchange_fused(nullptr);
+    }
+    else if (mode == kBoundaryStreams)
+    {
+        hipStream_t main_stream;
+        DISTCONV_CHECK_HIP(hipStreamCreate(&main_stream));
+        BoundaryAttributesV<hipStream_t> streams(nd);
+        for (int d = 0; d < nd; ++d)
+            for (Side side : SIDES)
+                DISTCONV_CHECK_HIP(hipStreamCreate(&streams(d, side)));
+        DISTCONV_CHECK_HIP(hipDeviceSynchronize()); // the fields were written on the null stream
+        const IntVector& w = ranks[0]->get_halo_width();
+        xch.exchange(w, w, w, w, streams, main_stream, false, true, false, false);
+        DISTCONV_CHECK_HIP(hipStreamSynchronize(main_stream)); // sync_back: main waits for the boundaries
+        for (int d = 0; d < nd; ++d)
+            for (Side side : SIDES)
+                DISTCONV_CHECK_HIP(hipStreamDestroy(streams(d, side)));
+        DISTCONV_CHECK_HIP(hipStreamDestroy(main_stream));
+    }
     else
+    {
         xch.exchange(nullptr);
+    }
     int errors = 0;
     for (int r = 0; r < n; ++r)
     {
@@ -71,8 +99,10 @@ int main()
         errors += run_case(Shape({8, 10, 12, 3, 2}), Shape({2, 2, 2, 1, 1}), IntVector({1, 1, 1, 0, 0}), periodic);
         errors += run_case(Shape({8, 9, 10, 2, 1}), Shape({1, 2, 2, 1, 1}), IntVector({0, 2, 1, 0, 0}), periodic);
         // tensor-to-tensor transfers instead of pack + unpack
-        errors += run_case(Shape({13, 11, 3, 2}), Shape({3, 2, 1, 1}), IntVector({1, 2, 0, 0}), periodic, true);
-        errors += run_case(Shape({8, 10, 12, 3, 2}), Shape({2, 2, 2, 1, 1}), IntVector({1, 1, 1, 0, 0}), periodic, true);
+        errors += run_case(Shape({13, 11, 3, 2}), Shape({3, 2, 1, 1}), IntVector({1, 2, 0, 0}), periodic, kFused);
+        errors += run_case(Shape({8, 10, 12, 3, 2}), Shape({2, 2, 2, 1, 1}), IntVector({1, 1, 1, 0, 0}), periodic, kFused);
+        errors += run_case(Shape({8, 10, 12, 3, 2}), Shape({2, 2, 2, 1, 1}), IntVector({1, 1, 1, 0, 0}), periodic,
+                           kBoundaryStreams);
     }
     // per-rank interface: pack one strip, unpack it on the neighbour
     {
