@@ -4,50 +4,51 @@
 // global offset; shuffle_backward restores the source.
 #include "test_common.hpp"
 
+template <typename T = float>
 static int run_case(const Shape& shape, const Distribution& sd, const Distribution& dd)
 {
     const int n = static_cast<int>(sd.get_locale_shape().get_size());
-    std::vector<std::unique_ptr<DevTensor<float>>> own;
-    std::vector<DevTensor<float>*> src, dst;
+    std::vector<std::unique_ptr<DevTensor<T>>> own;
+    std::vector<DevTensor<T>*> src, dst;
     for (int r = 0; r < n; ++r)
     {
-        own.emplace_back(new DevTensor<float>(shape, LocaleVirtual(r, n), sd));
+        own.emplace_back(new DevTensor<T>(shape, LocaleVirtual(r, n), sd));
         src.push_back(own.back().get());
-        own.emplace_back(new DevTensor<float>(shape, LocaleVirtual(r, n), dd));
+        own.emplace_back(new DevTensor<T>(shape, LocaleVirtual(r, n), dd));
         dst.push_back(own.back().get());
         src[r]->allocate();
         dst[r]->allocate();
-        to_device(*src[r], global_offset_field(*src[r], -1.0f));
-        to_device(*dst[r], std::vector<float>(dst[r]->get_local_real_size(), -7.0f));
+        to_device(*src[r], global_offset_field(*src[r], static_cast<T>(-1)));
+        to_device(*dst[r], std::vector<T>(dst[r]->get_local_real_size(), static_cast<T>(-7)));
     }
-    TensorShufflerVirtual<float> sh(src, dst);
+    TensorShufflerVirtual<T> sh(src, dst);
     sh.shuffle_forward();
     int errors = 0;
     for (int r = 0; r < n; ++r)
     {
-        std::vector<float> want = dst[r]->is_split_root() ? global_offset_field(*dst[r], -7.0f)
-                                                          : std::vector<float>(dst[r]->get_local_real_size(), -7.0f);
-        std::vector<float> got = to_host(*dst[r]);
+        std::vector<T> want = dst[r]->is_split_root() ? global_offset_field(*dst[r], static_cast<T>(-7))
+                                                          : std::vector<T>(dst[r]->get_local_real_size(), static_cast<T>(-7));
+        std::vector<T> got = to_host(*dst[r]);
         for (size_t i = 0; i < got.size(); ++i)
             errors += got[i] != want[i];
     }
-    std::vector<std::vector<float>> keep;
+    std::vector<std::vector<T>> keep;
     for (int r = 0; r < n; ++r)
     {
         keep.push_back(to_host(*src[r]));
         if (src[r]->is_split_root()) // interior is rewritten by the backward shuffle
         {
-            std::vector<float> h = keep.back();
+            std::vector<T> h = keep.back();
             const Shape& ls = src[r]->get_local_shape();
             for (index_t o = 0; o < src[r]->get_local_size(); ++o)
-                h[src[r]->get_local_offset(ls.get_index(o))] = -3.0f;
+                h[src[r]->get_local_offset(ls.get_index(o))] = static_cast<T>(-3);
             to_device(*src[r], h);
         }
     }
     sh.shuffle_backward();
     for (int r = 0; r < n; ++r)
     {
-        std::vector<float> got = to_host(*src[r]);
+        std::vector<T> got = to_host(*src[r]);
         for (size_t i = 0; i < got.size(); ++i)
             errors += got[i] != keep[r][i];
     }
@@ -77,6 +78,23 @@ int main()
     // shrink the spatial split (shared distribution)
     errors += run_case(s4, Distribution::make_distribution(Shape({2, 2, 1, 1})),
                        Distribution::make_shared_distribution(Shape({2, 2, 1, 1}), Shape({2, 1, 1, 1})));
+    // the other element types the reference instantiates (shuffle_mpi_cuda.cu:492-499): 2, 4 and 8 bytes
+    errors += run_case<short>(s4, Distribution::make_distribution(Shape({1, 1, 1, 4})),
+                              Distribution::make_distribution(Shape({2, 2, 1, 1})));
+    errors += run_case<unsigned short>(s4, Distribution::make_distribution(Shape({1, 1, 1, 4})),
+                                       Distribution::make_overlapped_distribution(Shape({2, 2, 1, 1}),
+                                                                                  IntVector({1, 1, 0, 0})));
+    errors += run_case<int>(Shape({11, 7, 3, 5}), Distribution::make_distribution(Shape({1, 1, 1, 4})),
+                            Distribution::make_distribution(Shape({2, 2, 1, 1})));
+    errors += run_case<unsigned>(s4, Distribution::make_distribution(Shape({2, 2, 1, 1})),
+                                 Distribution::make_distribution(Shape({1, 1, 1, 4})));
+    errors += run_case<long>(s4, Distribution::make_distribution(Shape({1, 1, 1, 4})),
+                             Distribution::make_distribution(Shape({2, 2, 1, 1})));
+    errors += run_case<unsigned long>(Shape({11, 7, 3, 5}), Distribution::make_distribution(Shape({1, 1, 1, 4})),
+                                      Distribution::make_distribution(Shape({2, 2, 1, 1})));
+    errors += run_case<double>(s4, Distribution::make_distribution(Shape({1, 1, 1, 4})),
+                               Distribution::make_overlapped_distribution(Shape({2, 2, 1, 1}),
+                                                                          IntVector({1, 1, 0, 0})));
     // 5-D
     errors += run_case(Shape({6, 8, 4, 2, 4}), Distribution::make_distribution(Shape({1, 1, 1, 1, 4})),
                        Distribution::make_overlapped_distribution(Shape({1, 2, 2, 1, 1}), IntVector({0, 1, 1, 0, 0})));
