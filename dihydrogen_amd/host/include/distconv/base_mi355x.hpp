@@ -108,6 +108,59 @@ inline void wait_stream(hipStream_t earlier, const hipStream_t* later, int num_s
         wait_stream(earlier, later[i]);
 }
 
+// Each stream continues only after the work queued on the other so far
+// (util::sync_stream, legacy/src/util/util_rocm.cpp:164-175).
+inline void sync_stream(hipStream_t s1, hipStream_t s2)
+{
+    if (s1 == s2)
+        return;
+    hipEvent_t ev1, ev2;
+    check_hip(hipEventCreateWithFlags(&ev1, hipEventDisableTiming), __FILE__, __LINE__);
+    check_hip(hipEventCreateWithFlags(&ev2, hipEventDisableTiming), __FILE__, __LINE__);
+    check_hip(hipEventRecord(ev1, s1), __FILE__, __LINE__);
+    check_hip(hipEventRecord(ev2, s2), __FILE__, __LINE__);
+    check_hip(hipStreamWaitEvent(s2, ev1, 0), __FILE__, __LINE__);
+    check_hip(hipStreamWaitEvent(s1, ev2, 0), __FILE__, __LINE__);
+    check_hip(hipEventDestroy(ev1), __FILE__, __LINE__);
+    check_hip(hipEventDestroy(ev2), __FILE__, __LINE__);
+}
+
+// Event timer on one stream (util::Clock,
+// legacy/include/distconv/util/util_rocm.hpp:110-138): start() and stop()
+// record events, get_time() waits for the second and returns milliseconds.
+struct Clock
+{
+    explicit Clock(hipStream_t s) : m_s(s)
+    {
+        check_hip(hipEventCreate(&m_ev1), __FILE__, __LINE__);
+        check_hip(hipEventCreate(&m_ev2), __FILE__, __LINE__);
+    }
+    Clock(const Clock& c) : Clock(c.m_s) {}
+    Clock& operator=(const Clock& c)
+    {
+        m_s = c.m_s;
+        return *this;
+    }
+    ~Clock()
+    {
+        (void) hipEventDestroy(m_ev2);
+        (void) hipEventDestroy(m_ev1);
+    }
+    void start() { check_hip(hipEventRecord(m_ev1, m_s), __FILE__, __LINE__); }
+    void stop() { check_hip(hipEventRecord(m_ev2, m_s), __FILE__, __LINE__); }
+    float get_time()
+    {
+        check_hip(hipEventSynchronize(m_ev2), __FILE__, __LINE__);
+        float elapsed = 0;
+        check_hip(hipEventElapsedTime(&elapsed, m_ev1, m_ev2), __FILE__, __LINE__);
+        return elapsed;
+    }
+
+    hipStream_t m_s;
+    hipEvent_t m_ev1 = nullptr;
+    hipEvent_t m_ev2 = nullptr;
+};
+
 } // namespace util
 
 #define assert_always(cond)                                                                        \

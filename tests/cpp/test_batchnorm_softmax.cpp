@@ -253,6 +253,22 @@ int main()
 {
     int errors = 0;
     errors += test_bn_haloed();
+    {
+        // util::Clock brackets work on a stream, as the reference's benchmark does
+        // (legacy/benchmarks/distconv_benchmark_bn.cpp:254-295); sync_stream orders two streams
+        hipStream_t a, b;
+        DISTCONV_CHECK_HIP(hipStreamCreate(&a));
+        DISTCONV_CHECK_HIP(hipStreamCreate(&b));
+        util::Clock clk(a);
+        clk.start();
+        util::sync_stream(a, b);
+        clk.stop();
+        const float ms = clk.get_time();
+        CHECK(ms >= 0.0f && ms < 1000.0f);
+        DISTCONV_CHECK_HIP(hipStreamSynchronize(b));
+        DISTCONV_CHECK_HIP(hipStreamDestroy(a));
+        DISTCONV_CHECK_HIP(hipStreamDestroy(b));
+    }
     errors += test_bn(Shape({56, 56, 64, 8}));   // BASELINE config 1
     errors += test_bn(Shape({5, 7, 3, 2}));
     errors += test_bn(Shape({16, 16, 16, 8, 4})); // 5-D
