@@ -266,6 +266,58 @@ KERNEL_OF = {
 }
 
 
+def dim0_study():
+    """The dimension-0 phase of the config 2 exchange (one 4-byte element per
+    520-byte row and side) as a rate of memory transactions: every packed
+    element costs the fetch of a 128-byte line (two neighbouring rows' ends
+    share one), every unpacked element a 32-byte masked write.  Timed for
+    launch groups of 2, 4 and 8 ranks, pack and unpack alone and together, and
+    for the tensor-to-tensor form."""
+    from dihydrogen_amd import capi
+    from dihydrogen_amd.layers import HaloExchangeAccumOp
+    lib = capi.load()
+    halo = HaloWorkload(128, 32, SEED + 2)
+    xch, dt = halo.xch, halo.ranks[0].h2x_dtype
+    rows = 130 * 130 * 32                      # rows of one rank
+    lines_per_rank = rows * (1 + 12 / 128)     # one line per row pair end, 12 bytes apart: 9 % straddle
+    writes_per_rank = 2 * rows
+    ident = HaloExchangeAccumOp.ID
+
+    def faces(group, is_pack):
+        out = []
+        for r in group:
+            for side in (capi.LHS, capi.RHS):
+                peer = xch.find_peer_rank(r, 0, side)
+                buf = xch._recv_buffer(peer, 0, capi.LHS if side == capi.RHS else capi.RHS) if is_pack \
+                    else xch._recv_buffer(r, 0, side)
+                out.append(xch._face(r, 0, side, 1, buf, is_pack, False, ident))
+        return (capi.HaloFace * len(out))(*out)
+
+    def launch(arr):
+        capi.check(lib.h2x_halo_pack_or_unpack_batched(dt, arr, len(arr), None), "halo")
+
+    result = {"rows_per_rank": rows, "lines_per_rank": int(lines_per_rank), "writes_per_rank": writes_per_rank,
+              "groups": {}}
+    for size in (2, 4, 8):
+        groups = [list(range(g, g + size)) for g in range(0, 8, size)]
+        packs = [faces(g, True) for g in groups]
+        unpacks = [faces(g, False) for g in groups]
+        t_pack = _time_events(lambda: [launch(a) for a in packs], 10, 3, inner=2)[0]
+        t_unpack = _time_events(lambda: [launch(a) for a in unpacks], 10, 3, inner=2)[0]
+        t_both = _time_events(lambda: [(launch(p), launch(u)) for p, u in zip(packs, unpacks)], 10, 3, inner=2)[0]
+        result["groups"][str(size)] = {
+            "pack_us": t_pack * 1e3, "unpack_us": t_unpack * 1e3, "pack_then_unpack_us": t_both * 1e3,
+            "pack_Glines_per_s": 8 * lines_per_rank / (t_pack * 1e-3) / 1e9,
+            "pack_line_traffic_GB/s": 8 * lines_per_rank * 128 / (t_pack * 1e-3) / 1e9,
+            "unpack_Gwrites_per_s": 8 * writes_per_rank / (t_unpack * 1e-3) / 1e9,
+        }
+    ov = [1, 0, 0, 0, 0]
+    t_fused = _time_events(lambda: xch.exchange(ov, ov, ov, ov, fused=True), 10, 3, inner=2)[0]
+    result["fused_us"] = t_fused * 1e3
+    result["fused_Gtransactions_per_s"] = 8 * (lines_per_rank + writes_per_rank) / (t_fused * 1e-3) / 1e9
+    return result
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -273,6 +325,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-breakdown", action="store_true")
+    ap.add_argument("--dim0-study", action="store_true",
+                    help="instead of the benchmark: the innermost-dimension halo phase alone, by number of "
+                         "ranks per launch group, as cache lines and masked writes per second")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (virtual ranks share it); "
@@ -286,6 +341,10 @@ def main() -> int:
         print("bench.py: no GPU visible", file=sys.stderr)
         return 2
     torch.cuda.set_device(0)
+
+    if args.dim0_study:
+        print(json.dumps(dim0_study()))
+        return 0
 
     bn3 = BatchNormWorkload((4, 64, 64, 64, 64), SEED + 3)
     halo = HaloWorkload(128, 32, SEED + 2)
