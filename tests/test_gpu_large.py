@@ -51,3 +51,34 @@ def test_batchnorm_beyond_2_31_elements():
     torch.cuda.synchronize()
     assert grads[0].tolist() == [0.0, 0.0]
     assert grads[1].tolist() == [float(spatial), 2.0 * spatial]
+
+
+def test_halo_faces_beyond_2_31_elements():
+    """Strips that start more than 2^31 elements into the tensor (64-bit offsets
+    in the copy kernel), dense and sparse faces, pack and unpack, bit-exact."""
+    import torch
+    from dihydrogen_amd import capi
+    lib = capi.load()
+    w, h, c = 1024, 1024, 2100  # 2.2e9 elements
+    free, _ = torch.cuda.mem_get_info()
+    if free < 2 * w * h * c * 4:
+        pytest.skip("not enough device memory")
+    t = torch.empty((1, c, h, w), device="cuda")
+    t.view(-1)[: 1 << 20].uniform_(-1, 1)
+    t.view(-1).copy_(t.view(-1)[: 1 << 20].repeat(c * h * w >> 20)[: c * h * w])  # cheap non-constant fill
+    t[0, :, :, :] += torch.arange(c, device="cuda", dtype=torch.float32).view(c, 1, 1)
+    shape = capi.i64_array((w, h, c, 1))
+    for dim, expect in ((1, lambda: t[0, :, h - 2, :]), (0, lambda: t[0, :, :, w - 2])):
+        n = lib.h2x_halo_size(4, shape, dim, 1)
+        buf = torch.full((n,), float("nan"), device="cuda")
+        capi.check(lib.h2x_halo_pack_or_unpack(capi.F32, _ptr(t), 4, shape, dim, capi.RHS, 1, _ptr(buf), 1, 0, 0,
+                                               None))
+        torch.cuda.synchronize()
+        assert torch.equal(buf, expect().reshape(-1))
+        # unpack the negated strip into the outer halo cells of the same side
+        buf.neg_()
+        capi.check(lib.h2x_halo_pack_or_unpack(capi.F32, _ptr(t), 4, shape, dim, capi.RHS, 1, _ptr(buf), 0, 0, 0,
+                                               None))
+        torch.cuda.synchronize()
+        outer = t[0, :, h - 1, :] if dim == 1 else t[0, :, :, w - 1]
+        assert torch.equal(outer.reshape(-1), buf)
