@@ -104,6 +104,37 @@ int main()
         errors += run_case(Shape({8, 10, 12, 3, 2}), Shape({2, 2, 2, 1, 1}), IntVector({1, 1, 1, 0, 0}), periodic,
                            kBoundaryStreams);
     }
+    // reverse exchange with SUM: transfers and pack + unpack leave the same tensors
+    {
+        const Shape shape({12, 10, 3, 2}), locale({2, 2, 1, 1});
+        const Distribution dist = Distribution::make_overlapped_distribution(locale, IntVector({1, 2, 0, 0}));
+        std::vector<std::unique_ptr<DevTensor<float>>> a, b;
+        std::vector<DevTensor<float>*> pa, pb;
+        std::mt19937 gen(5);
+        std::uniform_int_distribution<int> d(-8, 8);
+        for (int r = 0; r < 4; ++r)
+        {
+            a.emplace_back(new DevTensor<float>(shape, LocaleVirtual(r, 4), dist));
+            b.emplace_back(new DevTensor<float>(shape, LocaleVirtual(r, 4), dist));
+            CHECK(a.back()->allocate() == 0 && b.back()->allocate() == 0);
+            std::vector<float> h(a.back()->get_local_real_size());
+            for (auto& v : h)
+                v = static_cast<float>(d(gen));
+            to_device(*a.back(), h);
+            to_device(*b.back(), h);
+            pa.push_back(a.back().get());
+            pb.push_back(b.back().get());
+        }
+        HaloExchangeVirtual<float> xa(pa, true), xb(pb, true);
+        xa.exchange(nullptr, true, false, HaloExchangeAccumOp::SUM);
+        xb.exchange_fused(nullptr, true, HaloExchangeAccumOp::SUM);
+        for (int r = 0; r < 4; ++r)
+        {
+            const std::vector<float> ha = to_host(*a[r]), hb = to_host(*b[r]);
+            for (size_t i = 0; i < ha.size(); ++i)
+                errors += ha[i] != hb[i];
+        }
+    }
     // per-rank interface: pack one strip, unpack it on the neighbour
     {
         const Shape shape({8, 6, 2, 1}), locale({2, 1, 1, 1});
