@@ -70,6 +70,7 @@ struct BoxBatch
     Box box[kMaxBoxes];
     int32_t num_boxes;
     uint32_t num_blocks;
+    uint32_t blocks_per_box; // > 0: every box has this many workgroups and the boxes take turns
 };
 
 template <typename W, int VEC>
@@ -123,11 +124,25 @@ template <typename T, int VEC, typename Op, bool SPARSE>
 __global__ __launch_bounds__(kBlockSize) void box_copy_kernel(const BoxBatch batch, Op op)
 {
     // which box does this workgroup belong to?
+    // Boxes of equal size take turns workgroup by workgroup, so that the
+    // workgroups in flight at any time are spread over all tensors of the
+    // launch (measured: C2 exchange 425 -> 403 us, C5 round trip 191 -> 180 us
+    // against box after box); otherwise the boxes follow one another.
     int b = 0;
+    uint32_t local_block;
+    if (batch.blocks_per_box != 0)
+    {
+        b = blockIdx.x % batch.num_boxes;
+        local_block = blockIdx.x / batch.num_boxes;
+    }
+    else
+    {
 #pragma unroll 1
-    for (int i = 1; i < batch.num_boxes; ++i)
-        if (blockIdx.x >= batch.box[i].first_block)
-            b = i;
+        for (int i = 1; i < batch.num_boxes; ++i)
+            if (blockIdx.x >= batch.box[i].first_block)
+                b = i;
+        local_block = blockIdx.x - batch.box[b].first_block;
+    }
     const Box& box = batch.box[b];
     const uint32_t count = box.count;
     const int nd = box.num_dims;
@@ -136,7 +151,7 @@ __global__ __launch_bounds__(kBlockSize) void box_copy_kernel(const BoxBatch bat
     using WU = typename Words<T, VEC>::unaligned_t;
 
     constexpr uint32_t kStride = kBlockSize * VEC;
-    const uint32_t block_base = (blockIdx.x - box.first_block) * (kStride * kCopyUnroll);
+    const uint32_t block_base = local_block * (kStride * kCopyUnroll);
 
     int64_t toff[kCopyUnroll];
     int64_t soff[kCopyUnroll]; // kTransfer only: offset in the source tensor
@@ -538,6 +553,16 @@ struct Launcher
     {
         if (batch.num_boxes == 0)
             return H2X_SUCCESS;
+        batch.blocks_per_box = 0;
+        if (batch.num_boxes > 1 && batch.num_blocks % batch.num_boxes == 0)
+        {
+            const uint32_t per = batch.num_blocks / batch.num_boxes;
+            bool equal = true;
+            for (int i = 0; i < batch.num_boxes; ++i)
+                equal = equal && batch.box[i].first_block == per * static_cast<uint32_t>(i);
+            if (equal)
+                batch.blocks_per_box = per;
+        }
         int err;
         switch (elem_size)
         {
