@@ -243,12 +243,12 @@ PMC_KIB = {  # label -> (FETCH_SIZE KiB, fetch scale, WRITE_SIZE KiB) per launch
     "bn_apply": (131102, 2.0, 262162),
     "bn_backprop1": (262182, 2.0, 128),
     "bn_backprop2": (262178, 2.0, 262144),
-    "halo_dim0_pack": (153250, 2.0, 16900),    # 8 faces per launch, two launches per step
-    "halo_dim0_unpack": (8512, 2.0, 135200),
-    "halo_dim1_pack": (21181, 2.0, 33800),
-    "halo_dim1_unpack": (16968, 2.0, 37138),
-    "halo_dim2_pack": (17171, 2.0, 33800),
-    "halo_dim2_unpack": (16975, 2.0, 34929),
+    "halo_dim0_pack": (154900, 2.0, 16900),    # 8 faces per launch, two launches per step
+    "halo_dim0_unpack": (8503, 2.0, 135200),
+    "halo_dim1_pack": (21017, 2.0, 33800),
+    "halo_dim1_unpack": (16954, 2.0, 37365),
+    "halo_dim2_pack": (17048, 2.0, 33800),
+    "halo_dim2_unpack": (16956, 2.0, 35112),
 }
 
 KERNEL_OF = {
