@@ -70,7 +70,7 @@ struct BoxBatch
     Box box[kMaxBoxes];
     int32_t num_boxes;
     uint32_t num_blocks;
-    uint32_t blocks_per_box; // > 0: every box has this many workgroups and the boxes take turns
+    uint32_t blocks_per_box; // > 0: the boxes take turns, each for this many workgroups
 };
 
 template <typename W, int VEC>
@@ -124,10 +124,11 @@ template <typename T, int VEC, typename Op, bool SPARSE>
 __global__ __launch_bounds__(kBlockSize) void box_copy_kernel(const BoxBatch batch, Op op)
 {
     // which box does this workgroup belong to?
-    // Boxes of equal size take turns workgroup by workgroup, so that the
-    // workgroups in flight at any time are spread over all tensors of the
-    // launch (measured: C2 exchange 425 -> 403 us, C5 round trip 191 -> 180 us
-    // against box after box); otherwise the boxes follow one another.
+    // The boxes take turns workgroup by workgroup, so that the workgroups in
+    // flight at any time are spread over all tensors of the launch (measured:
+    // C2 exchange 425 -> 403 us, C5 round trip 191 -> 180 us against box after
+    // box).  A turn beyond the end of a smaller box finds every index out of
+    // range and does nothing.  With very unequal boxes they follow one another.
     int b = 0;
     uint32_t local_block;
     if (batch.blocks_per_box != 0)
@@ -466,6 +467,7 @@ struct Launcher
     bool sparse = false;
     HostBox last;         // geometry of the most recently queued box
     int last_mode = -1;
+    uint32_t launch_blocks = 0; // workgroups of the launch being issued
     BoxBatch batch;
 
     Launcher(hipStream_t s, int es, h2x_dtype dt, int o) : stream(s), elem_size(es), dtype(dt), op(o)
@@ -477,7 +479,7 @@ struct Launcher
     template <typename T, int VEC>
     int launch_typed()
     {
-        const dim3 grid(batch.num_blocks);
+        const dim3 grid(launch_blocks);
         switch (op)
         {
         case H2X_HALO_ID:
@@ -494,7 +496,7 @@ struct Launcher
     template <typename T, int VEC>
     int launch_accumulate()
     {
-        const dim3 grid(batch.num_blocks);
+        const dim3 grid(launch_blocks);
         switch (op)
         {
         case H2X_HALO_SUM:
@@ -553,16 +555,28 @@ struct Launcher
     {
         if (batch.num_boxes == 0)
             return H2X_SUCCESS;
+        // Taking turns needs one workgroup count for all boxes: the largest.  The
+        // surplus workgroups of smaller boxes find nothing to do; if they would
+        // more than double the grid, the boxes follow one another instead.
         batch.blocks_per_box = 0;
-        if (batch.num_boxes > 1 && batch.num_blocks % batch.num_boxes == 0)
+        uint32_t grid_blocks = batch.num_blocks;
+        if (batch.num_boxes > 1)
         {
-            const uint32_t per = batch.num_blocks / batch.num_boxes;
-            bool equal = true;
+            uint32_t most = 0;
             for (int i = 0; i < batch.num_boxes; ++i)
-                equal = equal && batch.box[i].first_block == per * static_cast<uint32_t>(i);
-            if (equal)
-                batch.blocks_per_box = per;
+            {
+                const uint32_t end = i + 1 < batch.num_boxes ? batch.box[i + 1].first_block
+                                                             : batch.num_blocks;
+                most = std::max(most, end - batch.box[i].first_block);
+            }
+            const uint64_t turns = static_cast<uint64_t>(most) * batch.num_boxes;
+            if (turns <= 2ull * batch.num_blocks && turns <= 0x7fffffffull)
+            {
+                batch.blocks_per_box = most;
+                grid_blocks = static_cast<uint32_t>(turns);
+            }
         }
+        launch_blocks = grid_blocks;
         int err;
         switch (elem_size)
         {
