@@ -643,6 +643,38 @@ int common_vector(std::initializer_list<const HostTensor*> ts, bool* strided)
     return v;
 }
 
+// Short segments.  A (sample, channel) segment much shorter than what a
+// workgroup moves (7 x 7 activations: 49 elements for 256 threads) leaves most
+// lanes idle in the dense kernels.  The samples of a channel are then folded
+// into the spatial index: the tensor is addressed as ONE sample whose segments
+// are N rows of `spatial` elements, `stride_n` apart, through the index
+// splitting of the strided kernels (x = i mod spatial, y = i / spatial), so
+// that a workgroup streams through many samples of its channel.
+// (N 256, C 2048, 7 x 7: normalise 387 us -> 75 us, backprop2 520 us -> 110 us.)
+constexpr size_t kFoldBelow = 1024;
+
+bool fold_samples(int* num_samples, size_t* spatial, std::initializer_list<HostTensor*> ts)
+{
+    if (*num_samples <= 1 || *spatial >= kFoldBelow)
+        return false;
+    for (const HostTensor* t : ts)
+        if (t->strided)
+            return false; // rows are already split
+    for (HostTensor* t : ts)
+    {
+        t->strided = true;
+        t->row = *spatial;
+        t->map.w = make_fastdiv(static_cast<uint32_t>(*spatial));
+        t->map.h = make_fastdiv(static_cast<uint32_t>(*num_samples));
+        t->map.sy = t->map.stride_n;
+        t->map.sz = 0;
+        t->aligned = false;
+    }
+    *spatial *= static_cast<size_t>(*num_samples); // < 1024 * 2^31: the callers' grid checks apply
+    *num_samples = 1;
+    return true;
+}
+
 // Launches kernel<T, V, STRIDED> for the width and layout chosen at run time.
 #define H2X_DISPATCH(KERNEL, GRID, ...)                                                            \
     do                                                                                             \
@@ -673,13 +705,17 @@ int zero_outputs(std::initializer_list<void*> outs, int num_channels, hipStream_
 }
 
 template <typename T>
-int sums_impl(int num_samples, int num_channels, size_t spatial, const HostTensor& tx, const void* x,
-              void* sums, void* sqsums, void* workspace, hipStream_t stream)
+int sums_impl(int num_samples, int num_channels, size_t spatial, const HostTensor& tx_in,
+              const void* x, void* sums, void* sqsums, void* workspace, hipStream_t stream)
 {
     if (num_channels == 0)
         return H2X_SUCCESS;
     if (num_samples == 0 || spatial == 0)
         return zero_outputs<T>({sums, sqsums}, num_channels, stream);
+    HostTensor tx = tx_in;
+    fold_samples(&num_samples, &spatial, {&tx});
+    if (spatial >= (1ull << 31) && tx.strided)
+        return H2X_ERR_TOO_LARGE;
     bool strided;
     const int vw = common_vector<T>({&tx}, &strided);
     const int gmax = max_groups_per_channel(num_channels);
@@ -725,13 +761,17 @@ Chunking elementwise_chunking(size_t spatial, size_t segments, int vw, int unrol
 }
 
 template <typename T>
-int apply_impl(int num_samples, int num_channels, size_t spatial, const HostTensor& tx,
-               const HostTensor& ty, const void* x, const void* mean, const void* var,
+int apply_impl(int num_samples, int num_channels, size_t spatial, const HostTensor& tx_in,
+               const HostTensor& ty_in, const void* x, const void* mean, const void* var,
                const void* scale, const void* bias, void* y, double epsilon, hipStream_t stream)
 {
-    const size_t segments = static_cast<size_t>(num_samples) * num_channels;
-    if (segments == 0 || spatial == 0)
+    if (static_cast<size_t>(num_samples) * num_channels == 0 || spatial == 0)
         return H2X_SUCCESS;
+    HostTensor tx = tx_in, ty = ty_in;
+    fold_samples(&num_samples, &spatial, {&tx, &ty});
+    if (spatial >= (1ull << 31) && (tx.strided || ty.strided))
+        return H2X_ERR_TOO_LARGE;
+    const size_t segments = static_cast<size_t>(num_samples) * num_channels;
     bool strided;
     const int vw = common_vector<T>({&tx, &ty}, &strided);
     const Chunking ch = elementwise_chunking(spatial, segments, vw, kUnroll);
@@ -747,8 +787,8 @@ int apply_impl(int num_samples, int num_channels, size_t spatial, const HostTens
 }
 
 template <typename T>
-int backprop1_impl(int num_samples, int num_channels, size_t spatial, const HostTensor& tx,
-                   const HostTensor& td, const void* x, const void* dy, const void* mean,
+int backprop1_impl(int num_samples, int num_channels, size_t spatial, const HostTensor& tx_in,
+                   const HostTensor& td_in, const void* x, const void* dy, const void* mean,
                    const void* var, const void* scale, void* dscale, void* dbias, void* dmean,
                    void* dvar, double epsilon, void* workspace, hipStream_t stream)
 {
@@ -756,6 +796,10 @@ int backprop1_impl(int num_samples, int num_channels, size_t spatial, const Host
         return H2X_SUCCESS;
     if (num_samples == 0 || spatial == 0)
         return zero_outputs<T>({dscale, dbias, dmean, dvar}, num_channels, stream);
+    HostTensor tx = tx_in, td = td_in;
+    fold_samples(&num_samples, &spatial, {&tx, &td});
+    if (spatial >= (1ull << 31) && (tx.strided || td.strided))
+        return H2X_ERR_TOO_LARGE;
     bool strided;
     const int vw = common_vector<T>({&tx, &td}, &strided);
     const int gmax = max_groups_per_channel(num_channels);
@@ -782,14 +826,18 @@ int backprop1_impl(int num_samples, int num_channels, size_t spatial, const Host
 
 template <typename T>
 int backprop2_impl(int num_samples, int num_channels, size_t spatial, size_t num_per_sum,
-                   const HostTensor& tx, const HostTensor& td, const HostTensor& to, const void* x,
-                   const void* dy, const void* mean, const void* var, const void* scale,
-                   const void* dmean, const void* dvar, void* dx, double epsilon,
-                   hipStream_t stream)
+                   const HostTensor& tx_in, const HostTensor& td_in, const HostTensor& to_in,
+                   const void* x, const void* dy, const void* mean, const void* var,
+                   const void* scale, const void* dmean, const void* dvar, void* dx,
+                   double epsilon, hipStream_t stream)
 {
-    const size_t segments = static_cast<size_t>(num_samples) * num_channels;
-    if (segments == 0 || spatial == 0)
+    if (static_cast<size_t>(num_samples) * num_channels == 0 || spatial == 0)
         return H2X_SUCCESS;
+    HostTensor tx = tx_in, td = td_in, to = to_in;
+    fold_samples(&num_samples, &spatial, {&tx, &td, &to});
+    if (spatial >= (1ull << 31) && (tx.strided || td.strided || to.strided))
+        return H2X_ERR_TOO_LARGE;
+    const size_t segments = static_cast<size_t>(num_samples) * num_channels;
     bool strided;
     const int vw = common_vector<T>({&tx, &td, &to}, &strided);
     const Chunking ch = elementwise_chunking(spatial, segments, vw, kUnroll / 2);

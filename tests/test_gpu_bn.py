@@ -24,6 +24,10 @@ CASES = [
     (64, 16, 7, 7),         # more samples than chunks
     (2, 130, 33, 31),       # many channels, odd sizes
     (4, 8, 16, 16, 16),     # 5-D vector path
+    (16, 24, 1, 1),         # one element per segment: samples folded into the spatial index
+    (32, 8, 3, 3),          # short odd segments, folded, scalar
+    (48, 40, 4, 4),         # short segments, folded, vector width 4
+    (6, 5, 2, 7, 9),        # 5-D, 126 elements per segment
 ]
 
 
