@@ -100,7 +100,8 @@ __global__ __launch_bounds__(kBlockSize) void softmax_fwd_reg_kernel(
     const T* __restrict__ x, T* __restrict__ y, int num_channels, size_t spatial)
 {
     using P = Pack<T, VEC>;
-    const size_t s = (static_cast<size_t>(blockIdx.x) * kBlockSize + threadIdx.x) * VEC;
+    const size_t s =
+        (static_cast<size_t>(xcd_contiguous(blockIdx.x, gridDim.x)) * kBlockSize + threadIdx.x) * VEC;
     if (s >= spatial)
         return;
     const size_t base = static_cast<size_t>(blockIdx.y) * num_channels * spatial + s;
@@ -154,37 +155,58 @@ __global__ __launch_bounds__(kBlockSize) void softmax_fwd_reg_kernel(
         }
 }
 
-// forward, any channel count: three passes over global memory per pixel.
+// forward, any channel count.  A workgroup serves 64 neighbouring pixels; its
+// four waves share the channels (wave g takes c = g, g + 4, ...), combine their
+// maxima and sums through LDS in wave order, and walk their channels again for
+// the second and third pass; the tile is 64 * C elements, so those re-reads are
+// served by the L2.  The sum is formed from four partial sums instead of one
+// running sum over all channels (softmax.cu:565-580).
 template <typename T>
-__global__ __launch_bounds__(kBlockSize) void softmax_fwd_stream_kernel(
+__global__ __launch_bounds__(kBlockSize) void softmax_fwd_wide_kernel(
     const T* __restrict__ x, T* __restrict__ y, int num_channels, size_t spatial)
 {
-    const size_t s = static_cast<size_t>(blockIdx.x) * kBlockSize + threadIdx.x;
-    if (s >= spatial)
-        return;
-    const size_t base = static_cast<size_t>(blockIdx.y) * num_channels * spatial + s;
+    __shared__ T lds[kWavesPerBlock][kWaveSize];
+    const int lane = threadIdx.x % kWaveSize;
+    const int g = threadIdx.x / kWaveSize;
+    const size_t s = static_cast<size_t>(xcd_contiguous(blockIdx.x, gridDim.x)) * kWaveSize + lane;
+    const bool active = s < spatial;
+    const size_t base = static_cast<size_t>(blockIdx.y) * num_channels * spatial + (active ? s : 0);
     const T* xp = x + base;
     T* yp = y + base;
     constexpr T kMin = Limits<T>::min_normal;
+
     T mx = kMin;
-    for (int c = 0; c < num_channels; ++c)
-    {
-        const T v = xp[static_cast<size_t>(c) * spatial];
-        mx = v > mx ? v : mx;
-    }
+    if (active)
+        for (int c = g; c < num_channels; c += kWavesPerBlock)
+        {
+            const T v = xp[static_cast<size_t>(c) * spatial];
+            mx = v > mx ? v : mx;
+        }
+    lds[g][lane] = mx;
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < kWavesPerBlock; ++w)
+        mx = lds[w][lane] > mx ? lds[w][lane] : mx;
+    __syncthreads();
+
     T sum = T(0);
-    for (int c = 0; c < num_channels; ++c)
-    {
-        const T e = exp_t(xp[static_cast<size_t>(c) * spatial] - mx);
-        yp[static_cast<size_t>(c) * spatial] = e;
-        sum += e;
-    }
-    sum = T(1) / sum;
-    for (int c = 0; c < num_channels; ++c)
-    {
-        const T r = yp[static_cast<size_t>(c) * spatial] * sum;
-        yp[static_cast<size_t>(c) * spatial] = r > kMin ? r : kMin;
-    }
+    if (active)
+        for (int c = g; c < num_channels; c += kWavesPerBlock)
+            sum += exp_t(xp[static_cast<size_t>(c) * spatial] - mx);
+    lds[g][lane] = sum;
+    __syncthreads();
+    sum = lds[0][lane];
+#pragma unroll
+    for (int w = 1; w < kWavesPerBlock; ++w)
+        sum += lds[w][lane];
+    const T inv = T(1) / sum;
+
+    if (active)
+        for (int c = g; c < num_channels; c += kWavesPerBlock)
+        {
+            const T r = exp_t(xp[static_cast<size_t>(c) * spatial] - mx) * inv;
+            yp[static_cast<size_t>(c) * spatial] = r > kMin ? r : kMin;
+        }
 }
 
 // backward, register-resident.  Replaces bp_channel_kernel, softmax.cu:621-669:
@@ -195,7 +217,8 @@ __global__ __launch_bounds__(kBlockSize) void softmax_bwd_reg_kernel(
     size_t spatial)
 {
     using P = Pack<T, VEC>;
-    const size_t s = (static_cast<size_t>(blockIdx.x) * kBlockSize + threadIdx.x) * VEC;
+    const size_t s =
+        (static_cast<size_t>(xcd_contiguous(blockIdx.x, gridDim.x)) * kBlockSize + threadIdx.x) * VEC;
     if (s >= spatial)
         return;
     const size_t base = static_cast<size_t>(blockIdx.y) * num_channels * spatial + s;
@@ -233,28 +256,42 @@ __global__ __launch_bounds__(kBlockSize) void softmax_bwd_reg_kernel(
         }
 }
 
+// backward, any channel count: the same tiling; dp is formed from the four
+// waves' partial dot products.
 template <typename T>
-__global__ __launch_bounds__(kBlockSize) void softmax_bwd_stream_kernel(
+__global__ __launch_bounds__(kBlockSize) void softmax_bwd_wide_kernel(
     const T* __restrict__ y, const T* __restrict__ dy, T* __restrict__ dx, int num_channels,
     size_t spatial)
 {
-    const size_t s = static_cast<size_t>(blockIdx.x) * kBlockSize + threadIdx.x;
-    if (s >= spatial)
-        return;
-    const size_t base = static_cast<size_t>(blockIdx.y) * num_channels * spatial + s;
+    __shared__ T lds[kWavesPerBlock][kWaveSize];
+    const int lane = threadIdx.x % kWaveSize;
+    const int g = threadIdx.x / kWaveSize;
+    const size_t s = static_cast<size_t>(xcd_contiguous(blockIdx.x, gridDim.x)) * kWaveSize + lane;
+    const bool active = s < spatial;
+    const size_t base = static_cast<size_t>(blockIdx.y) * num_channels * spatial + (active ? s : 0);
     const T* yp = y + base;
     const T* gp = dy + base;
     T* op = dx + base;
     constexpr T kMin = Limits<T>::min_normal;
+
     T dp = T(0);
-    for (int c = 0; c < num_channels; ++c)
-        dp = fma_t(yp[static_cast<size_t>(c) * spatial], gp[static_cast<size_t>(c) * spatial], dp);
-    for (int c = 0; c < num_channels; ++c)
-    {
-        const T yi = yp[static_cast<size_t>(c) * spatial];
-        op[static_cast<size_t>(c) * spatial] =
-            yi > kMin ? yi * (gp[static_cast<size_t>(c) * spatial] - dp) : T(0);
-    }
+    if (active)
+        for (int c = g; c < num_channels; c += kWavesPerBlock)
+            dp = fma_t(yp[static_cast<size_t>(c) * spatial], gp[static_cast<size_t>(c) * spatial], dp);
+    lds[g][lane] = dp;
+    __syncthreads();
+    dp = lds[0][lane];
+#pragma unroll
+    for (int w = 1; w < kWavesPerBlock; ++w)
+        dp += lds[w][lane];
+
+    if (active)
+        for (int c = g; c < num_channels; c += kWavesPerBlock)
+        {
+            const T yi = yp[static_cast<size_t>(c) * spatial];
+            op[static_cast<size_t>(c) * spatial] =
+                yi > kMin ? yi * (gp[static_cast<size_t>(c) * spatial] - dp) : T(0);
+        }
 }
 
 // Largest vector (elements) usable for all of the given pointers.
@@ -280,16 +317,32 @@ dim3 pixel_grid(size_t spatial, int vec, int num_samples)
     return dim3(static_cast<unsigned int>((spatial + per_block - 1) / per_block), num_samples);
 }
 
+// The same, padded to a multiple of the XCD count for kernels that reorder
+// their tiles with xcd_contiguous (tiles past the end do nothing).
+dim3 pixel_grid_xcd(size_t spatial, int vec, int num_samples)
+{
+    const size_t per_block = static_cast<size_t>(kBlockSize) * vec;
+    const size_t blocks = (spatial + per_block - 1) / per_block;
+    return dim3(static_cast<unsigned int>((blocks + kNumXcd - 1) / kNumXcd * kNumXcd), num_samples);
+}
+
+// 64 pixels per workgroup, padded for xcd_contiguous.
+dim3 wide_grid(size_t spatial, int num_samples)
+{
+    const size_t blocks = (spatial + kWaveSize - 1) / kWaveSize;
+    return dim3(static_cast<unsigned int>((blocks + kNumXcd - 1) / kNumXcd * kNumXcd), num_samples);
+}
+
 template <typename T, int VEC, int CMAX>
 void launch_fwd(const T* x, T* y, int n, int c, size_t s, hipStream_t st)
 {
-    softmax_fwd_reg_kernel<T, VEC, CMAX><<<pixel_grid(s, VEC, n), kBlockSize, 0, st>>>(x, y, c, s);
+    softmax_fwd_reg_kernel<T, VEC, CMAX><<<pixel_grid_xcd(s, VEC, n), kBlockSize, 0, st>>>(x, y, c, s);
 }
 
 template <typename T, int VEC, int CMAX>
 void launch_bwd(const T* y, const T* dy, T* dx, int n, int c, size_t s, hipStream_t st)
 {
-    softmax_bwd_reg_kernel<T, VEC, CMAX><<<pixel_grid(s, VEC, n), kBlockSize, 0, st>>>(y, dy, dx, c, s);
+    softmax_bwd_reg_kernel<T, VEC, CMAX><<<pixel_grid_xcd(s, VEC, n), kBlockSize, 0, st>>>(y, dy, dx, c, s);
 }
 
 // Register budget: CMAX * VEC * sizeof(T)/4 VGPRs for the forward tile, twice
@@ -344,7 +397,7 @@ int forward_impl(int n, int c, size_t s, const void* xv, void* yv, hipStream_t s
         if (c <= 64) H2X_FWD(1, 64);
     }
 #undef H2X_FWD
-    softmax_fwd_stream_kernel<T><<<pixel_grid(s, 1, n), kBlockSize, 0, st>>>(x, y, c, s);
+    softmax_fwd_wide_kernel<T><<<wide_grid(s, n), kBlockSize, 0, st>>>(x, y, c, s);
     return launch_status();
 }
 
@@ -393,7 +446,7 @@ int backward_impl(int n, int c, size_t s, const void* yv, const void* dyv, void*
         if (c <= 32) H2X_BWD(1, 32);
     }
 #undef H2X_BWD
-    softmax_bwd_stream_kernel<T><<<pixel_grid(s, 1, n), kBlockSize, 0, st>>>(y, dy, dx, c, s);
+    softmax_bwd_wide_kernel<T><<<wide_grid(s, n), kBlockSize, 0, st>>>(y, dy, dx, c, s);
     return launch_status();
 }
 
@@ -672,7 +725,7 @@ extern "C" int h2x_softmax_channel_forward(h2x_dtype dtype, int num_samples, int
         return H2X_SUCCESS; // empty local tensor: softmax.cu:600-603
     if (!x || !y)
         return H2X_ERR_INVALID_ARGUMENT;
-    if (num_samples > 65535 || (spatial_size + kBlockSize - 1) / kBlockSize > 0x7fffffffull)
+    if (num_samples > 65535 || (spatial_size + kWaveSize - 1) / kWaveSize > 0x7ffffff0ull)
         return H2X_ERR_TOO_LARGE;
     switch (dtype)
     {
@@ -694,7 +747,7 @@ extern "C" int h2x_softmax_channel_backward(h2x_dtype dtype, int num_samples, in
         return H2X_SUCCESS;
     if (!y || !dy || !dx)
         return H2X_ERR_INVALID_ARGUMENT;
-    if (num_samples > 65535 || (spatial_size + kBlockSize - 1) / kBlockSize > 0x7fffffffull)
+    if (num_samples > 65535 || (spatial_size + kWaveSize - 1) / kWaveSize > 0x7ffffff0ull)
         return H2X_ERR_TOO_LARGE;
     switch (dtype)
     {

@@ -19,7 +19,10 @@ CASES = [
     (2, 1, 4, 4),         # one channel
     (1, 33, 6, 10),       # float2 tile
     (2, 70, 3, 5),        # CMAX 128, scalar
-    (1, 200, 4, 4),       # streaming fallback
+    (1, 200, 4, 4),       # more than 128 channels: the waves of a workgroup share the channels
+    (2, 150, 9, 7),
+    (3, 300, 16, 16),
+    (4, 1000, 1, 1),      # one pixel per sample
     (2, 19, 4, 6, 10),    # 5-D
 ]
 
@@ -56,7 +59,15 @@ def test_forward_backward(shape, oracle_mod):
     torch.cuda.synchronize()
     dx = dxt.real_view().cpu().numpy()
     dx_o = oracle_mod.softmax_channel_backward(y, dy)
-    assert np.array_equal(dx, dx_o) or max_rel(dx, dx_o) <= TOL
+    if shape[1] <= 64:
+        assert np.array_equal(dx, dx_o) or max_rel(dx, dx_o) <= TOL
+    else:
+        # above 64 channels dp = sum_c y * dy is formed from four partial sums, the oracle's
+        # from one running sum: dx = y * (dy - dp) then agrees to the tolerance in units of
+        # the terms that are added up (|dy| and sum_c |y * dy|), not of their difference
+        terms = np.abs(dy) + (y.astype(np.float64) * np.abs(dy)).sum(axis=1, keepdims=True)
+        bound = TOL * y * terms
+        assert (np.abs(dx.astype(np.float64) - dx_o) <= bound + 1e-45).all()
 
 
 def test_underflow_clamp_and_guard(oracle_mod):
