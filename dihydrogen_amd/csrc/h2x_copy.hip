@@ -124,11 +124,14 @@ template <typename T, int VEC, typename Op, bool SPARSE>
 __global__ __launch_bounds__(kBlockSize) void box_copy_kernel(const BoxBatch batch, Op op)
 {
     // which box does this workgroup belong to?
-    // The boxes take turns workgroup by workgroup, so that the workgroups in
-    // flight at any time are spread over all tensors of the launch (measured:
-    // C2 exchange 425 -> 403 us, C5 round trip 191 -> 180 us against box after
-    // box).  A turn beyond the end of a smaller box finds every index out of
-    // range and does nothing.  With very unequal boxes they follow one another.
+    // The boxes take turns workgroup by workgroup.  Workgroups go to the eight
+    // XCDs round-robin, so with 8 or 16 boxes in a launch every box is served
+    // by one XCD, whose L2 then streams one contiguous region (measured: C2
+    // exchange 425 -> 403 us, C5 round trip 191 -> 180 us against box after
+    // box; rotating the turns so that a box wanders over the XCDs loses the
+    // gain again).  A turn beyond the end of a smaller box finds every index
+    // out of range and does nothing.  With very unequal boxes they follow one
+    // another.
     int b = 0;
     uint32_t local_block;
     if (batch.blocks_per_box != 0)
