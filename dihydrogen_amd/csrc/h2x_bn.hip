@@ -879,6 +879,18 @@ int sums_strided(int n, const h2x_tensor_geometry* g, const void* x, void* sums,
     return err ? err : sums_impl<T>(n, c, s, tx, x, sums, sqsums, ws, st);
 }
 
+// Two geometries describe the same elements only if every local extent agrees:
+// equal products are not enough (8 x 4 against 4 x 8 would pair other elements).
+bool same_local_shape(const h2x_tensor_geometry* a, const h2x_tensor_geometry* b)
+{
+    if (a->num_dims != b->num_dims)
+        return false;
+    for (int i = 0; i < a->num_dims; ++i)
+        if (a->local_shape[i] != b->local_shape[i])
+            return false;
+    return true;
+}
+
 template <typename T>
 int apply_strided(int n, const h2x_tensor_geometry* gx, const h2x_tensor_geometry* gy, const void* x,
                   const void* mean, const void* var, const void* scale, const void* bias, void* y,
@@ -890,7 +902,7 @@ int apply_strided(int n, const h2x_tensor_geometry* gx, const h2x_tensor_geometr
     int err = strided_tensor<T>(gx, x, n, &tx, &c, &s);
     if (!err)
         err = strided_tensor<T>(gy, y, n, &ty, &c2, &s2);
-    if (!err && (c != c2 || s != s2))
+    if (!err && (c != c2 || s != s2 || !same_local_shape(gx, gy)))
         err = H2X_ERR_INVALID_ARGUMENT;
     return err ? err : apply_impl<T>(n, c, s, tx, ty, x, mean, var, scale, bias, y, eps, st);
 }
@@ -907,7 +919,7 @@ int backprop1_strided(int n, const h2x_tensor_geometry* gx, const h2x_tensor_geo
     int err = strided_tensor<T>(gx, x, n, &tx, &c, &s);
     if (!err)
         err = strided_tensor<T>(gd, dy, n, &td, &c2, &s2);
-    if (!err && (c != c2 || s != s2))
+    if (!err && (c != c2 || s != s2 || !same_local_shape(gx, gd)))
         err = H2X_ERR_INVALID_ARGUMENT;
     return err ? err
                : backprop1_impl<T>(n, c, s, tx, td, x, dy, mean, var, scale, dscale, dbias, dmean,
@@ -928,7 +940,9 @@ int backprop2_strided(int n, size_t num_per_sum, const h2x_tensor_geometry* gx,
         err = strided_tensor<T>(gd, dy, n, &td, &c2, &s2);
     if (!err)
         err = strided_tensor<T>(go, dx, n, &to, &c3, &s3);
-    if (!err && (c != c2 || s != s2 || c != c3 || s != s3))
+    if (!err
+        && (c != c2 || s != s2 || c != c3 || s != s3 || !same_local_shape(gx, gd)
+            || !same_local_shape(gx, go)))
         err = H2X_ERR_INVALID_ARGUMENT;
     return err ? err
                : backprop2_impl<T>(n, c, s, num_per_sum, tx, td, to, x, dy, mean, var, scale, dmean,

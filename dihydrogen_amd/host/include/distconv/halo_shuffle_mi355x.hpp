@@ -538,7 +538,10 @@ private:
 // shuffle_mpi_cuda.hpp:14-512 for one rank.  The constructor builds the
 // reference's tables (rank limits of the peer grid in local coordinates,
 // counts and displacements in rank order, :129-287); `transfer` is virtual, as
-// in the reference, and by default copies nothing.
+// in the reference.  The reference's default is the all-to-all over the ranks
+// (:342-403); one rank of a virtual locale can deliver only to itself, so the
+// default here moves the rank's own chunk and aborts if another rank has
+// anything to send or receive (TensorShufflerVirtual does the all-to-all).
 template <typename DataType>
 class TensorMPICUDAShuffler
 {
@@ -549,7 +552,7 @@ public:
                           DataType* src_buf = nullptr, DataType* dst_buf = nullptr)
         : m_src_local_size(src_tensor.get_local_size()), m_dst_local_size(dst_tensor.get_local_size()),
           m_src_split_root(src_tensor.is_split_root()), m_dst_split_root(dst_tensor.is_split_root()),
-          m_src_buf(src_buf), m_dst_buf(dst_buf)
+          m_rank(src_tensor.get_locale().get_rank()), m_src_buf(src_buf), m_dst_buf(dst_buf)
     {
         const int n = src_tensor.get_locale().get_size();
         m_rank_limits_fwd = rank_limits(src_tensor, dst_tensor);
@@ -647,12 +650,26 @@ public:
 
 protected:
     // shuffle_mpi_cuda.hpp:342-403: moves the packed chunks between ranks.  One
-    // rank alone has no one to exchange with; TensorShufflerVirtual supplies it.
+    // rank alone can deliver only its own chunk; a shuffle that involves other
+    // ranks must go through TensorShufflerVirtual (or an override), so a non-zero
+    // count for another rank aborts instead of leaving `recv_buf` unwritten.
     virtual void transfer(const DataType* send_buf, size_t send_buffer_size, DataType* recv_buf,
                           size_t recv_buffer_size, bool is_forward, hipStream_t stream)
     {
-        (void) send_buf, (void) send_buffer_size, (void) recv_buf, (void) recv_buffer_size;
-        (void) is_forward, (void) stream;
+        const std::vector<int>& send_counts = get_send_counts(is_forward);
+        const std::vector<int>& recv_counts = get_recv_counts(is_forward);
+        for (size_t p = 0; p < send_counts.size(); ++p)
+            if (static_cast<int>(p) != m_rank)
+                assert_always(send_counts[p] == 0 && recv_counts[p] == 0);
+        const size_t bytes = static_cast<size_t>(send_counts[m_rank]) * sizeof(DataType);
+        assert_always(send_counts[m_rank] == recv_counts[m_rank]);
+        const size_t from = static_cast<size_t>(get_send_displs_h(is_forward)[m_rank]);
+        const size_t to = static_cast<size_t>(get_recv_displs_h(is_forward)[m_rank]);
+        assert_always(from * sizeof(DataType) + bytes <= send_buffer_size
+                      && to * sizeof(DataType) + bytes <= recv_buffer_size);
+        if (bytes > 0)
+            DISTCONV_CHECK_HIP(hipMemcpyAsync(recv_buf + to, send_buf + from, bytes,
+                                              hipMemcpyDeviceToDevice, stream));
     }
 
     void shuffle(const DataType* src, DataType* dst, hipStream_t stream, bool is_forward)
@@ -737,6 +754,7 @@ private:
 
     size_t m_src_local_size, m_dst_local_size;
     bool m_src_split_root, m_dst_split_root;
+    int m_rank;
     std::vector<int> m_rank_limits_fwd, m_rank_limits_bwd;
     std::vector<int> m_send_counts, m_recv_counts, m_send_displs, m_recv_displs;
     DataType* m_src_buf;

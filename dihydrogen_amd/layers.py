@@ -384,6 +384,19 @@ class HaloExchangeVirtual:
             return None
         return peer
 
+    def _check_widths(self, dim: int, widths) -> None:
+        """The receive buffers hold `overlap[dim]` cells per row and the strips lie
+        inside the halo: TraverseHalo's precondition, halo_cuda.hpp:909-916."""
+        for t in self.tensors:
+            if max(widths) > t.overlap[dim]:
+                raise ValueError(f"halo width {max(widths)} exceeds the overlap {t.overlap[dim]} of "
+                                 f"dimension {dim}")
+
+    def _addresses(self):
+        """Device addresses the cached face tables were built for; a tensor that
+        was reallocated gets new tables."""
+        return tuple(t.get_buffer() if t.data is not None else 0 for t in self.tensors)
+
     def _recv_buffer(self, rank: int, dim: int, side: int) -> torch.Tensor:
         key = (rank, dim, side)
         if key not in self._recv:
@@ -413,6 +426,7 @@ class HaloExchangeVirtual:
         move straight from tensor to tensor in one launch per group of ranks;
         the result is the same."""
         dtype = self.tensors[0].h2x_dtype
+        self._check_widths(dim, (width_rhs_send, width_rhs_recv, width_lhs_send, width_lhs_recv))
         if fused:
             if skip_unpack:
                 raise ValueError("a fused exchange has no separate unpack to skip")
@@ -420,7 +434,7 @@ class HaloExchangeVirtual:
                                      width_lhs_recv, is_reverse, op)
             return
         key = (dim, width_rhs_send, width_rhs_recv, width_lhs_send, width_lhs_recv, is_reverse,
-               skip_unpack, op)
+               skip_unpack, op, self._addresses())
         cached = self._faces.get(key)
         if cached is None:
             widths = (width_rhs_send, width_rhs_recv, width_lhs_send, width_lhs_recv)
@@ -443,7 +457,7 @@ class HaloExchangeVirtual:
                             src = self._recv_buffer(r, dim, side)
                             unpacks.append(self._face(r, dim, side, w_recv, src, False, is_reverse, op))
                 # the face tables depend only on the arguments and on the tensors'
-                # addresses, which do not change: build them once
+                # addresses (part of the key): build them once
                 cached.append(tuple((capi.HaloFace * len(f))(*f) if f else None for f in (packs, unpacks)))
             self._faces[key] = cached
         st = _stream_handle(self.stream)
@@ -462,7 +476,7 @@ class HaloExchangeVirtual:
                             width_lhs_recv, is_reverse, op) -> None:
         dtype = self.tensors[0].h2x_dtype
         widths = (width_rhs_send, width_rhs_recv, width_lhs_send, width_lhs_recv)
-        key = ("fused", dim) + widths + (is_reverse, op)
+        key = ("fused", dim) + widths + (is_reverse, op, self._addresses())
         cached = self._faces.get(key)
         if cached is None:
             cached = []

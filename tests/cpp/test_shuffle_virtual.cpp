@@ -108,6 +108,32 @@ int main()
         CHECK((sh.get_send_displs_h(true) == std::vector<int>{0, 32, 64, 96}));
         CHECK(TensorMPICUDAShuffler<float>::get_buf_size(a) == 8 * 8 * 2 * 1 * sizeof(float));
     }
+    // one rank alone: shuffle_forward / shuffle_backward of the per-rank class itself
+    // (pack -> default transfer of the rank's own chunk -> unpack), plain source into a
+    // haloed destination and back
+    {
+        const Shape s1({6, 5, 3, 2});
+        DevTensor<float> a(s1, LocaleVirtual(0, 1), Distribution::make_distribution(Shape({1, 1, 1, 1})));
+        DevTensor<float> b(s1, LocaleVirtual(0, 1),
+                           Distribution::make_overlapped_distribution(Shape({1, 1, 1, 1}), IntVector({1, 2, 0, 0})));
+        a.allocate();
+        b.allocate();
+        const std::vector<float> field = global_offset_field(a, -1.0f);
+        to_device(a, field);
+        to_device(b, std::vector<float>(b.get_local_real_size(), -7.0f));
+        TensorMPICUDAShuffler<float> sh(a, b);
+        sh.shuffle_forward(a.get_const_base_ptr(), b.get_base_ptr());
+        DISTCONV_CHECK_HIP(hipDeviceSynchronize());
+        const std::vector<float> want = global_offset_field(b, -7.0f), got = to_host(b);
+        for (size_t i = 0; i < got.size(); ++i)
+            errors += got[i] != want[i];
+        to_device(a, std::vector<float>(a.get_local_real_size(), -3.0f));
+        sh.shuffle_backward(b.get_const_base_ptr(), a.get_base_ptr());
+        DISTCONV_CHECK_HIP(hipDeviceSynchronize());
+        const std::vector<float> back = to_host(a);
+        for (size_t i = 0; i < back.size(); ++i)
+            errors += back[i] != field[i];
+    }
     std::printf("test_shuffle_virtual: %d errors\n", errors);
     return errors ? 1 : 0;
 }

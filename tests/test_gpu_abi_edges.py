@@ -141,7 +141,26 @@ def test_rejected_calls_return_status_and_write_nothing():
         g.local_shape[i], g.strides[i] = e, s
     assert lib.h2x_bn_channel_sums_and_sqsums_strided(capi.F32, 2, ctypes.byref(g), p(x), p(out[0]),
                                                       p(out[1]), p(ws), None) == UNSUPPORTED
+    # two geometries with equal channel count and equal spatial size but other extents
+    # (4 x 2 against 2 x 4) would pair different elements: rejected
+    ga, gb = capi.TensorGeometry(), capi.TensorGeometry()
+    ga.num_dims = gb.num_dims = 4
+    for i, (e, s) in enumerate(zip((4, 2, c, 2), (1, 4, 8, 8 * c))):
+        ga.local_shape[i], ga.strides[i] = e, s
+    for i, (e, s) in enumerate(zip((2, 4, c, 2), (1, 2, 8, 8 * c))):
+        gb.local_shape[i], gb.strides[i] = e, s
+    y = torch.full_like(x, POISON)
+    assert lib.h2x_bn_batch_normalization_strided(
+        capi.F32, 2, ctypes.byref(ga), ctypes.byref(gb), p(x), p(out[0]), p(out[1]), p(out[2]), p(out[3]),
+        p(y), 1e-5, None) == INVALID
+    assert lib.h2x_bn_backprop1_strided(
+        capi.F32, 2, ctypes.byref(ga), ctypes.byref(gb), p(x), p(x), p(x), p(x), p(x), p(out[0]), p(out[1]),
+        p(out[2]), p(out[3]), 1e-5, p(ws), None) == INVALID
+    assert lib.h2x_bn_backprop2_strided(
+        capi.F32, 2, 16, ctypes.byref(ga), ctypes.byref(ga), ctypes.byref(gb), p(x), p(x), p(x), p(x), p(x),
+        p(x), p(x), p(y), 1e-5, None) == INVALID
     torch.cuda.synchronize()
+    assert (y == POISON).all()
     for o in out:
         assert (o == POISON).all()
     assert (x == 1).all()

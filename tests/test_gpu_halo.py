@@ -221,6 +221,37 @@ def test_exchange_narrower_than_halo(oracle_mod):
         assert np.array_equal(w, g, equal_nan=True)
 
 
+def test_exchange_wider_than_halo_is_rejected_and_reallocation_is_seen(oracle_mod):
+    """Strips wider than the halo would run past the receive buffers: the layer
+    refuses them.  Face tables are cached per tensor address: an exchange after
+    a tensor was reallocated works on the new allocation."""
+    import torch
+    from dihydrogen_amd.layers import HaloExchangeVirtual
+    from dihydrogen_amd.tensor import Distribution, LocaleVirtual, Tensor
+    shape, locale, overlap = (12, 10, 3, 2), (2, 2, 1, 1), (1, 1, 0, 0)
+    dist = Distribution.make_overlapped_distribution(locale, overlap)
+    tensors = [Tensor(shape, LocaleVirtual(r, 4), dist).allocate() for r in range(4)]
+    xch = HaloExchangeVirtual(tensors, periodic=True)
+    for fused in (False, True):
+        with pytest.raises(ValueError):
+            xch.exchange([2, 1, 0, 0], [2, 1, 0, 0], [2, 1, 0, 0], [2, 1, 0, 0], fused=fused)
+    for fused in (False, True):
+        for t in tensors:
+            t.real_view().fill_(float("nan"))
+            t.interior_view().fill_(1.0)
+        xch.exchange(fused=fused)
+        torch.cuda.synchronize()
+        keep = [t.data for t in tensors]          # old allocations stay alive, so the new ones differ
+        for t in tensors:
+            t.data = torch.full_like(t.data, float("nan"))
+            t.interior_view().fill_(2.0)
+        xch.exchange(fused=fused)
+        torch.cuda.synchronize()
+        for t in tensors:
+            assert (t.real_view() == 2.0).all()   # periodic: every halo cell has a source
+        del keep
+
+
 def test_reverse_sum_exchange(oracle_mod):
     """Reverse exchange with SUM: halo contributions are added onto the
     neighbour's boundary cells (used by backward-data and pooling)."""
