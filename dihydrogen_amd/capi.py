@@ -87,6 +87,9 @@ SIGNATURES = {
     "h2x_bn_workspace_bytes": (c_size_t, [c_int]),
     "h2x_bn_channel_sums_and_sqsums": (c_int, [c_int, c_int, c_int, c_size_t, c_size_t, c_void_p,
                                                c_void_p, c_void_p, c_void_p, c_void_p]),
+    "h2x_bn_channel_sums_and_sqsums_static": (c_int, [c_int, c_int, c_int, c_size_t, c_size_t, c_void_p,
+                                                      c_void_p, c_void_p, c_void_p]),
+    "h2x_bn_static_max_channels": (c_size_t, []),
     "h2x_bn_sums_to_statistics": (c_int, [c_int, c_int, c_size_t, c_double, c_void_p, c_void_p,
                                           c_void_p, c_void_p, c_void_p]),
     "h2x_bn_batch_normalization": (c_int, [c_int, c_int, c_int, c_size_t, c_size_t, c_size_t,

@@ -14,6 +14,9 @@ extern "C" const char* h2x_status_string(int status)
     case H2X_ERR_INVALID_ARGUMENT: return "invalid argument";
     case H2X_ERR_UNSUPPORTED: return "unsupported element type, size or operation";
     case H2X_ERR_TOO_LARGE: return "size exceeds what one launch can address";
+    case H2X_ERR_SCRATCH_LIMIT:
+        return "input exceeds the fixed capacity of the library's static scratch array "
+               "(use the entry point that takes a workspace)";
     default: break;
     }
     if (status > 0)

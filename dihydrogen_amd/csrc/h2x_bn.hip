@@ -32,11 +32,48 @@
 #include "h2x_device.hpp"
 
 #include <algorithm>
+#include <mutex>
+
+// Partial sums of h2x_bn_channel_sums_and_sqsums_static, the entry point for
+// callers that can neither allocate nor bring a workspace.  Every device the
+// library runs on holds its own copy of this array, at its own address, until
+// the process ends.  In host code the name is only a handle for
+// hipGetSymbolAddress; kernels receive the address that call returned.
+static constexpr size_t kStaticScratchBytes = size_t(1) << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 namespace h2x
 {
 namespace
 {
+
+// Device address of `scratch` on the current device, looked up once per device.
+constexpr int kMaxDevices = 64;
+std::mutex static_scratch_mutex;
+void* static_scratch_address[kMaxDevices] = {};
+
+int static_scratch(void** out)
+{
+    int device = -1;
+    hipError_t err = hipGetDevice(&device);
+    if (err != hipSuccess)
+        return static_cast<int>(err);
+    if (device < 0 || device >= kMaxDevices)
+        return H2X_ERR_UNSUPPORTED;
+    std::lock_guard<std::mutex> lock(static_scratch_mutex);
+    if (static_scratch_address[device] == nullptr)
+    {
+        void* p = nullptr;
+        err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (err != hipSuccess)
+            return static_cast<int>(err);
+        if (p == nullptr)
+            return static_cast<int>(hipErrorInvalidSymbol);
+        static_scratch_address[device] = p;
+    }
+    *out = static_scratch_address[device];
+    return H2X_SUCCESS;
+}
 
 constexpr int kUnroll = 4;
 // Workgroups a reduction aims at over all channels (bounds the workspace) and
@@ -982,6 +1019,38 @@ extern "C" int h2x_bn_channel_sums_and_sqsums(h2x_dtype dtype, int num_samples, 
                                    sqsums, workspace, as_stream(stream)),
                  sums_dense<double>(num_samples, num_channels, spatial_size, spatial_real_size, x,
                                     sums, sqsums, workspace, as_stream(stream)));
+}
+
+extern "C" size_t h2x_bn_static_max_channels(void)
+{
+    // largest channel count whose partial sums fit in the scratch array
+    int lo = 0, hi = 65535;
+    while (lo < hi)
+    {
+        const int mid = (lo + hi + 1) / 2;
+        if (h2x_bn_workspace_bytes(mid) <= kStaticScratchBytes)
+            lo = mid;
+        else
+            hi = mid - 1;
+    }
+    return static_cast<size_t>(lo);
+}
+
+extern "C" int h2x_bn_channel_sums_and_sqsums_static(h2x_dtype dtype, int num_samples,
+                                                     int num_channels, size_t spatial_size,
+                                                     size_t spatial_real_size, const void* x,
+                                                     void* sums, void* sqsums, h2x_stream_t stream)
+{
+    if (num_channels > 0 && h2x_bn_workspace_bytes(num_channels) > kStaticScratchBytes)
+        return H2X_ERR_SCRATCH_LIMIT;
+    void* workspace = nullptr;
+    const int err = static_scratch(&workspace);
+    if (err != 0)
+        return err;
+    // The partial sums need no clearing: every slot the finishing kernel reads
+    // is written by this call's reduction kernel first.
+    return h2x_bn_channel_sums_and_sqsums(dtype, num_samples, num_channels, spatial_size,
+                                          spatial_real_size, x, sums, sqsums, workspace, stream);
 }
 
 extern "C" int h2x_bn_channel_sums_and_sqsums_strided(h2x_dtype dtype, int num_samples,

@@ -39,7 +39,8 @@ typedef enum h2x_status
     H2X_SUCCESS = 0,
     H2X_ERR_INVALID_ARGUMENT = -1,
     H2X_ERR_UNSUPPORTED = -2,
-    H2X_ERR_TOO_LARGE = -3
+    H2X_ERR_TOO_LARGE = -3,
+    H2X_ERR_SCRATCH_LIMIT = -4 /* beyond the fixed capacity of an entry point that allocates nothing */
 } h2x_status;
 
 /** Element type of floating-point tensors (batch-norm, softmax, halo accumulate). */
@@ -118,6 +119,32 @@ int h2x_bn_channel_sums_and_sqsums(h2x_dtype dtype,
                                    void* sqsums,
                                    void* workspace,
                                    h2x_stream_t stream);
+
+/**
+ * h2x_bn_channel_sums_and_sqsums for callers that cannot allocate device
+ * memory and have no workspace to pass: code under HIP graph capture, serving
+ * loops, harnesses that forbid allocation.  It has no counterpart in the
+ * reference.  Same arguments, kernels and results (bit for bit) as
+ * h2x_bn_channel_sums_and_sqsums, but the partial sums live in a 1 MiB array
+ * inside the library's device image, one copy per device; the call performs no
+ * allocation of any kind.  num_channels above h2x_bn_static_max_channels() is
+ * rejected with H2X_ERR_SCRATCH_LIMIT.  All calls on one device share that array:
+ * two calls that may run concurrently on one device (different streams) race.
+ * The array's device address is looked up on the first call on each device
+ * (hipGetSymbolAddress, no allocation); make that call outside graph capture.
+ */
+int h2x_bn_channel_sums_and_sqsums_static(h2x_dtype dtype,
+                                          int num_samples,
+                                          int num_channels,
+                                          size_t spatial_size,
+                                          size_t spatial_real_size,
+                                          const void* x,
+                                          void* sums,
+                                          void* sqsums,
+                                          h2x_stream_t stream);
+
+/** Largest num_channels h2x_bn_channel_sums_and_sqsums_static accepts. */
+size_t h2x_bn_static_max_channels(void);
 
 /**
  * In place: mean = sums / n; var = max(sqsums / n - mean^2, 0) * n / (n - 1);
