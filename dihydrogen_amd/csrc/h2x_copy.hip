@@ -23,354 +23,107 @@
 // A fourth mode moves a strip straight from one tensor into another (the
 // neighbour's interior strip into this rank's halo) when both live on the same
 // device: pack and unpack of a halo exchange without the buffer in between.
-#include "h2x_device.hpp"
+#include "h2x_copy_kernel.hpp"
 
 #include <algorithm>
 #include <cstring>
 #include <new>
-#include <type_traits>
 #include <vector>
 
 namespace h2x
 {
+namespace copy
+{
+
+// ---- launches of the identity instantiations -------------------------------------
+
 namespace
 {
 
-constexpr int kMaxBoxes = 16;
-constexpr int kMaxBoxDims = H2X_MAX_DIMS;
-constexpr int kCopyUnroll = 4;
-
-enum Mode : int
+template <typename T, int VEC, bool SPARSE>
+int launch_mode(const LaunchShape& s, const BoxBatch& batch)
 {
-    kPack = 0,    // buffer <- tensor
-    kUnpack = 1,  // tensor <- op(tensor, buffer)
-    kClear = 2,   // tensor <- 0
-    kTransfer = 3 // tensor <- op(tensor, source tensor)
-};
-
-// One reduced box.  Packed element g (natural order of extent[]) lives at
-// tensor[tensor_offset + sum idx[i] * stride[i]].
-struct Box
-{
-    char* tensor;            // base the strides are relative to
-    char* buffer;            // start of this box's contiguous image (kTransfer: source box origin)
-    char* tensor2;           // second box of identical geometry (sparse pairs), or null
-    char* buffer2;
-    int64_t stride[kMaxBoxDims]; // elements
-    int64_t stride_src[kMaxBoxDims]; // kTransfer: strides of the source tensor
-    FastDiv div[kMaxBoxDims];    // by extent[i]; the last used one is never divided by
-    uint32_t count;          // elements in the box (< 2^31)
-    uint32_t first_block;    // first workgroup of this box in the launch
-    int32_t num_dims;
-    int32_t mode;            // Mode
-};
-
-struct BoxBatch
-{
-    Box box[kMaxBoxes];
-    int32_t num_boxes;
-    uint32_t num_blocks;
-    uint32_t blocks_per_box; // > 0: the boxes take turns, each for this many workgroups
-};
-
-template <typename W, int VEC>
-struct Words
-{
-    typedef W aligned_t __attribute__((ext_vector_type(VEC)));
-    typedef W unaligned_t __attribute__((ext_vector_type(VEC), aligned(sizeof(W))));
-};
-
-struct OpId
-{
-    template <typename T>
-    __device__ __forceinline__ T operator()(T, T b) const { return b; }
-};
-struct OpSum
-{
-    template <typename T>
-    __device__ __forceinline__ T operator()(T a, T b) const { return a + b; }
-};
-struct OpMax
-{
-    template <typename T>
-    __device__ __forceinline__ T operator()(T a, T b) const { return a > b ? a : b; }
-};
-struct OpMin
-{
-    template <typename T>
-    __device__ __forceinline__ T operator()(T a, T b) const { return a < b ? a : b; }
-};
-
-// Loads and stores of "sparse" boxes: runs shorter than a cache line that are
-// a row apart (a halo face of the innermost dimension).  Every element costs a
-// whole 128-byte line of HBM traffic; stores are write-through so that the
-// line is not allocated for a 4-byte write.
-template <typename T>
-__device__ __forceinline__ void sparse_store_scalar(T* p, T v)
-{
-    if constexpr (sizeof(T) >= 4)
-        __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    else
-        *p = v;
+    const dim3 grid(s.grid);
+    switch (s.mode)
+    {
+    case kPack:
+        box_copy_kernel<T, VEC, OpId, SPARSE, kPack, false><<<grid, kCopyBlock, 0, s.stream>>>(batch, OpId());
+        break;
+    case kUnpack:
+        box_copy_kernel<T, VEC, OpId, SPARSE, kUnpack, false><<<grid, kCopyBlock, 0, s.stream>>>(batch, OpId());
+        break;
+    case kClear:
+        box_copy_kernel<T, VEC, OpId, SPARSE, kClear, false><<<grid, kCopyBlock, 0, s.stream>>>(batch, OpId());
+        break;
+    case kTransfer:
+        box_copy_kernel<T, VEC, OpId, SPARSE, kTransfer, false><<<grid, kCopyBlock, 0, s.stream>>>(batch, OpId());
+        break;
+    default: return H2X_ERR_UNSUPPORTED;
+    }
+    return launch_status();
 }
 
-// T: element type the op sees (an unsigned integer of the element's size for
-// plain copies).  VEC elements of one run move per thread and step; the buffer
-// side is VEC-aligned, the tensor side may start on any element.  SPARSE boxes
-// come in pairs of identical geometry (the LHS and RHS face of one tensor):
-// one thread serves the same index of both, so that neighbouring rows' ends,
-// which share a cache line, are touched by neighbouring lanes of one wave.
-template <typename T, int VEC, typename Op, bool SPARSE>
-__global__ __launch_bounds__(kBlockSize) void box_copy_kernel(const BoxBatch batch, Op op)
+template <typename T, int VEC>
+int launch_sparse(const LaunchShape& s, const BoxBatch& batch)
 {
-    // which box does this workgroup belong to?
-    // The boxes take turns workgroup by workgroup.  Workgroups go to the eight
-    // XCDs round-robin, so with 8 or 16 boxes in a launch every box is served
-    // by one XCD, whose L2 then streams one contiguous region (measured: C2
-    // exchange 425 -> 403 us, C5 round trip 191 -> 180 us against box after
-    // box; rotating the turns so that a box wanders over the XCDs loses the
-    // gain again).  A turn beyond the end of a smaller box finds every index
-    // out of range and does nothing.  With very unequal boxes they follow one
-    // another.
-    int b = 0;
-    uint32_t local_block;
-    if (batch.blocks_per_box != 0)
-    {
-        b = blockIdx.x % batch.num_boxes;
-        local_block = blockIdx.x / batch.num_boxes;
-    }
-    else
-    {
-#pragma unroll 1
-        for (int i = 1; i < batch.num_boxes; ++i)
-            if (blockIdx.x >= batch.box[i].first_block)
-                b = i;
-        local_block = blockIdx.x - batch.box[b].first_block;
-    }
-    const Box& box = batch.box[b];
-    const uint32_t count = box.count;
-    const int nd = box.num_dims;
-    const int mode = box.mode;
-    using WA = typename Words<T, VEC>::aligned_t;
-    using WU = typename Words<T, VEC>::unaligned_t;
-
-    constexpr uint32_t kStride = kBlockSize * VEC;
-    const uint32_t block_base = local_block * (kStride * kCopyUnroll);
-
-    int64_t toff[kCopyUnroll];
-    int64_t soff[kCopyUnroll]; // kTransfer only: offset in the source tensor
-    uint32_t g[kCopyUnroll];
-#pragma unroll
-    for (int u = 0; u < kCopyUnroll; ++u)
-    {
-        g[u] = block_base + u * kStride + threadIdx.x * VEC;
-        uint32_t rem = g[u];
-        int64_t off = 0, src = 0;
-#pragma unroll
-        for (int i = 0; i < kMaxBoxDims - 1; ++i)
-        {
-            if (i < nd - 1)
-            {
-                const uint32_t q = fastdiv(rem, box.div[i]);
-                const int64_t idx = rem - q * box.div[i].divisor;
-                off += idx * box.stride[i];
-                if (mode == kTransfer)
-                    src += idx * box.stride_src[i];
-                rem = q;
-            }
-        }
-        off += static_cast<int64_t>(rem) * box.stride[nd - 1];
-        if (mode == kTransfer)
-            src += static_cast<int64_t>(rem) * box.stride_src[nd - 1];
-        toff[u] = off;
-        soff[u] = src;
-    }
-
-    constexpr int kSides = SPARSE ? 2 : 1;
-#pragma unroll
-    for (int side = 0; side < kSides; ++side)
-    {
-        T* const tensor = reinterpret_cast<T*>(side == 0 ? box.tensor : box.tensor2);
-        T* const buffer = reinterpret_cast<T*>(side == 0 ? box.buffer : box.buffer2);
-        if (side == 1 && tensor == nullptr)
-            break;
-        if (mode == kPack)
-        {
-            if constexpr (SPARSE)
-            {
-                // both faces' loads are issued before any store, so that the
-                // two touches of a shared line meet in the cache
-                if (side == 1)
-                    break;
-                T* const tensor_b = reinterpret_cast<T*>(box.tensor2);
-                T* const buffer_b = reinterpret_cast<T*>(box.buffer2);
-                WU va[kCopyUnroll], vb[kCopyUnroll];
-#pragma unroll
-                for (int u = 0; u < kCopyUnroll; ++u)
-                    if (g[u] < count)
-                    {
-                        va[u] = *reinterpret_cast<const WU*>(tensor + toff[u]);
-                        if (tensor_b != nullptr)
-                            vb[u] = *reinterpret_cast<const WU*>(tensor_b + toff[u]);
-                    }
-#pragma unroll
-                for (int u = 0; u < kCopyUnroll; ++u)
-                    if (g[u] < count)
-                    {
-                        *reinterpret_cast<WA*>(buffer + g[u]) = va[u];
-                        if (tensor_b != nullptr)
-                            *reinterpret_cast<WA*>(buffer_b + g[u]) = vb[u];
-                    }
-            }
-            else
-            {
-                // The tensor is read once and streams past the memory-side
-                // cache; the packed image is stored normally so that it is
-                // still there when the matching unpack reads it.
-                WU v[kCopyUnroll];
-#pragma unroll
-                for (int u = 0; u < kCopyUnroll; ++u)
-                    if (g[u] < count)
-                        v[u] = __builtin_nontemporal_load(
-                            reinterpret_cast<const WU*>(tensor + toff[u]));
-#pragma unroll
-                for (int u = 0; u < kCopyUnroll; ++u)
-                    if (g[u] < count)
-                        *reinterpret_cast<WA*>(buffer + g[u]) = v[u];
-            }
-        }
-        else if (mode == kUnpack)
-        {
-            WA v[kCopyUnroll];
-#pragma unroll
-            for (int u = 0; u < kCopyUnroll; ++u)
-                if (g[u] < count)
-                    v[u] = __builtin_nontemporal_load(
-                        reinterpret_cast<const WA*>(buffer + g[u])); // last use of the image
-            if constexpr (std::is_same<Op, OpId>::value)
-            {
-#pragma unroll
-                for (int u = 0; u < kCopyUnroll; ++u)
-                    if (g[u] < count)
-                    {
-                        if constexpr (SPARSE && VEC == 1)
-                            sparse_store_scalar(tensor + toff[u], v[u][0]);
-                        else
-                            __builtin_nontemporal_store(
-                                static_cast<WU>(v[u]), reinterpret_cast<WU*>(tensor + toff[u]));
-                    }
-            }
-            else
-            {
-#pragma unroll
-                for (int u = 0; u < kCopyUnroll; ++u)
-                    if (g[u] < count)
-                    {
-                        WU t = *reinterpret_cast<const WU*>(tensor + toff[u]);
-#pragma unroll
-                        for (int j = 0; j < VEC; ++j)
-                            t[j] = op(t[j], v[u][j]);
-                        *reinterpret_cast<WU*>(tensor + toff[u]) = t;
-                    }
-            }
-        }
-        else if (mode == kTransfer)
-        {
-            // `buffer` is the origin of the source box in the other tensor
-            WU v[kCopyUnroll];
-            if constexpr (SPARSE)
-            {
-                // both faces' loads before any store, as for sparse packs
-                if (side == 1)
-                    break;
-                T* const tensor_b = reinterpret_cast<T*>(box.tensor2);
-                const T* const source_b = reinterpret_cast<const T*>(box.buffer2);
-                WU w[kCopyUnroll];
-#pragma unroll
-                for (int u = 0; u < kCopyUnroll; ++u)
-                    if (g[u] < count)
-                    {
-                        v[u] = *reinterpret_cast<const WU*>(buffer + soff[u]);
-                        if (tensor_b != nullptr)
-                            w[u] = *reinterpret_cast<const WU*>(source_b + soff[u]);
-                    }
-#pragma unroll
-                for (int u = 0; u < kCopyUnroll; ++u)
-                    if (g[u] < count)
-                    {
-                        if constexpr (std::is_same<Op, OpId>::value && VEC == 1)
-                        {
-                            sparse_store_scalar(tensor + toff[u], v[u][0]);
-                            if (tensor_b != nullptr)
-                                sparse_store_scalar(tensor_b + toff[u], w[u][0]);
-                        }
-                        else
-                        {
-                            WU t = *reinterpret_cast<const WU*>(tensor + toff[u]);
-#pragma unroll
-                            for (int j = 0; j < VEC; ++j)
-                                t[j] = op(t[j], v[u][j]);
-                            *reinterpret_cast<WU*>(tensor + toff[u]) = t;
-                            if (tensor_b != nullptr)
-                            {
-                                WU tb = *reinterpret_cast<const WU*>(tensor_b + toff[u]);
-#pragma unroll
-                                for (int j = 0; j < VEC; ++j)
-                                    tb[j] = op(tb[j], w[u][j]);
-                                *reinterpret_cast<WU*>(tensor_b + toff[u]) = tb;
-                            }
-                        }
-                    }
-            }
-            else
-            {
-#pragma unroll
-                for (int u = 0; u < kCopyUnroll; ++u)
-                    if (g[u] < count)
-                        v[u] = __builtin_nontemporal_load(
-                            reinterpret_cast<const WU*>(buffer + soff[u]));
-#pragma unroll
-                for (int u = 0; u < kCopyUnroll; ++u)
-                    if (g[u] < count)
-                    {
-                        if constexpr (std::is_same<Op, OpId>::value)
-                        {
-                            __builtin_nontemporal_store(
-                                v[u], reinterpret_cast<WU*>(tensor + toff[u]));
-                        }
-                        else
-                        {
-                            WU t = *reinterpret_cast<const WU*>(tensor + toff[u]);
-#pragma unroll
-                            for (int j = 0; j < VEC; ++j)
-                                t[j] = op(t[j], v[u][j]);
-                            *reinterpret_cast<WU*>(tensor + toff[u]) = t;
-                        }
-                    }
-            }
-        }
-        else
-        {
-#pragma unroll
-            for (int u = 0; u < kCopyUnroll; ++u)
-                if (g[u] < count)
-                {
-                    if constexpr (SPARSE && VEC == 1)
-                    {
-                        sparse_store_scalar(tensor + toff[u], T(0));
-                    }
-                    else
-                    {
-                        WU z;
-#pragma unroll
-                        for (int j = 0; j < VEC; ++j)
-                            z[j] = T(0);
-                        *reinterpret_cast<WU*>(tensor + toff[u]) = z;
-                    }
-                }
-        }
-    }
+    return s.sparse ? launch_mode<T, VEC, true>(s, batch) : launch_mode<T, VEC, false>(s, batch);
 }
+
+template <typename T, int VEC>
+int launch_table_mode(const LaunchShape& s, const TableBatch& batch)
+{
+    const dim3 grid(s.grid);
+    if (s.mode == kPack)
+        box_copy_kernel<T, VEC, OpId, false, kPack, true><<<grid, kCopyBlock, 0, s.stream>>>(batch, OpId());
+    else if (s.mode == kUnpack)
+        box_copy_kernel<T, VEC, OpId, false, kUnpack, true><<<grid, kCopyBlock, 0, s.stream>>>(batch, OpId());
+    else
+        return H2X_ERR_UNSUPPORTED;
+    return launch_status();
+}
+
+} // namespace
+
+int launch_identity(const LaunchShape& s, const BoxBatch& batch)
+{
+    switch (s.elem_size * 16 + s.vec)
+    {
+    case 2 * 16 + 8: return launch_sparse<uint16_t, 8>(s, batch);
+    case 2 * 16 + 4: return launch_sparse<uint16_t, 4>(s, batch);
+    case 2 * 16 + 2: return launch_sparse<uint16_t, 2>(s, batch);
+    case 2 * 16 + 1: return launch_sparse<uint16_t, 1>(s, batch);
+    case 4 * 16 + 4: return launch_sparse<uint32_t, 4>(s, batch);
+    case 4 * 16 + 2: return launch_sparse<uint32_t, 2>(s, batch);
+    case 4 * 16 + 1: return launch_sparse<uint32_t, 1>(s, batch);
+    case 8 * 16 + 2: return launch_sparse<uint64_t, 2>(s, batch);
+    case 8 * 16 + 1: return launch_sparse<uint64_t, 1>(s, batch);
+    }
+    return H2X_ERR_UNSUPPORTED;
+}
+
+int launch_tables(const LaunchShape& s, const TableBatch& batch)
+{
+    switch (s.elem_size * 16 + s.vec)
+    {
+    case 2 * 16 + 8: return launch_table_mode<uint16_t, 8>(s, batch);
+    case 2 * 16 + 4: return launch_table_mode<uint16_t, 4>(s, batch);
+    case 2 * 16 + 2: return launch_table_mode<uint16_t, 2>(s, batch);
+    case 2 * 16 + 1: return launch_table_mode<uint16_t, 1>(s, batch);
+    case 4 * 16 + 4: return launch_table_mode<uint32_t, 4>(s, batch);
+    case 4 * 16 + 2: return launch_table_mode<uint32_t, 2>(s, batch);
+    case 4 * 16 + 1: return launch_table_mode<uint32_t, 1>(s, batch);
+    case 8 * 16 + 2: return launch_table_mode<uint64_t, 2>(s, batch);
+    case 8 * 16 + 1: return launch_table_mode<uint64_t, 1>(s, batch);
+    }
+    return H2X_ERR_UNSUPPORTED;
+}
+
+} // namespace copy
+
+using namespace copy;
+
+namespace
+{
 
 // ---- host: box reduction ------------------------------------------------------
 
@@ -426,27 +179,45 @@ HostBox reduce_box(int nd, const int64_t* extent, const int64_t* stride, int64_t
     return h;
 }
 
-// Largest power-of-two vector (elements, at most 16 bytes) that never crosses a
-// run of the box and keeps the buffer side aligned.
-int box_vector(const HostBox& h, int elem_size, const void* buffer)
+// Vector width (elements, at most 16 bytes) of a box.  The image side must be
+// aligned to it.  Runs that are a multiple of it move in whole vectors; longer
+// runs of any other length still move in 16-byte vectors indexed from the
+// image side, and the few vectors that straddle the end of a run are split
+// (`ragged`): a 130-element row is 32 vectors and one straddler instead of 65
+// 8-byte pieces.
+constexpr int64_t kMinRaggedRun = 16; // shorter runs: straddlers would be the rule
+
+int box_vector(const HostBox& h, int elem_size, const void* buffer, bool allow_ragged, bool* ragged)
 {
+    *ragged = false;
     int v = 16 / elem_size;
     if (h.stride[0] != 1 || (h.transfer && h.stride_src[0] != 1))
         return 1;
+    // a transfer has no image side: both tensors take unaligned vectors
+    auto buffer_ok = [&](int w) {
+        return h.transfer
+               || (h.buffer_offset % w == 0
+                   && reinterpret_cast<uintptr_t>(buffer) % (static_cast<size_t>(w) * elem_size) == 0);
+    };
+    if (allow_ragged && v > 1 && h.extent[0] % v != 0 && h.extent[0] >= kMinRaggedRun && buffer_ok(v))
+    {
+        *ragged = true;
+        return v;
+    }
     while (v > 1)
     {
-        // a transfer has no buffer side: both tensors take unaligned vectors
-        const bool ok = h.extent[0] % v == 0
-                        && (h.transfer
-                            || (h.buffer_offset % v == 0
-                                && reinterpret_cast<uintptr_t>(buffer)
-                                           % (static_cast<size_t>(v) * elem_size)
-                                       == 0));
-        if (ok)
+        if (h.extent[0] % v == 0 && buffer_ok(v))
             break;
         v /= 2;
     }
     return v;
+}
+
+// sparse: every run is shorter than a cache line and the runs are apart
+bool box_is_sparse(const HostBox& h, int elem_size)
+{
+    return h.nd > 1 ? h.extent[0] * h.stride[0] * elem_size < 128
+                    : (h.stride[0] != 1 && h.extent[0] > 1);
 }
 
 bool same_geometry(const HostBox& a, const HostBox& b)
@@ -460,6 +231,34 @@ bool same_geometry(const HostBox& a, const HostBox& b)
     return true;
 }
 
+// Geometry of a device descriptor; pointers and flags are the caller's.
+void fill_box(Box* b, const HostBox& h)
+{
+    for (int i = 0; i < kMaxBoxDims; ++i)
+    {
+        b->stride[i] = i < h.nd ? h.stride[i] : 0;
+        b->stride_src[i] = i < h.nd ? h.stride_src[i] : 0;
+        b->div[i] = make_fastdiv(i < h.nd ? static_cast<uint32_t>(h.extent[i]) : 1u);
+    }
+    b->count = static_cast<uint32_t>(h.count);
+    b->first_block = 0;
+    b->ragged = 0;
+    b->seam = 0;
+    b->deep = h.nd > 3;
+    b->reserved = 0;
+    b->tensor2 = nullptr;
+    b->buffer2 = nullptr;
+}
+
+uint64_t box_blocks(int64_t count, int vec)
+{
+    const uint64_t per_block = static_cast<uint64_t>(kCopyBlock) * vec * kCopyUnroll;
+    return (static_cast<uint64_t>(count) + per_block - 1) / per_block;
+}
+
+// Queues boxes whose descriptors travel in the kernel arguments and launches
+// them, kMaxBoxes at a time; boxes of one launch share vector width, kind
+// (sparse or dense) and mode.
 struct Launcher
 {
     hipStream_t stream;
@@ -468,90 +267,14 @@ struct Launcher
     int op;          // h2x_halo_op
     int vec = 0;
     bool sparse = false;
-    HostBox last;         // geometry of the most recently queued box
-    int last_mode = -1;
-    uint32_t launch_blocks = 0; // workgroups of the launch being issued
+    int mode = -1;
+    HostBox last;    // geometry of the most recently queued box
+    uint32_t num_blocks = 0;
     BoxBatch batch;
 
     Launcher(hipStream_t s, int es, h2x_dtype dt, int o) : stream(s), elem_size(es), dtype(dt), op(o)
     {
         batch.num_boxes = 0;
-        batch.num_blocks = 0;
-    }
-
-    template <typename T, int VEC>
-    int launch_typed()
-    {
-        const dim3 grid(launch_blocks);
-        switch (op)
-        {
-        case H2X_HALO_ID:
-            if (sparse)
-                box_copy_kernel<T, VEC, OpId, true><<<grid, kBlockSize, 0, stream>>>(batch, OpId());
-            else
-                box_copy_kernel<T, VEC, OpId, false><<<grid, kBlockSize, 0, stream>>>(batch, OpId());
-            break;
-        default: return H2X_ERR_UNSUPPORTED;
-        }
-        return launch_status();
-    }
-
-    template <typename T, int VEC>
-    int launch_accumulate()
-    {
-        const dim3 grid(launch_blocks);
-        switch (op)
-        {
-        case H2X_HALO_SUM:
-            if (sparse)
-                box_copy_kernel<T, VEC, OpSum, true><<<grid, kBlockSize, 0, stream>>>(batch, OpSum());
-            else
-                box_copy_kernel<T, VEC, OpSum, false><<<grid, kBlockSize, 0, stream>>>(batch, OpSum());
-            break;
-        case H2X_HALO_MAX:
-            if (sparse)
-                box_copy_kernel<T, VEC, OpMax, true><<<grid, kBlockSize, 0, stream>>>(batch, OpMax());
-            else
-                box_copy_kernel<T, VEC, OpMax, false><<<grid, kBlockSize, 0, stream>>>(batch, OpMax());
-            break;
-        case H2X_HALO_MIN:
-            if (sparse)
-                box_copy_kernel<T, VEC, OpMin, true><<<grid, kBlockSize, 0, stream>>>(batch, OpMin());
-            else
-                box_copy_kernel<T, VEC, OpMin, false><<<grid, kBlockSize, 0, stream>>>(batch, OpMin());
-            break;
-        default: return H2X_ERR_UNSUPPORTED;
-        }
-        return launch_status();
-    }
-
-    template <typename U, typename F, int V>
-    int launch_width()
-    {
-        if constexpr (!std::is_void<F>::value)
-            if (op != H2X_HALO_ID)
-                return launch_accumulate<F, V>();
-        return launch_typed<U, V>();
-    }
-
-    template <typename U, typename F>
-    int launch_vec()
-    {
-        constexpr int kFull = 16 / sizeof(U);
-        switch (vec)
-        {
-        case 8:
-            if constexpr (kFull >= 8)
-                return launch_width<U, F, 8>();
-            break;
-        case 4:
-            if constexpr (kFull >= 4)
-                return launch_width<U, F, 4>();
-            break;
-        case 2: return launch_width<U, F, 2>();
-        case 1: return launch_width<U, F, 1>();
-        }
-        return H2X_ERR_UNSUPPORTED;
     }
 
     int flush()
@@ -562,62 +285,61 @@ struct Launcher
         // surplus workgroups of smaller boxes find nothing to do; if they would
         // more than double the grid, the boxes follow one another instead.
         batch.blocks_per_box = 0;
-        uint32_t grid_blocks = batch.num_blocks;
+        uint32_t grid_blocks = num_blocks;
         if (batch.num_boxes > 1)
         {
             uint32_t most = 0;
             for (int i = 0; i < batch.num_boxes; ++i)
             {
-                const uint32_t end = i + 1 < batch.num_boxes ? batch.box[i + 1].first_block
-                                                             : batch.num_blocks;
+                const uint32_t end = i + 1 < batch.num_boxes ? batch.box[i + 1].first_block : num_blocks;
                 most = std::max(most, end - batch.box[i].first_block);
             }
             const uint64_t turns = static_cast<uint64_t>(most) * batch.num_boxes;
-            if (turns <= 2ull * batch.num_blocks && turns <= 0x7fffffffull)
+            if (turns <= 2ull * num_blocks && turns <= 0x7fffffffull)
             {
                 batch.blocks_per_box = most;
                 grid_blocks = static_cast<uint32_t>(turns);
             }
         }
-        launch_blocks = grid_blocks;
-        int err;
-        switch (elem_size)
-        {
-        case 2: err = op == H2X_HALO_ID ? launch_vec<uint16_t, void>() : H2X_ERR_UNSUPPORTED; break;
-        case 4: err = launch_vec<uint32_t, float>(); break;
-        case 8: err = launch_vec<uint64_t, double>(); break;
-        default: err = H2X_ERR_UNSUPPORTED;
-        }
+        LaunchShape shape{elem_size, op, vec, sparse, mode, grid_blocks, stream};
+        const int err = op == H2X_HALO_ID ? launch_identity(shape, batch)
+                                          : launch_accumulate(shape, dtype, batch);
         batch.num_boxes = 0;
-        batch.num_blocks = 0;
+        num_blocks = 0;
         vec = 0;
-        last_mode = -1;
+        mode = -1;
         return err;
     }
 
     // Queues one box; launches what is queued when the batch is full or the
-    // new box needs another vector width.
-    int add(const HostBox& h, void* tensor, void* buffer, int mode)
+    // new box needs another kernel.
+    int add(const HostBox& h, void* tensor, void* buffer, int box_mode)
     {
         if (h.count == 0)
             return H2X_SUCCESS;
         if (h.count >= (1ll << 31))
             return H2X_ERR_TOO_LARGE;
-        const int v = mode == kClear ? box_vector(h, elem_size, nullptr) : box_vector(h, elem_size, buffer);
-        // sparse: every run is shorter than a cache line and the runs are apart
-        const bool sp = h.nd > 1 ? h.extent[0] * h.stride[0] * elem_size < 128
-                                 : (h.stride[0] != 1 && h.extent[0] > 1);
+        const bool sp = box_is_sparse(h, elem_size);
+        bool rg;
+        const int v = box_vector(h, elem_size, box_mode == kClear ? nullptr : buffer, !sp, &rg);
         char* const tptr = static_cast<char*>(tensor) + h.tensor_offset * elem_size;
         char* const bptr = static_cast<char*>(buffer) + h.buffer_offset * elem_size;
         // second box of a sparse pair: same geometry and mode as the box queued last
-        if (sp && batch.num_boxes > 0 && sparse && v == vec && last_mode == mode
+        if (sp && batch.num_boxes > 0 && sparse && v == vec && mode == box_mode
             && batch.box[batch.num_boxes - 1].tensor2 == nullptr && same_geometry(h, last))
         {
-            batch.box[batch.num_boxes - 1].tensor2 = tptr;
-            batch.box[batch.num_boxes - 1].buffer2 = bptr;
+            Box& first = batch.box[batch.num_boxes - 1];
+            first.tensor2 = tptr;
+            first.buffer2 = bptr;
+            // one element per row on each side, and this box's element of a row
+            // lies directly in front of the first box's element of the next row
+            // (the RHS and the LHS halo cell at a row seam): unpacked in one store
+            first.seam = box_mode == kUnpack && v == 1 && h.nd == 1
+                         && tptr + elem_size == first.tensor + h.stride[0] * elem_size;
             return H2X_SUCCESS;
         }
-        if (batch.num_boxes == kMaxBoxes || (batch.num_boxes > 0 && (v != vec || sp != sparse)))
+        if (batch.num_boxes == kMaxBoxes
+            || (batch.num_boxes > 0 && (v != vec || sp != sparse || box_mode != mode)))
         {
             const int err = flush();
             if (err != 0)
@@ -625,31 +347,43 @@ struct Launcher
         }
         vec = v;
         sparse = sp;
+        mode = box_mode;
         last = h;
-        last_mode = mode;
         Box& b = batch.box[batch.num_boxes];
+        fill_box(&b, h);
         b.tensor = tptr;
         b.buffer = bptr;
-        b.tensor2 = nullptr;
-        b.buffer2 = nullptr;
-        for (int i = 0; i < kMaxBoxDims; ++i)
-        {
-            b.stride[i] = i < h.nd ? h.stride[i] : 0;
-            b.stride_src[i] = i < h.nd ? h.stride_src[i] : 0;
-            b.div[i] = make_fastdiv(i < h.nd ? static_cast<uint32_t>(h.extent[i]) : 1u);
-        }
-        b.count = static_cast<uint32_t>(h.count);
-        b.first_block = batch.num_blocks;
-        b.num_dims = h.nd;
-        b.mode = mode;
-        const uint64_t per_block = static_cast<uint64_t>(kBlockSize) * v * kCopyUnroll;
-        const uint64_t blocks = (static_cast<uint64_t>(h.count) + per_block - 1) / per_block;
-        if (batch.num_blocks + blocks > 0x7fffffffull)
+        b.ragged = rg;
+        b.first_block = num_blocks;
+        const uint64_t blocks = box_blocks(h.count, v);
+        if (num_blocks + blocks > 0x7fffffffull)
             return H2X_ERR_TOO_LARGE;
-        batch.num_blocks += static_cast<uint32_t>(blocks);
+        num_blocks += static_cast<uint32_t>(blocks);
         ++batch.num_boxes;
         return H2X_SUCCESS;
     }
+};
+
+// The reduced boxes of one call: on the stack for the usual handful of faces,
+// on the heap beyond that.
+class BoxList
+{
+public:
+    explicit BoxList(int n) : m_data(m_local)
+    {
+        if (n > kLocal)
+        {
+            m_heap.resize(static_cast<size_t>(n));
+            m_data = m_heap.data();
+        }
+    }
+    HostBox& operator[](int i) { return m_data[i]; }
+
+private:
+    static constexpr int kLocal = 32;
+    HostBox m_local[kLocal];
+    std::vector<HostBox> m_heap;
+    HostBox* m_data;
 };
 
 int elem_size_of(h2x_dtype dtype)
@@ -718,7 +452,8 @@ extern "C" int h2x_halo_pack_or_unpack_batched(h2x_dtype dtype, const h2x_halo_f
     if (num_faces < 0 || (num_faces > 0 && !faces))
         return H2X_ERR_INVALID_ARGUMENT;
     // validate everything before anything is launched
-    std::vector<HostBox> boxes(num_faces);
+    BoxList boxes(num_faces);
+    unsigned int ops_present = 0;
     for (int i = 0; i < num_faces; ++i)
     {
         const int err = halo_box(faces[i], &boxes[i]);
@@ -730,10 +465,13 @@ extern "C" int h2x_halo_pack_or_unpack_batched(h2x_dtype dtype, const h2x_halo_f
             return H2X_ERR_TOO_LARGE;
         if (faces[i].op < H2X_HALO_ID || faces[i].op > H2X_HALO_MIN)
             return H2X_ERR_INVALID_ARGUMENT;
+        ops_present |= 1u << (faces[i].is_pack ? H2X_HALO_ID : faces[i].op);
     }
     // faces with the same effective op share launches
     for (int op = H2X_HALO_ID; op <= H2X_HALO_MIN; ++op)
     {
+        if (!(ops_present & (1u << op)))
+            continue;
         Launcher l(as_stream(stream), es, dtype, op);
         for (int i = 0; i < num_faces; ++i)
         {
@@ -819,7 +557,8 @@ extern "C" int h2x_halo_exchange_fused(h2x_dtype dtype, const h2x_halo_transfer*
     if (num_transfers < 0 || (num_transfers > 0 && !transfers))
         return H2X_ERR_INVALID_ARGUMENT;
     // validate everything before anything is launched
-    std::vector<HostBox> boxes(num_transfers);
+    BoxList boxes(num_transfers);
+    unsigned int ops_present = 0;
     for (int i = 0; i < num_transfers; ++i)
     {
         const h2x_halo_transfer& t = transfers[i];
@@ -869,9 +608,12 @@ extern "C" int h2x_halo_exchange_fused(h2x_dtype dtype, const h2x_halo_transfer*
             return H2X_ERR_INVALID_ARGUMENT;
         if (boxes[i].count >= (1ll << 31))
             return H2X_ERR_TOO_LARGE;
+        ops_present |= 1u << t.op;
     }
     for (int op = H2X_HALO_ID; op <= H2X_HALO_MIN; ++op)
     {
+        if (!(ops_present & (1u << op)))
+            continue;
         Launcher l(as_stream(stream), es, dtype, op);
         for (int i = 0; i < num_transfers; ++i)
         {
@@ -895,7 +637,63 @@ struct h2x_shuffle_plan
 {
     int elem_size;
     std::vector<HostBox> boxes; // one per peer with a non-empty intersection
+    // Device table of the same boxes for launches that take their descriptors
+    // from memory (null if the plan does not qualify: sparse boxes).  Entries
+    // hold byte offsets where a launch from kernel arguments holds addresses.
+    Box* table = nullptr;
+    int table_device = -1;
+    int table_vec = 0;         // vector width the table's `ragged` flags were made for
+    uint32_t most_blocks = 0;  // workgroups of the largest box at table_vec
+    uint64_t total_blocks = 0; // over all boxes
 };
+
+namespace
+{
+
+// Builds the device table of a plan.  Assumes buffers aligned to 16 bytes; a
+// launch with a less aligned buffer goes through the kernel arguments instead.
+int make_table(h2x_shuffle_plan* p)
+{
+    const int n = static_cast<int>(p->boxes.size());
+    if (n == 0)
+        return H2X_SUCCESS;
+    int vec = 16 / p->elem_size;
+    for (const HostBox& h : p->boxes)
+    {
+        if (box_is_sparse(h, p->elem_size))
+            return H2X_SUCCESS; // pairs of sparse boxes are formed per launch
+        bool rg;
+        vec = std::min(vec, box_vector(h, p->elem_size, nullptr, true, &rg));
+    }
+    std::vector<Box> host(static_cast<size_t>(n));
+    for (int i = 0; i < n; ++i)
+    {
+        const HostBox& h = p->boxes[i];
+        fill_box(&host[i], h);
+        host[i].tensor = reinterpret_cast<char*>(static_cast<intptr_t>(h.tensor_offset * p->elem_size));
+        host[i].buffer = reinterpret_cast<char*>(static_cast<intptr_t>(h.buffer_offset * p->elem_size));
+        host[i].ragged = vec > 1 && h.extent[0] % vec != 0;
+        const uint64_t blocks = box_blocks(h.count, vec);
+        p->most_blocks = std::max<uint64_t>(p->most_blocks, blocks);
+        p->total_blocks += blocks;
+    }
+    hipError_t err = hipGetDevice(&p->table_device);
+    if (err == hipSuccess)
+        err = hipMalloc(reinterpret_cast<void**>(&p->table), sizeof(Box) * host.size());
+    if (err == hipSuccess)
+        err = hipMemcpy(p->table, host.data(), sizeof(Box) * host.size(), hipMemcpyHostToDevice);
+    if (err != hipSuccess)
+    {
+        if (p->table)
+            (void) hipFree(p->table);
+        p->table = nullptr;
+        return static_cast<int>(err);
+    }
+    p->table_vec = vec;
+    return H2X_SUCCESS;
+}
+
+} // namespace
 
 extern "C" int h2x_shuffle_plan_create(const h2x_shuffle_geometry* g, h2x_shuffle_plan** plan)
 {
@@ -962,14 +760,98 @@ extern "C" int h2x_shuffle_plan_create(const h2x_shuffle_geometry* g, h2x_shuffl
         }
         p->boxes.push_back(h);
     }
+    const int err = make_table(p);
+    if (err != 0)
+    {
+        delete p;
+        return err;
+    }
     *plan = p;
     return H2X_SUCCESS;
 }
 
 extern "C" int h2x_shuffle_plan_destroy(h2x_shuffle_plan* plan)
 {
+    if (plan && plan->table)
+        (void) hipFree(plan->table);
     delete plan;
     return H2X_SUCCESS;
+}
+
+// All plans of a call through their device tables, kMaxPlans per launch.
+// Returns false (nothing launched) if the call does not qualify: a plan
+// without a table or made on another device, mixed element sizes or vector
+// widths, a buffer that is not 16-byte aligned, or boxes so unequal that
+// taking turns would more than double the grid.
+static bool shuffle_through_tables(const h2x_shuffle_plan* const* plans, void* const* tensors,
+                                   void* const* buffers, int num_plans, int mode,
+                                   h2x_stream_t stream, int* status)
+{
+    int device = -1;
+    if (hipGetDevice(&device) != hipSuccess)
+        return false;
+    const h2x_shuffle_plan* first = nullptr;
+    uint32_t most = 0;
+    uint64_t total = 0, boxes = 0;
+    for (int i = 0; i < num_plans; ++i)
+    {
+        const h2x_shuffle_plan* p = plans[i];
+        if (p->boxes.empty())
+            continue;
+        if (!p->table || p->table_device != device
+            || reinterpret_cast<uintptr_t>(buffers[i]) % 16 != 0)
+            return false;
+        if (!first)
+            first = p;
+        if (p->elem_size != first->elem_size || p->table_vec != first->table_vec)
+            return false;
+        most = std::max(most, p->most_blocks);
+        total += p->total_blocks;
+        boxes += p->boxes.size();
+    }
+    *status = H2X_SUCCESS;
+    if (!first)
+        return true; // nothing to move
+    if (static_cast<uint64_t>(most) * boxes > 2 * total)
+        return false;
+    int i = 0;
+    while (i < num_plans)
+    {
+        TableBatch batch;
+        batch.num_plans = 0;
+        batch.num_boxes = 0;
+        batch.reserved = 0;
+        uint32_t launch_most = 0;
+        for (; i < num_plans && batch.num_plans < kMaxPlans; ++i)
+        {
+            const h2x_shuffle_plan* p = plans[i];
+            if (p->boxes.empty())
+                continue;
+            PlanRef& ref = batch.plan[batch.num_plans++];
+            ref.table = p->table;
+            ref.tensor = static_cast<char*>(tensors[i]);
+            ref.buffer = static_cast<char*>(buffers[i]);
+            ref.first_box = batch.num_boxes;
+            ref.reserved = 0;
+            batch.num_boxes += static_cast<uint32_t>(p->boxes.size());
+            launch_most = std::max(launch_most, p->most_blocks);
+        }
+        if (batch.num_plans == 0)
+            break;
+        const uint64_t grid = static_cast<uint64_t>(launch_most) * batch.num_boxes;
+        if (grid > 0x7fffffffull)
+        {
+            *status = H2X_ERR_TOO_LARGE;
+            return true;
+        }
+        batch.blocks_per_box = launch_most;
+        LaunchShape shape{first->elem_size, H2X_HALO_ID, first->table_vec, false, mode,
+                          static_cast<uint32_t>(grid), as_stream(stream)};
+        *status = launch_tables(shape, batch);
+        if (*status != 0)
+            return true;
+    }
+    return true;
 }
 
 static int shuffle_batched(const h2x_shuffle_plan* const* plans, void* const* tensors,
@@ -984,6 +866,9 @@ static int shuffle_batched(const h2x_shuffle_plan* const* plans, void* const* te
         if (!plans[i]->boxes.empty() && (!tensors[i] || !buffers[i]))
             return H2X_ERR_INVALID_ARGUMENT;
     }
+    int status = H2X_SUCCESS;
+    if (shuffle_through_tables(plans, tensors, buffers, num_plans, mode, stream, &status))
+        return status;
     for (int es : {2, 4, 8})
     {
         Launcher l(as_stream(stream), es, H2X_F32, H2X_HALO_ID);

@@ -46,9 +46,7 @@ inline FastDiv make_fastdiv(uint32_t d)
     FastDiv f{d, 0u, 0u};
     if (d > 1)
     {
-        uint32_t log2 = 0;
-        while ((1ull << log2) < d)
-            ++log2;
+        const uint32_t log2 = 32u - static_cast<uint32_t>(__builtin_clz(d - 1)); // ceil(log2 d), d >= 2
         const uint32_t p = 31 + log2;
         f.multiplier = static_cast<uint32_t>(((1ull << p) + d - 1) / d);
         f.shift = p - 32;

@@ -447,13 +447,14 @@ public:
     // Ranks that exchange dimension `dim` together, group after group.  Faces
     // of the innermost dimension touch one short run per row, each costing a
     // 128-byte line, and the unpack writes into the lines its rank's pack has
-    // just read: a group is kept small enough for those lines to stay in the
-    // 256 MB memory-side cache between the two launches.  Neighbours along
-    // `dim` always share a group.
+    // just read: a group is kept small enough (160 MB of lines) for those
+    // lines to stay in the 256 MB memory-side cache between the two launches,
+    // where the unpack's partial writes merge into whole lines.  Neighbours
+    // along `dim` always share a group.
     std::vector<std::vector<int>> rank_groups(int dim, int width) const
     {
         constexpr size_t kLineBytes = 128;
-        constexpr size_t kGroupBytes = size_t(320) << 20;
+        constexpr size_t kGroupBytes = size_t(160) << 20;
         std::vector<std::vector<int>> groups;
         if (dim != 0 || width * sizeof(DataType) >= kLineBytes)
         {

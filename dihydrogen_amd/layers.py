@@ -524,10 +524,11 @@ class HaloExchangeVirtual:
     # Faces of the innermost dimension touch one short run per row, and every
     # run costs a whole 128-byte line of memory traffic; the unpack writes into
     # the lines its rank's pack has just read.  Exchanging a few ranks at a time
-    # keeps those lines in the 256 MB memory-side cache between the two launches
-    # (measured on the 8-rank, 130^3 x 32 case: two groups of four ranks take
-    # 340 us, one group of eight 380 us).
-    _SPARSE_GROUP_BYTES = 320 << 20
+    # keeps those lines in the 256 MB memory-side cache between the two launches,
+    # where the unpack's partial writes merge into whole lines (measured on the
+    # 8-rank, 130^3 x 32 case: groups of two ranks, 138 MB of lines, take 275 us,
+    # groups of four 290 us, all eight at once more than 300 us).
+    _SPARSE_GROUP_BYTES = 160 << 20
     _LINE_BYTES = 128
 
     def _rank_groups(self, dim: int, width: int) -> List[List[int]]:

@@ -61,6 +61,62 @@ def test_accumulate_ops(op, dtype, oracle_mod):
             _single_face((4, 4, 8, 12), dim, side, 1, False, False, op, dtype, oracle_mod)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("real_shape_np", [(2, 3, 5, 21), (1, 2, 4, 6, 19), (1, 2, 3, 130), (2, 2, 3, 3, 34)])
+def test_rows_that_are_no_multiple_of_the_vector(real_shape_np, dtype, oracle_mod):
+    """Runs of 17..130 elements move in 16-byte vectors indexed from the buffer
+    side; the vectors that straddle a row end, and the last one of a strip whose
+    size is no multiple of 4, go element by element.  Every dimension whose strip
+    has such runs, both sides, widths 1-3, pack, unpack and an accumulating unpack."""
+    nd = len(real_shape_np)
+    shape = real_shape_np[::-1]
+    for dim, side in itertools.product(range(1, nd), (0, 1)):
+        for width in (1, 2, 3):
+            if 2 * width > shape[dim]:
+                continue
+            _single_face(real_shape_np, dim, side, width, True, False, 0, dtype, oracle_mod)
+            _single_face(real_shape_np, dim, side, width, False, False, 0, dtype, oracle_mod)
+            _single_face(real_shape_np, dim, side, width, False, True, 1, dtype, oracle_mod)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("op", [0, 1, 2])
+def test_both_faces_of_the_innermost_dimension_in_one_call(op, dtype, oracle_mod):
+    """LHS and RHS face of dimension 0, width 1, unpacked by one batched call: the
+    RHS halo cell of a row and the LHS halo cell of the next row are neighbours in
+    memory and are written together.  Identity and accumulating ops, against
+    the oracle's two separate unpacks; then the same pair packed."""
+    import torch
+    from dihydrogen_amd import capi
+    lib = capi.load()
+    real_np = (2, 3, 7, 9)
+    shape = real_np[::-1]
+    rng = np.random.default_rng(17 + op)
+    t = rng.uniform(-1, 1, real_np).astype(dtype)
+    n = oracle_mod.halo_size(shape, 0, 1)
+    bufs = [rng.uniform(-1, 1, n).astype(dtype) for _ in range(2)]
+    h2x_dt = capi.F32 if dtype == np.float32 else capi.F64
+    for is_pack in (False, True):
+        t_o, b_o = t.copy(), [b.copy() for b in bufs]
+        for side in (0, 1):
+            oracle_mod.halo_pack_or_unpack(t_o, 0, side, 1, b_o[side], is_pack, False, op)
+        td = torch.from_numpy(t).cuda()
+        bd = [torch.from_numpy(b).cuda() for b in bufs]
+        faces = (capi.HaloFace * 2)()
+        for side in (0, 1):
+            f = faces[side]
+            f.tensor, f.buffer = td.data_ptr(), bd[side].data_ptr()
+            for i, e in enumerate(shape):
+                f.real_shape[i] = e
+            f.num_dims, f.dim, f.side, f.width = len(shape), 0, side, 1
+            f.inner, f.is_pack, f.op = int(is_pack), int(is_pack), op
+        capi.check(lib.h2x_halo_pack_or_unpack_batched(h2x_dt, faces, 2, None))
+        torch.cuda.synchronize()
+        assert np.array_equal(td.cpu().numpy(), t_o)
+        for side in (0, 1):
+            assert np.array_equal(bd[side].cpu().numpy(), b_o[side])
+
+
 def _exchange_case(shape, locale, overlap, periodic, oracle_mod, widths=None, dtype=np.float32,
                    fused=False):
     """Runs the exchange on the GPU and on the CPU oracle; returns both."""

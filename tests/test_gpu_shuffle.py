@@ -29,6 +29,9 @@ CASES = {
     "five_d": ((6, 8, 4, 2, 4), ((1, 1, 1, 1, 4), None, None), ((1, 2, 2, 1, 1), None, (0, 1, 1, 0, 0))),
     "sixteen_ranks_even": ((32, 4, 2, 16), ((1, 1, 1, 16), None, None), ((16, 1, 1, 1), None, None)),
     "empty_ranks": ((2, 8, 2, 4), ((1, 1, 1, 4), None, None), ((4, 1, 1, 1), None, None)),
+    # runs of 19 and 18 elements (and 37 when rows are whole): 16-byte vectors with straddlers
+    "odd_runs": ((37, 6, 3, 4), ((1, 1, 1, 4), None, None), ((2, 2, 1, 1), None, None)),
+    "odd_runs_halo": ((37, 5, 2, 4), ((1, 1, 1, 4), None, None), ((2, 2, 1, 1), None, (1, 1, 0, 0))),
 }
 
 
@@ -89,7 +92,8 @@ def interior_slices_of(t):
 
 
 @pytest.mark.parametrize("case", ["sample_to_spatial", "uneven", "overlap_to_nonoverlap",
-                                  "sample_to_spatial_halo", "five_d", "sixteen_ranks_even"])
+                                  "sample_to_spatial_halo", "five_d", "sixteen_ranks_even", "odd_runs",
+                                  "odd_runs_halo"])
 @pytest.mark.parametrize("np_dtype", [np.float32, np.int16, np.float64])
 def test_single_rank_pack_unpack_vs_oracle(case, np_dtype, oracle_mod):
     """h2x_shuffle_pack / h2x_shuffle_unpack with the reference's own table
@@ -149,6 +153,50 @@ def test_single_rank_pack_unpack_vs_oracle(case, np_dtype, oracle_mod):
             torch.cuda.synchronize()
             assert np.array_equal(td.cpu().numpy(), field_o)
             lib.h2x_shuffle_plan_destroy(plan)
+
+
+@pytest.mark.parametrize("shift", [1, 2, 3])
+def test_pack_unpack_with_a_buffer_that_is_not_16_byte_aligned(shift, oracle_mod):
+    """Plans keep their boxes in a device table made for 16-byte aligned staging
+    buffers; a buffer that starts `shift` elements later goes through the
+    launch-argument path with narrower vectors.  Same bits either way."""
+    import torch
+    from oracle import geometry as G
+    from dihydrogen_amd import capi
+    lib = capi.load()
+    shape, (sl, ss, so), (dl, ds, do) = CASES["odd_runs"]
+    nd, n = len(shape), int(np.prod(sl))
+    mine = G.TensorGeom(shape, G.Dist(sl, sl, [0] * nd), 1)
+    other = G.TensorGeom(shape, G.Dist(dl, dl, [0] * nd), 1)
+    limits = G.rank_limits(mine, other)
+    counts, displs, _, _ = G.counts_and_displs(mine, other)
+    rng = np.random.default_rng(5)
+    field = rng.integers(-20000, 20000, mine.real_size).astype(np.float32)
+    buf_o = np.zeros(mine.local_size, np.float32)
+    oracle_mod.shuffle_pack_or_unpack(field, mine.local_shape, mine.strides(), other.dist.locale_shape,
+                                      limits, buf_o, displs, True)
+    g = capi.ShuffleGeometry()
+    g.num_dims, g.elem_size = nd, 4
+    for i in range(nd):
+        g.local_shape[i], g.strides[i] = mine.local_shape[i], mine.strides()[i]
+        g.peer_locale_shape[i] = other.dist.locale_shape[i]
+    rl = (ctypes.c_int32 * len(limits))(*limits)
+    dp = (ctypes.c_int32 * len(displs))(*displs)
+    g.rank_limits, g.displs = rl, dp
+    plan = ctypes.c_void_p()
+    capi.check(lib.h2x_shuffle_plan_create(ctypes.byref(g), ctypes.byref(plan)))
+    td = torch.from_numpy(field).cuda()
+    bd = torch.full((mine.local_size + 8,), -1.0, device="cuda")
+    capi.check(lib.h2x_shuffle_pack(plan, td.data_ptr(), bd.data_ptr() + 4 * shift, None))
+    torch.cuda.synchronize()
+    got = bd.cpu().numpy()
+    assert np.array_equal(got[shift:shift + mine.local_size], buf_o)
+    assert (got[:shift] == -1).all() and (got[shift + mine.local_size:] == -1).all()
+    t2 = torch.zeros_like(td)
+    capi.check(lib.h2x_shuffle_unpack(plan, t2.data_ptr(), bd.data_ptr() + 4 * shift, None))
+    torch.cuda.synchronize()
+    assert np.array_equal(t2.cpu().numpy(), field)  # the rank's boxes tile its whole local tensor
+    lib.h2x_shuffle_plan_destroy(plan)
 
 
 def test_plan_rejects_bad_tables():
