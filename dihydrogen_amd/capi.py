@@ -101,6 +101,12 @@ SIGNATURES = {
     "h2x_bn_backprop2": (c_int, [c_int, c_int, c_int, c_size_t, c_size_t, c_size_t, c_size_t,
                                  c_size_t, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_void_p, c_void_p, c_void_p, c_double, c_void_p]),
+    "h2x_bn_forward_local": (c_int, [c_int, c_int, c_int, c_size_t, c_size_t, c_size_t, c_void_p, c_void_p,
+                                     c_void_p, c_size_t, c_double, c_double, c_void_p, c_void_p, c_void_p,
+                                     c_void_p, c_void_p, c_void_p, c_void_p]),
+    "h2x_bn_backward_local": (c_int, [c_int, c_int, c_int, c_size_t, c_size_t, c_size_t, c_size_t, c_size_t,
+                                      c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                      c_void_p, c_void_p, c_void_p, c_double, c_void_p, c_void_p]),
     "h2x_bn_channel_sums_and_sqsums_strided": (c_int, [c_int, c_int, POINTER(TensorGeometry), c_void_p,
                                                        c_void_p, c_void_p, c_void_p, c_void_p]),
     "h2x_bn_batch_normalization_strided": (c_int, [c_int, c_int, POINTER(TensorGeometry),

@@ -212,11 +212,11 @@ __device__ __forceinline__ double inv_sqrt_t(double v)
 // otherwise stores this workgroup's partials for the finishing kernel.
 template <int K>
 __device__ __forceinline__ bool finish_workgroup(double (&acc)[K], double* partials, int channel,
-                                                 int groups_per_channel_max)
+                                                 int groups_per_channel_max, bool always_partials)
 {
     __shared__ double lds[K * kWavesPerBlock];
     block_sum<K>(acc, lds);
-    if (gridDim.x == 1)
+    if (gridDim.x == 1 && !always_partials)
         return true;
     if (threadIdx.x == 0)
     {
@@ -260,13 +260,46 @@ __global__ __launch_bounds__(kBlockSize) void bn_finish_kernel(
     }
 }
 
+// The K sums of channel c from its `groups` partials, in the order of
+// bn_finish_kernel (so a consumer that adds them itself gets the same bits).
+template <int K>
+__device__ __forceinline__ void channel_totals(const double* __restrict__ partials, int groups,
+                                               int groups_per_channel_max, int c, double (&t)[K],
+                                               double* lds)
+{
+    const double* mine = partials + static_cast<size_t>(c) * groups_per_channel_max * K;
+#pragma unroll
+    for (int k = 0; k < K; ++k)
+        t[k] = 0.0;
+    for (int g = threadIdx.x; g < groups; g += kBlockSize)
+    {
+#pragma unroll
+        for (int k = 0; k < K; ++k)
+            t[k] += mine[static_cast<size_t>(g) * K + k];
+    }
+    block_sum<K>(t, lds);
+}
+
+// What the statistics kernel below makes of a channel's sum and sum of squares.
+template <typename T>
+__device__ __forceinline__ void sums_to_mean_var(T sum, T sqsum, T n, T* mean, T* var)
+{
+    const T m = sum / n;
+    const T sqmean = sqsum / n;
+    T v = fma_t(-m, m, sqmean);
+    v = v > T(0) ? v : T(0);
+    v *= n / (n - T(1));
+    *mean = m;
+    *var = v;
+}
+
 // ---- forward: sums and sums of squares --------------------------------------
 // Replaces channel_sums_and_sqsums_opt_kernel, batchnorm.cu:92-132.
 template <typename T, int VEC, bool STRIDED>
 __global__ __launch_bounds__(kBlockSize) void bn_sums_kernel(
     const T* __restrict__ x, T* __restrict__ sums, T* __restrict__ sqsums, double* partials,
     const TensorMap mx, size_t spatial, size_t chunk, int chunks_per_seg, unsigned int num_units,
-    int groups_per_channel_max)
+    int groups_per_channel_max, bool always_partials)
 {
     const int c = blockIdx.y;
     constexpr size_t kStride = static_cast<size_t>(kBlockSize) * VEC;
@@ -313,7 +346,8 @@ __global__ __launch_bounds__(kBlockSize) void bn_sums_kernel(
                 accumulate(v[j]);
         }
     }
-    if (finish_workgroup<2>(acc, partials, c, groups_per_channel_max) && threadIdx.x == 0)
+    if (finish_workgroup<2>(acc, partials, c, groups_per_channel_max, always_partials)
+        && threadIdx.x == 0)
     {
         sums[c] = static_cast<T>(acc[0]);
         sqsums[c] = static_cast<T>(acc[1]);
@@ -343,11 +377,8 @@ __global__ void bn_statistics_kernel(int num_channels, size_t num_per_sum, T dec
             var[c] = T(1);
             continue;
         }
-        const T m = mean[c] / n;
-        const T sqmean = var[c] / n;
-        T v = fma_t(-m, m, sqmean);
-        v = v > T(0) ? v : T(0);
-        v *= n / (n - T(1));
+        T m, v;
+        sums_to_mean_var(mean[c], var[c], n, &m, &v);
         mean[c] = m;
         var[c] = v;
         running_mean[c] = fma_t(decay, running_mean[c], (T(1) - decay) * m);
@@ -355,20 +386,59 @@ __global__ void bn_statistics_kernel(int num_channels, size_t num_per_sum, T dec
     }
 }
 
+// What a consumer kernel needs to finish a reduction itself: the partial sums
+// the reduction kernel left in the workspace, and where the channel results go.
+// Every workgroup of a channel adds that channel's partials in the order of
+// bn_finish_kernel and so arrives at the same bits; the channel's first
+// workgroup stores them.  Saves the finishing launch (and, forward, the
+// statistics launch) when no all-reduce sits between the two stages.
+template <typename T>
+struct FusedStats
+{
+    const double* partials;
+    int groups;
+    int groups_per_channel_max;
+    size_t num_per_sum;
+    T decay;
+    T* out[4];          // forward: mean, var, running_mean, running_var; backward: dscale, dbias, dmean, dvar
+};
+
 // ---- forward: normalise ------------------------------------------------------
-// Replaces batch_normalization_opt_kernel, batchnorm.cu:420-455.
-template <typename T, int VEC, bool STRIDED>
+// Replaces batch_normalization_opt_kernel, batchnorm.cu:420-455.  FUSED: mean
+// and variance are not read but made from the partial sums of bn_sums_kernel
+// (bn_finish_kernel + bn_statistics_kernel folded in).
+template <typename T, int VEC, bool STRIDED, bool FUSED = false>
 __global__ __launch_bounds__(kBlockSize) void bn_apply_kernel(
     const T* __restrict__ x, const T* __restrict__ mean, const T* __restrict__ var,
     const T* __restrict__ scale, const T* __restrict__ bias, T* __restrict__ y, T epsilon,
     int num_channels, size_t spatial, const TensorMap mx, const TensorMap my, size_t chunk,
-    int chunks_per_seg)
+    int chunks_per_seg, const FusedStats<T> fused = FusedStats<T>())
 {
     const size_t seg = blockIdx.x / chunks_per_seg;
     const int k = blockIdx.x - seg * chunks_per_seg;
     const int c = seg % num_channels;
-    const T m = mean[c];
-    const T inv_stdev = inv_sqrt_t(var[c] + epsilon);
+    T m, variance;
+    if constexpr (FUSED)
+    {
+        __shared__ double lds[2 * kWavesPerBlock];
+        double t[2];
+        channel_totals<2>(fused.partials, fused.groups, fused.groups_per_channel_max, c, t, lds);
+        sums_to_mean_var(static_cast<T>(t[0]), static_cast<T>(t[1]),
+                         static_cast<T>(fused.num_per_sum), &m, &variance);
+        if (seg < static_cast<size_t>(num_channels) && k == 0 && threadIdx.x == 0) // sample 0, chunk 0
+        {
+            fused.out[0][c] = m;
+            fused.out[1][c] = variance;
+            fused.out[2][c] = fma_t(fused.decay, fused.out[2][c], (T(1) - fused.decay) * m);
+            fused.out[3][c] = fma_t(fused.decay, fused.out[3][c], (T(1) - fused.decay) * variance);
+        }
+    }
+    else
+    {
+        m = mean[c];
+        variance = var[c];
+    }
+    const T inv_stdev = inv_sqrt_t(variance + epsilon);
     const T sc = scale[c];
     const T bi = bias[c];
     const size_t begin = static_cast<size_t>(k) * chunk;
@@ -416,7 +486,7 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop1_kernel(
     const T* __restrict__ var, const T* __restrict__ scale, T* __restrict__ dscale,
     T* __restrict__ dbias, T* __restrict__ dmean, T* __restrict__ dvar, T epsilon,
     double* partials, size_t spatial, const TensorMap mx, const TensorMap md, size_t chunk,
-    int chunks_per_seg, unsigned int num_units, int groups_per_channel_max)
+    int chunks_per_seg, unsigned int num_units, int groups_per_channel_max, bool always_partials)
 {
     const int c = blockIdx.y;
     const T m = mean[c];
@@ -478,7 +548,8 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop1_kernel(
                 accumulate(xv[j], dv[j]);
         }
     }
-    if (finish_workgroup<4>(acc, partials, c, groups_per_channel_max) && threadIdx.x == 0)
+    if (finish_workgroup<4>(acc, partials, c, groups_per_channel_max, always_partials)
+        && threadIdx.x == 0)
     {
         dscale[c] = static_cast<T>(acc[0]);
         dbias[c] = static_cast<T>(acc[1]);
@@ -491,13 +562,13 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop1_kernel(
 // Replaces backprop2_opt_kernel, batchnorm.cu:1371-1418.  x and dx may alias:
 // each thread reads its elements before it writes them, so neither is
 // restrict-qualified.
-template <typename T, int VEC, bool STRIDED>
+template <typename T, int VEC, bool STRIDED, bool FUSED = false>
 __global__ __launch_bounds__(kBlockSize) void bn_backprop2_kernel(
     const T* x, const T* __restrict__ dy, const T* __restrict__ mean,
     const T* __restrict__ var, const T* __restrict__ scale, const T* __restrict__ dmean,
     const T* __restrict__ dvar, T* dx, T epsilon, size_t num_per_sum, int num_channels,
     size_t spatial, const TensorMap mx, const TensorMap md, const TensorMap mo, size_t chunk,
-    int chunks_per_seg)
+    int chunks_per_seg, const FusedStats<T> fused = FusedStats<T>())
 {
     const size_t seg = blockIdx.x / chunks_per_seg;
     const int k = blockIdx.x - seg * chunks_per_seg;
@@ -505,8 +576,30 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop2_kernel(
     const T m = mean[c];
     const T sc = scale[c];
     const T inv_stdev = inv_sqrt_t(var[c] + epsilon);
-    const T dmean_term = dmean[c] / static_cast<T>(num_per_sum);
-    const T dvar_term = dvar[c] * T(2) / static_cast<T>(num_per_sum - 1);
+    T dmean_c, dvar_c;
+    if constexpr (FUSED)
+    {
+        // the four sums of bn_backprop1_kernel, finished here (bn_finish_kernel folded in)
+        __shared__ double lds[4 * kWavesPerBlock];
+        double t[4];
+        channel_totals<4>(fused.partials, fused.groups, fused.groups_per_channel_max, c, t, lds);
+        dmean_c = static_cast<T>(t[2]);
+        dvar_c = static_cast<T>(t[3]);
+        if (seg < static_cast<size_t>(num_channels) && k == 0 && threadIdx.x == 0)
+        {
+            fused.out[0][c] = static_cast<T>(t[0]);
+            fused.out[1][c] = static_cast<T>(t[1]);
+            fused.out[2][c] = dmean_c;
+            fused.out[3][c] = dvar_c;
+        }
+    }
+    else
+    {
+        dmean_c = dmean[c];
+        dvar_c = dvar[c];
+    }
+    const T dmean_term = dmean_c / static_cast<T>(num_per_sum);
+    const T dvar_term = dvar_c * T(2) / static_cast<T>(num_per_sum - 1);
     const size_t begin = static_cast<size_t>(k) * chunk;
     const size_t end = begin + chunk < spatial ? begin + chunk : spatial;
     const size_t n = seg / num_channels;
@@ -732,6 +825,26 @@ bool fold_samples(int* num_samples, size_t* spatial, std::initializer_list<HostT
         }                                                                                          \
     } while (0)
 
+// The same for the variants that finish the preceding reduction themselves.
+#define H2X_DISPATCH_FUSED(KERNEL, GRID, ...)                                                      \
+    do                                                                                             \
+    {                                                                                              \
+        if (strided)                                                                               \
+        {                                                                                          \
+            if (vw > 1)                                                                            \
+                KERNEL<T, full_vec<T>(), true, true><<<GRID, kBlockSize, 0, stream>>>(__VA_ARGS__); \
+            else                                                                                   \
+                KERNEL<T, 1, true, true><<<GRID, kBlockSize, 0, stream>>>(__VA_ARGS__);            \
+        }                                                                                          \
+        else                                                                                       \
+        {                                                                                          \
+            if (vw > 1)                                                                            \
+                KERNEL<T, full_vec<T>(), false, true><<<GRID, kBlockSize, 0, stream>>>(__VA_ARGS__); \
+            else                                                                                   \
+                KERNEL<T, 1, false, true><<<GRID, kBlockSize, 0, stream>>>(__VA_ARGS__);           \
+        }                                                                                          \
+    } while (0)
+
 template <typename T>
 int zero_outputs(std::initializer_list<void*> outs, int num_channels, hipStream_t stream)
 {
@@ -741,9 +854,12 @@ int zero_outputs(std::initializer_list<void*> outs, int num_channels, hipStream_
     return launch_status();
 }
 
+// `groups_out` non-null: the caller finishes the reduction itself (a fused
+// consumer kernel): every workgroup stores partials, no finishing launch.
 template <typename T>
 int sums_impl(int num_samples, int num_channels, size_t spatial, const HostTensor& tx_in,
-              const void* x, void* sums, void* sqsums, void* workspace, hipStream_t stream)
+              const void* x, void* sums, void* sqsums, void* workspace, hipStream_t stream,
+              int* groups_out = nullptr)
 {
     if (num_channels == 0)
         return H2X_SUCCESS;
@@ -766,7 +882,12 @@ int sums_impl(int num_samples, int num_channels, size_t spatial, const HostTenso
     const dim3 grid(static_cast<unsigned int>(groups), num_channels);
     H2X_DISPATCH(bn_sums_kernel, grid, static_cast<const T*>(x), static_cast<T*>(sums),
                  static_cast<T*>(sqsums), partials, tx.map, spatial, ch.chunk, ch.chunks_per_seg,
-                 static_cast<unsigned int>(units), gmax);
+                 static_cast<unsigned int>(units), gmax, groups_out != nullptr);
+    if (groups_out != nullptr)
+    {
+        *groups_out = static_cast<int>(groups);
+        return launch_status();
+    }
     if (groups > 1)
         bn_finish_kernel<T, 2><<<num_channels, kBlockSize, 0, stream>>>(
             partials, static_cast<int>(groups), gmax, static_cast<T*>(sums),
@@ -800,7 +921,8 @@ Chunking elementwise_chunking(size_t spatial, size_t segments, int vw, int unrol
 template <typename T>
 int apply_impl(int num_samples, int num_channels, size_t spatial, const HostTensor& tx_in,
                const HostTensor& ty_in, const void* x, const void* mean, const void* var,
-               const void* scale, const void* bias, void* y, double epsilon, hipStream_t stream)
+               const void* scale, const void* bias, void* y, double epsilon, hipStream_t stream,
+               const FusedStats<T>* fused = nullptr)
 {
     if (static_cast<size_t>(num_samples) * num_channels == 0 || spatial == 0)
         return H2X_SUCCESS;
@@ -816,10 +938,16 @@ int apply_impl(int num_samples, int num_channels, size_t spatial, const HostTens
     if (!grid_ok(blocks))
         return H2X_ERR_TOO_LARGE;
     const unsigned int grid = static_cast<unsigned int>(blocks);
-    H2X_DISPATCH(bn_apply_kernel, grid, static_cast<const T*>(x), static_cast<const T*>(mean),
-                 static_cast<const T*>(var), static_cast<const T*>(scale),
-                 static_cast<const T*>(bias), static_cast<T*>(y), static_cast<T>(epsilon),
-                 num_channels, spatial, tx.map, ty.map, ch.chunk, ch.chunks_per_seg);
+    if (fused)
+        H2X_DISPATCH_FUSED(bn_apply_kernel, grid, static_cast<const T*>(x), nullptr, nullptr,
+                           static_cast<const T*>(scale), static_cast<const T*>(bias),
+                           static_cast<T*>(y), static_cast<T>(epsilon), num_channels, spatial,
+                           tx.map, ty.map, ch.chunk, ch.chunks_per_seg, *fused);
+    else
+        H2X_DISPATCH(bn_apply_kernel, grid, static_cast<const T*>(x), static_cast<const T*>(mean),
+                     static_cast<const T*>(var), static_cast<const T*>(scale),
+                     static_cast<const T*>(bias), static_cast<T*>(y), static_cast<T>(epsilon),
+                     num_channels, spatial, tx.map, ty.map, ch.chunk, ch.chunks_per_seg);
     return launch_status();
 }
 
@@ -827,7 +955,8 @@ template <typename T>
 int backprop1_impl(int num_samples, int num_channels, size_t spatial, const HostTensor& tx_in,
                    const HostTensor& td_in, const void* x, const void* dy, const void* mean,
                    const void* var, const void* scale, void* dscale, void* dbias, void* dmean,
-                   void* dvar, double epsilon, void* workspace, hipStream_t stream)
+                   void* dvar, double epsilon, void* workspace, hipStream_t stream,
+                   int* groups_out = nullptr)
 {
     if (num_channels == 0)
         return H2X_SUCCESS;
@@ -853,7 +982,12 @@ int backprop1_impl(int num_samples, int num_channels, size_t spatial, const Host
                  static_cast<const T*>(scale), static_cast<T*>(dscale), static_cast<T*>(dbias),
                  static_cast<T*>(dmean), static_cast<T*>(dvar), static_cast<T>(epsilon), partials,
                  spatial, tx.map, td.map, ch.chunk, ch.chunks_per_seg,
-                 static_cast<unsigned int>(units), gmax);
+                 static_cast<unsigned int>(units), gmax, groups_out != nullptr);
+    if (groups_out != nullptr)
+    {
+        *groups_out = static_cast<int>(groups);
+        return launch_status();
+    }
     if (groups > 1)
         bn_finish_kernel<T, 4><<<num_channels, kBlockSize, 0, stream>>>(
             partials, static_cast<int>(groups), gmax, static_cast<T*>(dscale),
@@ -866,7 +1000,7 @@ int backprop2_impl(int num_samples, int num_channels, size_t spatial, size_t num
                    const HostTensor& tx_in, const HostTensor& td_in, const HostTensor& to_in,
                    const void* x, const void* dy, const void* mean, const void* var,
                    const void* scale, const void* dmean, const void* dvar, void* dx,
-                   double epsilon, hipStream_t stream)
+                   double epsilon, hipStream_t stream, const FusedStats<T>* fused = nullptr)
 {
     if (static_cast<size_t>(num_samples) * num_channels == 0 || spatial == 0)
         return H2X_SUCCESS;
@@ -882,12 +1016,20 @@ int backprop2_impl(int num_samples, int num_channels, size_t spatial, size_t num
     if (!grid_ok(blocks))
         return H2X_ERR_TOO_LARGE;
     const unsigned int grid = static_cast<unsigned int>(blocks);
-    H2X_DISPATCH(bn_backprop2_kernel, grid, static_cast<const T*>(x), static_cast<const T*>(dy),
-                 static_cast<const T*>(mean), static_cast<const T*>(var),
-                 static_cast<const T*>(scale), static_cast<const T*>(dmean),
-                 static_cast<const T*>(dvar), static_cast<T*>(dx), static_cast<T>(epsilon),
-                 num_per_sum, num_channels, spatial, tx.map, td.map, to.map, ch.chunk,
-                 ch.chunks_per_seg);
+    if (fused)
+        H2X_DISPATCH_FUSED(bn_backprop2_kernel, grid, static_cast<const T*>(x),
+                           static_cast<const T*>(dy), static_cast<const T*>(mean),
+                           static_cast<const T*>(var), static_cast<const T*>(scale), nullptr,
+                           nullptr, static_cast<T*>(dx), static_cast<T>(epsilon), num_per_sum,
+                           num_channels, spatial, tx.map, td.map, to.map, ch.chunk,
+                           ch.chunks_per_seg, *fused);
+    else
+        H2X_DISPATCH(bn_backprop2_kernel, grid, static_cast<const T*>(x), static_cast<const T*>(dy),
+                     static_cast<const T*>(mean), static_cast<const T*>(var),
+                     static_cast<const T*>(scale), static_cast<const T*>(dmean),
+                     static_cast<const T*>(dvar), static_cast<T*>(dx), static_cast<T>(epsilon),
+                     num_per_sum, num_channels, spatial, tx.map, td.map, to.map, ch.chunk,
+                     ch.chunks_per_seg);
     return launch_status();
 }
 
@@ -984,6 +1126,69 @@ int backprop2_strided(int n, size_t num_per_sum, const h2x_tensor_geometry* gx,
     return err ? err
                : backprop2_impl<T>(n, c, s, num_per_sum, tx, td, to, x, dy, mean, var, scale, dmean,
                                    dvar, dx, eps, st);
+}
+
+// Forward pass of a rank that shares its statistics with no one: sums, then a
+// normalising kernel that finishes them itself (2 launches instead of 4).
+template <typename T>
+int forward_local(int n, int c, size_t s, size_t x_real, size_t y_real, const void* x,
+                  const void* scale, const void* bias, size_t num_per_sum, double decay, double eps,
+                  void* mean, void* var, void* running_mean, void* running_var, void* y, void* ws,
+                  hipStream_t st)
+{
+    if (c == 0)
+        return H2X_SUCCESS;
+    const HostTensor tx = dense_tensor<T>(x, c, s, x_real), ty = dense_tensor<T>(y, c, s, y_real);
+    if (n == 0 || s == 0 || num_per_sum == 0)
+    {
+        // nothing to normalise or nothing counted: the staged calls define the result
+        int err = sums_impl<T>(n, c, s, tx, x, mean, var, ws, st);
+        if (!err)
+            err = statistics_impl<T>(c, num_per_sum, decay, mean, var, running_mean, running_var, st);
+        return err ? err : apply_impl<T>(n, c, s, tx, ty, x, mean, var, scale, bias, y, eps, st);
+    }
+    FusedStats<T> f;
+    f.partials = static_cast<const double*>(ws);
+    f.groups_per_channel_max = max_groups_per_channel(c);
+    f.num_per_sum = num_per_sum;
+    f.decay = static_cast<T>(decay);
+    f.out[0] = static_cast<T*>(mean);
+    f.out[1] = static_cast<T*>(var);
+    f.out[2] = static_cast<T*>(running_mean);
+    f.out[3] = static_cast<T*>(running_var);
+    const int err = sums_impl<T>(n, c, s, tx, x, nullptr, nullptr, ws, st, &f.groups);
+    return err ? err : apply_impl<T>(n, c, s, tx, ty, x, nullptr, nullptr, scale, bias, y, eps, st, &f);
+}
+
+// Backward pass likewise: the four sums, then an input-gradient kernel that
+// finishes them itself (2 launches instead of 3).
+template <typename T>
+int backward_local(int n, int c, size_t s, size_t x_real, size_t dy_real, size_t dx_real,
+                   size_t num_per_sum, const void* x, const void* dy, const void* mean,
+                   const void* var, const void* scale, void* dscale, void* dbias, void* dmean,
+                   void* dvar, void* dx, double eps, void* ws, hipStream_t st)
+{
+    if (c == 0)
+        return H2X_SUCCESS;
+    const HostTensor tx = dense_tensor<T>(x, c, s, x_real), td = dense_tensor<T>(dy, c, s, dy_real),
+                     to = dense_tensor<T>(dx, c, s, dx_real);
+    if (n == 0 || s == 0)
+        return backprop1_impl<T>(n, c, s, tx, td, x, dy, mean, var, scale, dscale, dbias, dmean,
+                                 dvar, eps, ws, st); // zeroes the four outputs; no dx to write
+    FusedStats<T> f;
+    f.partials = static_cast<const double*>(ws);
+    f.groups_per_channel_max = max_groups_per_channel(c);
+    f.num_per_sum = num_per_sum;
+    f.decay = T(0);
+    f.out[0] = static_cast<T*>(dscale);
+    f.out[1] = static_cast<T*>(dbias);
+    f.out[2] = static_cast<T*>(dmean);
+    f.out[3] = static_cast<T*>(dvar);
+    const int err = backprop1_impl<T>(n, c, s, tx, td, x, dy, mean, var, scale, nullptr, nullptr,
+                                      nullptr, nullptr, eps, ws, st, &f.groups);
+    return err ? err
+               : backprop2_impl<T>(n, c, s, num_per_sum, tx, td, to, x, dy, mean, var, scale,
+                                   nullptr, nullptr, dx, eps, st, &f);
 }
 
 } // namespace
@@ -1214,4 +1419,55 @@ extern "C" int h2x_bn_backprop2_strided(h2x_dtype dtype, int num_samples, size_t
                  backprop2_strided<double>(num_samples, num_per_sum, x_geometry, dy_geometry,
                                            dx_geometry, x, dy, mean, var, scale, dmean, dvar, dx,
                                            epsilon, as_stream(stream)));
+}
+
+extern "C" int h2x_bn_forward_local(h2x_dtype dtype, int num_samples, int num_channels,
+                                    size_t spatial_size, size_t x_spatial_real_size,
+                                    size_t y_spatial_real_size, const void* x, const void* scale,
+                                    const void* bias, size_t num_per_sum, double decay,
+                                    double epsilon, void* mean, void* var, void* running_mean,
+                                    void* running_var, void* y, void* workspace,
+                                    h2x_stream_t stream)
+{
+    if (bad_geometry(num_samples, num_channels, spatial_size, x_spatial_real_size)
+        || y_spatial_real_size < spatial_size || !scale || !bias || !mean || !var || !running_mean
+        || !running_var || !workspace)
+        return H2X_ERR_INVALID_ARGUMENT;
+    if ((!x || !y) && static_cast<size_t>(num_samples) * num_channels * spatial_size > 0)
+        return H2X_ERR_INVALID_ARGUMENT;
+    H2X_BY_DTYPE(dtype,
+                 forward_local<float>(num_samples, num_channels, spatial_size, x_spatial_real_size,
+                                      y_spatial_real_size, x, scale, bias, num_per_sum, decay,
+                                      epsilon, mean, var, running_mean, running_var, y, workspace,
+                                      as_stream(stream)),
+                 forward_local<double>(num_samples, num_channels, spatial_size, x_spatial_real_size,
+                                       y_spatial_real_size, x, scale, bias, num_per_sum, decay,
+                                       epsilon, mean, var, running_mean, running_var, y, workspace,
+                                       as_stream(stream)));
+}
+
+extern "C" int h2x_bn_backward_local(h2x_dtype dtype, int num_samples, int num_channels,
+                                     size_t spatial_size, size_t x_spatial_real_size,
+                                     size_t dy_spatial_real_size, size_t dx_spatial_real_size,
+                                     size_t num_per_sum, const void* x, const void* dy,
+                                     const void* mean, const void* var, const void* scale,
+                                     void* dscale, void* dbias, void* dmean, void* dvar, void* dx,
+                                     double epsilon, void* workspace, h2x_stream_t stream)
+{
+    if (bad_geometry(num_samples, num_channels, spatial_size, x_spatial_real_size)
+        || dy_spatial_real_size < spatial_size || dx_spatial_real_size < spatial_size || !mean
+        || !var || !scale || !dscale || !dbias || !dmean || !dvar || !workspace)
+        return H2X_ERR_INVALID_ARGUMENT;
+    if ((!x || !dy || !dx) && static_cast<size_t>(num_samples) * num_channels * spatial_size > 0)
+        return H2X_ERR_INVALID_ARGUMENT;
+    H2X_BY_DTYPE(dtype,
+                 backward_local<float>(num_samples, num_channels, spatial_size, x_spatial_real_size,
+                                       dy_spatial_real_size, dx_spatial_real_size, num_per_sum, x,
+                                       dy, mean, var, scale, dscale, dbias, dmean, dvar, dx, epsilon,
+                                       workspace, as_stream(stream)),
+                 backward_local<double>(num_samples, num_channels, spatial_size,
+                                        x_spatial_real_size, dy_spatial_real_size,
+                                        dx_spatial_real_size, num_per_sum, x, dy, mean, var, scale,
+                                        dscale, dbias, dmean, dvar, dx, epsilon, workspace,
+                                        as_stream(stream)));
 }

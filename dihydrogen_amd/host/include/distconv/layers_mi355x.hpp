@@ -316,10 +316,30 @@ public:
         return 0;
     }
 
+    // forward() and backward() of a rank that all-reduces nothing between its
+    // stages (one rank, or local statistics) run as two launches each: the
+    // second kernel finishes the first one's sums itself.  Same results as the
+    // staged calls, bit for bit.  set_fuse_local(false) keeps the staged calls.
+    void set_fuse_local(bool on) { m_fuse_local = on; }
+
     template <typename Tensor>
     int forward(const Tensor& input, Tensor& mean, Tensor& var, Tensor& running_mean,
                 Tensor& running_var, Tensor& scale, Tensor& bias, Tensor& output, bool is_training)
     {
+        if (is_training && runs_local(input) && batchnorm::is_dense(input)
+            && batchnorm::is_dense(output))
+        {
+            set_num_samples(static_cast<int>(input.get_local_shape()[-1]));
+            const batchnorm::ChannelGeometry<Tensor> gi(input), go(output);
+            DISTCONV_CHECK_H2X(h2x_bn_forward_local(
+                Tensor::h2x_type(), m_num_current_samples, gi.num_channels, gi.spatial,
+                gi.spatial_real, go.spatial_real, input.get_const_base_ptr(),
+                scale.get_const_base_ptr(), bias.get_const_base_ptr(), num_per_sum(input), m_decay,
+                m_epsilon, mean.get_base_ptr(), var.get_base_ptr(), running_mean.get_base_ptr(),
+                running_var.get_base_ptr(), output.get_base_ptr(), m_ws.get(gi.num_channels),
+                m_stream));
+            return 0;
+        }
         forward_stage1(input, mean, var, is_training);
         forward_allreduce(mean, var, is_training);
         forward_stage2(input, mean, var, running_mean, running_var, scale, bias, output,
@@ -370,6 +390,21 @@ public:
                  const Tensor& scale, Tensor& scale_gradient, Tensor& bias_gradient,
                  Tensor& mean_gradient, Tensor& var_gradient, Tensor& d_input)
     {
+        if (runs_local(input) && batchnorm::is_dense(input) && batchnorm::is_dense(d_output)
+            && batchnorm::is_dense(d_input))
+        {
+            set_num_samples(static_cast<int>(input.get_local_shape()[-1]));
+            const batchnorm::ChannelGeometry<Tensor> gi(input), go(d_output), gd(d_input);
+            DISTCONV_CHECK_H2X(h2x_bn_backward_local(
+                Tensor::h2x_type(), m_num_current_samples, gi.num_channels, gi.spatial,
+                gi.spatial_real, go.spatial_real, gd.spatial_real, num_per_sum(input),
+                input.get_const_base_ptr(), d_output.get_const_base_ptr(),
+                mean.get_const_base_ptr(), var.get_const_base_ptr(), scale.get_const_base_ptr(),
+                scale_gradient.get_base_ptr(), bias_gradient.get_base_ptr(),
+                mean_gradient.get_base_ptr(), var_gradient.get_base_ptr(), d_input.get_base_ptr(),
+                m_epsilon, m_ws.get(gi.num_channels), m_stream));
+            return 0;
+        }
         backward_stage1(input, d_output, mean, var, scale, scale_gradient, bias_gradient,
                         mean_gradient, var_gradient);
         backward_allreduce(scale_gradient, bias_gradient, mean_gradient, var_gradient);
@@ -381,6 +416,14 @@ public:
     void set_num_samples(int n) { m_num_current_samples = n; }
 
 private:
+    // no all-reduce would run between the stages, and the rank owns elements
+    template <typename Tensor>
+    bool runs_local(const Tensor& input) const
+    {
+        return m_fuse_local && !(m_global_stats && m_allreducer) && input.get_local_size() > 0
+               && input.is_split_root();
+    }
+
     // elements per channel of the global (global statistics) or local shape:
     // batchnorm.hpp:232-236,414-418
     template <typename Tensor>
@@ -417,6 +460,7 @@ private:
     DataType m_epsilon;
     BatchnormImpl m_impl;
     bool m_global_stats;
+    bool m_fuse_local = true;
     Allreduce m_allreducer;
     batchnorm::Workspace m_ws;
 };

@@ -71,11 +71,15 @@ class BatchNormalization:
 
     def __init__(self, num_dims: int, decay: float, epsilon: float, global_stats: bool = False,
                  allreduce: Optional[Callable[[List[torch.Tensor]], None]] = None,
-                 stream: Optional[torch.cuda.Stream] = None):
+                 stream: Optional[torch.cuda.Stream] = None, fuse_local: bool = True):
         if num_dims not in (4, 5):
             raise ValueError("4-D (NCHW) or 5-D (NCDHW) tensors only")  # batchnorm.cu:259-270
         self.num_dims, self.decay, self.epsilon = num_dims, float(decay), float(epsilon)
         self.global_stats, self.allreduce, self.stream = global_stats, allreduce, stream
+        # forward()/backward() of a rank that all-reduces nothing between its two
+        # stages run as two launches each (h2x_bn_forward_local / _backward_local);
+        # the staged methods always use the staged entry points
+        self.fuse_local = fuse_local
         self.num_current_samples = 0
         self._lib = capi.load()
         self._workspace: Optional[torch.Tensor] = None
@@ -159,8 +163,24 @@ class BatchNormalization:
             self.batch_normalization(input, running_mean, running_var, scale, bias, output)  # :243-247
         return 0
 
+    def _runs_local(self, *tensors: Tensor) -> bool:
+        """No all-reduce between the stages, dense tensors, a rank that owns elements."""
+        t0 = tensors[0]
+        return (self.fuse_local and not (self.global_stats and self.allreduce is not None)
+                and all(_is_dense(t) for t in tensors) and t0.is_split_root() and t0.get_local_size() > 0)
+
     def forward(self, input, mean, var, running_mean, running_var, scale, bias, output,
                 is_training: bool = True) -> int:
+        if is_training and self._runs_local(input, output):
+            self.set_num_samples(input.local_shape[-1])
+            n, c, s, sr = _channel_geometry(input)
+            _, _, _, sro = _channel_geometry(output)
+            capi.check(self._lib.h2x_bn_forward_local(
+                input.h2x_dtype, self.num_current_samples, c, s, sr, sro, _ptr(input.get_base_ptr()),
+                _ptr(scale), _ptr(bias), self._num_per_sum(input), self.decay, self.epsilon, _ptr(mean),
+                _ptr(var), _ptr(running_mean), _ptr(running_var), _ptr(output.get_base_ptr()),
+                _ptr(self._ws(c)), _stream_handle(self.stream)), "bn forward (local)")
+            return 0
         self.forward_stage1(input, mean, var, is_training)
         self.forward_allreduce(mean, var, is_training)
         return self.forward_stage2(input, mean, var, running_mean, running_var, scale, bias, output,
@@ -220,6 +240,18 @@ class BatchNormalization:
 
     def backward(self, input, d_output, mean, var, scale, scale_gradient, bias_gradient,
                  mean_gradient, var_gradient, d_input) -> int:
+        if self._runs_local(input, d_output, d_input):
+            self.set_num_samples(input.local_shape[-1])
+            n, c, s, sr = _channel_geometry(input)
+            _, _, _, sro = _channel_geometry(d_output)
+            _, _, _, sri = _channel_geometry(d_input)
+            capi.check(self._lib.h2x_bn_backward_local(
+                input.h2x_dtype, self.num_current_samples, c, s, sr, sro, sri, self._num_per_sum(input),
+                _ptr(input.get_base_ptr()), _ptr(d_output.get_base_ptr()), _ptr(mean), _ptr(var),
+                _ptr(scale), _ptr(scale_gradient), _ptr(bias_gradient), _ptr(mean_gradient),
+                _ptr(var_gradient), _ptr(d_input.get_base_ptr()), self.epsilon, _ptr(self._ws(c)),
+                _stream_handle(self.stream)), "bn backward (local)")
+            return 0
         self.backward_stage1(input, d_output, mean, var, scale, scale_gradient, bias_gradient,
                              mean_gradient, var_gradient)
         self.backward_allreduce(scale_gradient, bias_gradient, mean_gradient, var_gradient)

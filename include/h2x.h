@@ -234,6 +234,65 @@ int h2x_bn_backprop2(h2x_dtype dtype,
                      h2x_stream_t stream);
 
 /**
+ * Forward pass of a rank whose statistics are its own (one rank, or
+ * global_stats == false: no all-reduce between the stages): what
+ *   h2x_bn_channel_sums_and_sqsums, h2x_bn_sums_to_statistics(num_per_sum, decay)
+ *   and h2x_bn_batch_normalization
+ * leave in mean, var, running_mean, running_var and y, bit for bit, in two
+ * launches instead of four: the normalising kernel finishes the sums itself.
+ * This is BatchNormalization::forward without its allreduce stage
+ * (legacy/include/distconv/dnn_backend/batchnorm.hpp:171-250); the staged entry
+ * points remain for ranks that all-reduce between stage 1 and stage 2.
+ */
+int h2x_bn_forward_local(h2x_dtype dtype,
+                         int num_samples,
+                         int num_channels,
+                         size_t spatial_size,
+                         size_t x_spatial_real_size,
+                         size_t y_spatial_real_size,
+                         const void* x,
+                         const void* scale,
+                         const void* bias,
+                         size_t num_per_sum,
+                         double decay,
+                         double epsilon,
+                         void* mean,
+                         void* var,
+                         void* running_mean,
+                         void* running_var,
+                         void* y,
+                         void* workspace,
+                         h2x_stream_t stream);
+
+/**
+ * Backward pass likewise: h2x_bn_backprop1 followed by h2x_bn_backprop2 with
+ * the sums it produced, bit for bit, in two launches instead of three
+ * (BatchNormalization::backward without its allreduce stage,
+ * batchnorm.hpp:360-475).  dx may alias x.
+ */
+int h2x_bn_backward_local(h2x_dtype dtype,
+                          int num_samples,
+                          int num_channels,
+                          size_t spatial_size,
+                          size_t x_spatial_real_size,
+                          size_t dy_spatial_real_size,
+                          size_t dx_spatial_real_size,
+                          size_t num_per_sum,
+                          const void* x,
+                          const void* dy,
+                          const void* mean,
+                          const void* var,
+                          const void* scale,
+                          void* dscale,
+                          void* dbias,
+                          void* dmean,
+                          void* dvar,
+                          void* dx,
+                          double epsilon,
+                          void* workspace,
+                          h2x_stream_t stream);
+
+/**
  * Local part of a tensor given by shape and strides, for tensors that carry a
  * halo on an inner spatial dimension.  Innermost first; the last two
  * dimensions are channel and sample; num_dims is 3, 4 or 5.  strides are in

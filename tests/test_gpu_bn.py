@@ -122,6 +122,49 @@ def test_backward_matches_oracle(shape, oracle_mod):
     assert max_rel(dxt.real_view().cpu().numpy(), dx_o) <= TOL
 
 
+@pytest.mark.parametrize("dtype", ["float32", "float64"])
+@pytest.mark.parametrize("shape", [(8, 64, 56, 56), (2, 3, 4, 5), (3, 5, 7, 9, 11), (64, 32, 7, 7), (1, 1, 1, 1),
+                                   (2, 4, 40, 40, 40), (1, 300, 3, 3)])
+def test_two_launch_forward_and_backward_equal_the_staged_calls(shape, dtype):
+    """forward()/backward() of a single rank finish the channel sums inside the
+    normalising / input-gradient kernel (h2x_bn_forward_local, _backward_local);
+    the staged methods launch the finishing kernels.  Same additions in the same
+    order: every output must agree bit for bit (NaNs included)."""
+    import torch
+    from dihydrogen_amd.layers import BatchNormalization
+    from dihydrogen_amd.tensor import Distribution, LocaleVirtual, Tensor
+    np_dt = np.float32 if dtype == "float32" else np.float64
+    tdt = getattr(torch, dtype)
+    x, dy, scale, bias = bn_inputs(shape, seed=99, dtype=np_dt)
+    nd, c = x.ndim, shape[1]
+    dist = Distribution.make_localized_distribution(nd)
+    loc = LocaleVirtual(0, 1)
+    results = []
+    for fuse in (True, False):
+        mk = lambda: Tensor(list(x.shape[::-1]), loc, dist, tdt).allocate()
+        xt, yt, dyt, dxt = mk(), mk(), mk(), mk()
+        xt.real_view().copy_(torch.from_numpy(x))
+        dyt.real_view().copy_(torch.from_numpy(dy))
+        vec = lambda v: torch.full((c,), v, dtype=tdt, device="cuda")
+        mean, var, rm, rv = vec(float("nan")), vec(float("nan")), vec(0.25), vec(0.75)
+        grads = [vec(float("nan")) for _ in range(4)]
+        sc, bi = torch.from_numpy(scale).cuda(), torch.from_numpy(bias).cuda()
+        bn = BatchNormalization(nd, 0.9, 1e-5, fuse_local=fuse)
+        if fuse:
+            assert bn.forward(xt, mean, var, rm, rv, sc, bi, yt, True) == 0
+            assert bn.backward(xt, dyt, mean, var, sc, *grads, dxt) == 0
+        else:
+            bn.forward_stage1(xt, mean, var, True)
+            bn.forward_stage2(xt, mean, var, rm, rv, sc, bi, yt, True)
+            bn.backward_stage1(xt, dyt, mean, var, sc, *grads)
+            bn.backward_stage2(xt, dyt, mean, var, sc, grads[2], grads[3], dxt)
+        torch.cuda.synchronize()
+        results.append([t.cpu().numpy() for t in (mean, var, rm, rv, yt.real_view(), *grads, dxt.real_view())])
+    names = ("mean", "var", "running_mean", "running_var", "y", "dscale", "dbias", "dmean", "dvar", "dx")
+    for name, a, b in zip(names, *results):
+        assert np.array_equal(a, b, equal_nan=True), name
+
+
 def test_backprop2_in_place(oracle_mod):
     """dx may alias x (legacy/src/dnn_backend/batchnorm.cu:1303-1314)."""
     import torch
