@@ -16,6 +16,7 @@ H2X_MAX_DIMS = 6
 F32, F64 = 0, 1
 LHS, RHS = 0, 1
 HALO_ID, HALO_SUM, HALO_MAX, HALO_MIN = 0, 1, 2, 3
+TRANSFORM_SCALE, TRANSFORM_COPY, TRANSFORM_SCALE_BIAS, TRANSFORM_SUMS_TO_STATISTICS = 0, 1, 2, 3
 
 ABI_VERSION = 1
 
@@ -120,6 +121,11 @@ SIGNATURES = {
                                          POINTER(TensorGeometry), POINTER(TensorGeometry), c_void_p,
                                          c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                          c_void_p, c_double, c_void_p]),
+    "h2x_tensor_transform": (c_int, [c_int, c_int, c_int, POINTER(POINTER(TensorGeometry)), POINTER(c_void_p),
+                                     POINTER(c_double), c_void_p]),
+    "h2x_tensor_reduce_sum_workspace_bytes": (c_size_t, [POINTER(TensorGeometry), POINTER(TensorGeometry)]),
+    "h2x_tensor_reduce_sum": (c_int, [c_int, POINTER(TensorGeometry), c_void_p, POINTER(TensorGeometry), c_void_p,
+                                      c_int, c_void_p, c_void_p]),
     "h2x_softmax_channel_forward": (c_int, [c_int, c_int, c_int, c_size_t, c_void_p, c_void_p,
                                             c_void_p]),
     "h2x_softmax_channel_backward": (c_int, [c_int, c_int, c_int, c_size_t, c_void_p, c_void_p,

@@ -1,0 +1,505 @@
+// Elementwise transforms over the interiors of up to four tensors and sums over
+// chosen dimensions, for gfx950: what the reference builds its per-channel
+// statistics, scaling and copies from
+// (legacy/include/distconv/tensor/algorithms/transform_cuda.hpp:359-693,
+//  reduce_sum_cuda.hpp:56-113,388-439).
+//
+// The reference instantiates a kernel per functor; a C interface cannot take a
+// functor, so the operations this path uses are named (h2x_transform_op).  All
+// tensors of a call share one local shape and bring their own strides (halos);
+// the host merges dimensions that are contiguous in every tensor, and a thread
+// finds its element with one multiply-high division per remaining dimension.
+//
+// Sums are deterministic: every output element's addends are cut into groups,
+// a group is added up in fp64 by one workgroup (reduced dimension innermost) or
+// one thread (kept dimension innermost), in index order, and a second kernel
+// adds the groups in order and accumulates into the destination -- where the
+// reference adds floats with atomics in whatever order they arrive
+// (reduce_sum_cuda.hpp:108).
+#include "h2x_device.hpp"
+
+#include <algorithm>
+
+namespace h2x
+{
+namespace
+{
+
+constexpr int kMaxDims = H2X_MAX_DIMS;
+constexpr int kMaxTensors = 4;
+
+struct TransformArgs
+{
+    char* base[kMaxTensors];
+    int64_t stride[kMaxTensors][kMaxDims]; // elements; merged dimensions
+    FastDiv div[kMaxDims];
+    uint32_t count;
+    int32_t num_dims;
+    double p[4];
+};
+
+__device__ __forceinline__ float fma_t(float a, float b, float c)
+{
+    return __builtin_fmaf(a, b, c);
+}
+__device__ __forceinline__ double fma_t(double a, double b, double c)
+{
+    return __builtin_fma(a, b, c);
+}
+
+// legacy/src/dnn_backend/batchnorm.cu:297-312: the same operations, in the same
+// order, as the dedicated statistics kernel of the batch-norm entry points
+template <typename T>
+__device__ __forceinline__ void sums_to_statistics(T& mean, T& var, T& rmean, T& rvar, T n, T decay)
+{
+    const T m = mean / n;
+    const T sqmean = var / n;
+    T v = fma_t(-m, m, sqmean);
+    v = v > T(0) ? v : T(0);
+    v *= n / (n - T(1));
+    mean = m;
+    var = v;
+    rmean = fma_t(decay, rmean, (T(1) - decay) * m);
+    rvar = fma_t(decay, rvar, (T(1) - decay) * v);
+}
+
+template <typename T, int OP>
+__global__ __launch_bounds__(kBlockSize) void transform_kernel(const TransformArgs a)
+{
+    constexpr int N = OP == H2X_TRANSFORM_SCALE ? 1 : OP == H2X_TRANSFORM_SUMS_TO_STATISTICS ? 4 : 2;
+    for (uint64_t i = blockIdx.x * static_cast<uint64_t>(kBlockSize) + threadIdx.x; i < a.count;
+         i += static_cast<uint64_t>(gridDim.x) * kBlockSize)
+    {
+        uint32_t rem = static_cast<uint32_t>(i);
+        int64_t off[N];
+#pragma unroll
+        for (int t = 0; t < N; ++t)
+            off[t] = 0;
+#pragma unroll
+        for (int d = 0; d < kMaxDims; ++d)
+        {
+            if (d < a.num_dims)
+            {
+                uint32_t idx = rem;
+                if (d + 1 < a.num_dims)
+                {
+                    const uint32_t q = fastdiv(rem, a.div[d]);
+                    idx = rem - q * a.div[d].divisor;
+                    rem = q;
+                }
+#pragma unroll
+                for (int t = 0; t < N; ++t)
+                    off[t] += static_cast<int64_t>(idx) * a.stride[t][d];
+            }
+        }
+        T* p[N];
+#pragma unroll
+        for (int t = 0; t < N; ++t)
+            p[t] = reinterpret_cast<T*>(a.base[t]) + off[t];
+        if constexpr (OP == H2X_TRANSFORM_SCALE)
+        {
+            *p[0] = *p[0] * static_cast<T>(a.p[0]); // internal::ScaleFunctor, tensor_mpi_cuda.cu:86-92
+        }
+        else if constexpr (OP == H2X_TRANSFORM_COPY)
+        {
+            *p[1] = *p[0];
+        }
+        else if constexpr (OP == H2X_TRANSFORM_SCALE_BIAS)
+        {
+            // CastScaleBiasFuctor with equal types: dst = alpha * src + beta (tensor_mpi_cuda.cu:113-128)
+            *p[1] = static_cast<T>(a.p[0]) * *p[0] + static_cast<T>(a.p[1]);
+        }
+        else
+        {
+            T m = *p[0], v = *p[1], rm = *p[2], rv = *p[3];
+            if (a.p[0] == 0.0) // nothing was counted: batchnorm.cu:337-345
+            {
+                *p[1] = T(1);
+            }
+            else
+            {
+                sums_to_statistics(m, v, rm, rv, static_cast<T>(a.p[0]), static_cast<T>(a.p[1]));
+                *p[0] = m;
+                *p[1] = v;
+                *p[2] = rm;
+                *p[3] = rv;
+            }
+        }
+    }
+}
+
+// ---- reduce ------------------------------------------------------------------
+
+struct ReduceArgs
+{
+    const char* src;
+    char* dst;
+    double* partials;
+    int32_t num_kept, num_reduced;
+    FastDiv kept_div[kMaxDims];
+    int64_t kept_src[kMaxDims], kept_dst[kMaxDims];
+    FastDiv red_div[kMaxDims];
+    int64_t red_src[kMaxDims];
+    uint32_t kept_count, red_count; // K outputs, R addends each
+    uint32_t groups, chunk;         // addends per group
+    int32_t square;                 // add x * x instead of x
+};
+
+__device__ __forceinline__ int64_t chain(uint32_t i, int nd, const FastDiv* div, const int64_t* stride,
+                                         const int64_t* stride2, int64_t* off2)
+{
+    uint32_t rem = i;
+    int64_t off = 0, o2 = 0;
+#pragma unroll
+    for (int d = 0; d < kMaxDims; ++d)
+    {
+        if (d < nd)
+        {
+            uint32_t idx = rem;
+            if (d + 1 < nd)
+            {
+                const uint32_t q = fastdiv(rem, div[d]);
+                idx = rem - q * div[d].divisor;
+                rem = q;
+            }
+            off += static_cast<int64_t>(idx) * stride[d];
+            if (stride2)
+                o2 += static_cast<int64_t>(idx) * stride2[d];
+        }
+    }
+    if (off2)
+        *off2 = o2;
+    return off;
+}
+
+// The innermost dimension is reduced: a workgroup adds one group of one output
+// element's addends; neighbouring threads read neighbouring addends.
+template <typename T>
+__global__ __launch_bounds__(kBlockSize) void reduce_inner_kernel(const ReduceArgs a)
+{
+    __shared__ double lds[kWavesPerBlock];
+    const uint32_t k = blockIdx.x, g = blockIdx.y;
+    const T* src = reinterpret_cast<const T*>(a.src)
+                   + chain(k, a.num_kept, a.kept_div, a.kept_src, nullptr, nullptr);
+    const uint32_t begin = g * a.chunk;
+    const uint32_t end = begin + a.chunk < a.red_count ? begin + a.chunk : a.red_count;
+    double acc[1] = {0.0};
+    for (uint32_t r = begin + threadIdx.x; r < end; r += kBlockSize)
+    {
+        const double x = static_cast<double>(
+            src[chain(r, a.num_reduced, a.red_div, a.red_src, nullptr, nullptr)]);
+        acc[0] += a.square ? x * x : x;
+    }
+    block_sum<1>(acc, lds);
+    if (threadIdx.x == 0)
+        a.partials[static_cast<size_t>(k) * a.groups + g] = acc[0];
+}
+
+// The innermost dimension is kept: a thread adds one group of its own output
+// element's addends; neighbouring threads own neighbouring outputs.
+template <typename T>
+__global__ __launch_bounds__(kBlockSize) void reduce_outer_kernel(const ReduceArgs a)
+{
+    const uint32_t k = blockIdx.x * kBlockSize + threadIdx.x, g = blockIdx.y;
+    if (k >= a.kept_count)
+        return;
+    const T* src = reinterpret_cast<const T*>(a.src)
+                   + chain(k, a.num_kept, a.kept_div, a.kept_src, nullptr, nullptr);
+    const uint32_t begin = g * a.chunk;
+    const uint32_t end = begin + a.chunk < a.red_count ? begin + a.chunk : a.red_count;
+    double acc = 0.0;
+    for (uint32_t r = begin; r < end; ++r)
+    {
+        const double x = static_cast<double>(
+            src[chain(r, a.num_reduced, a.red_div, a.red_src, nullptr, nullptr)]);
+        acc += a.square ? x * x : x;
+    }
+    a.partials[static_cast<size_t>(g) * a.kept_count + k] = acc;
+}
+
+// dst[k] += sum over the groups, in group order.
+template <typename T>
+__global__ __launch_bounds__(kBlockSize) void reduce_finish_kernel(const ReduceArgs a, int inner)
+{
+    const uint32_t k = blockIdx.x * kBlockSize + threadIdx.x;
+    if (k >= a.kept_count)
+        return;
+    double t = 0.0;
+    for (uint32_t g = 0; g < a.groups; ++g)
+        t += inner ? a.partials[static_cast<size_t>(k) * a.groups + g]
+                   : a.partials[static_cast<size_t>(g) * a.kept_count + k];
+    int64_t dst_off;
+    chain(k, a.num_kept, a.kept_div, a.kept_src, a.kept_dst, &dst_off);
+    T* p = reinterpret_cast<T*>(a.dst) + dst_off;
+    *p = *p + static_cast<T>(t);
+}
+
+// ---- host ---------------------------------------------------------------------
+
+int check_geometry(const h2x_tensor_geometry* g)
+{
+    if (!g || g->num_dims < 1 || g->num_dims > kMaxDims)
+        return H2X_ERR_INVALID_ARGUMENT;
+    for (int i = 0; i < g->num_dims; ++i)
+        if (g->local_shape[i] < 0 || g->strides[i] < 0)
+            return H2X_ERR_INVALID_ARGUMENT;
+    return H2X_SUCCESS;
+}
+
+template <typename T>
+int transform_typed(int op, const TransformArgs& a, hipStream_t stream)
+{
+    const unsigned int blocks =
+        static_cast<unsigned int>(std::min<uint64_t>((a.count + kBlockSize - 1) / kBlockSize, 65536));
+    switch (op)
+    {
+    case H2X_TRANSFORM_SCALE:
+        transform_kernel<T, H2X_TRANSFORM_SCALE><<<blocks, kBlockSize, 0, stream>>>(a);
+        break;
+    case H2X_TRANSFORM_COPY:
+        transform_kernel<T, H2X_TRANSFORM_COPY><<<blocks, kBlockSize, 0, stream>>>(a);
+        break;
+    case H2X_TRANSFORM_SCALE_BIAS:
+        transform_kernel<T, H2X_TRANSFORM_SCALE_BIAS><<<blocks, kBlockSize, 0, stream>>>(a);
+        break;
+    case H2X_TRANSFORM_SUMS_TO_STATISTICS:
+        transform_kernel<T, H2X_TRANSFORM_SUMS_TO_STATISTICS><<<blocks, kBlockSize, 0, stream>>>(a);
+        break;
+    default: return H2X_ERR_UNSUPPORTED;
+    }
+    return launch_status();
+}
+
+// How a sum is cut up.  Shared by the entry point and the workspace query.
+struct ReducePlan
+{
+    ReduceArgs args;
+    bool inner = false; // the innermost dimension with more than one element is reduced
+    bool empty = false; // nothing to add
+};
+
+int plan_reduce(const h2x_tensor_geometry* src, const h2x_tensor_geometry* dst, ReducePlan* plan)
+{
+    int err = check_geometry(src);
+    if (!err)
+        err = check_geometry(dst);
+    if (err)
+        return err;
+    if (src->num_dims != dst->num_dims)
+        return H2X_ERR_INVALID_ARGUMENT;
+    ReduceArgs& a = plan->args;
+    a.num_kept = a.num_reduced = 0;
+    uint64_t kept = 1, red = 1;
+    bool first = true;
+    int64_t kept_extent[kMaxDims], red_extent[kMaxDims];
+    for (int i = 0; i < src->num_dims; ++i)
+    {
+        const int64_t e = src->local_shape[i];
+        // reduce to a single entry or not at all: reduce_sum_cuda.hpp:160-171
+        if (dst->local_shape[i] != 1 && dst->local_shape[i] != e)
+            return H2X_ERR_INVALID_ARGUMENT;
+        if (e == 0)
+            plan->empty = true;
+        if (e == 1)
+            continue;
+        const bool reduced = dst->local_shape[i] == 1;
+        if (first)
+        {
+            plan->inner = reduced;
+            first = false;
+        }
+        if (reduced)
+        {
+            // merge with the previous reduced dimension when contiguous in the source
+            if (a.num_reduced > 0
+                && src->strides[i] == a.red_src[a.num_reduced - 1] * red_extent[a.num_reduced - 1])
+            {
+                red_extent[a.num_reduced - 1] *= e;
+            }
+            else
+            {
+                red_extent[a.num_reduced] = e;
+                a.red_src[a.num_reduced] = src->strides[i];
+                ++a.num_reduced;
+            }
+            red *= static_cast<uint64_t>(e);
+        }
+        else
+        {
+            kept_extent[a.num_kept] = e;
+            a.kept_src[a.num_kept] = src->strides[i];
+            a.kept_dst[a.num_kept] = dst->strides[i];
+            ++a.num_kept;
+            kept *= static_cast<uint64_t>(e);
+        }
+    }
+    if (kept >= (1ull << 31) || red >= (1ull << 31))
+        return H2X_ERR_TOO_LARGE;
+    for (int i = 0; i < kMaxDims; ++i)
+    {
+        a.kept_div[i] = make_fastdiv(i < a.num_kept ? static_cast<uint32_t>(kept_extent[i]) : 1u);
+        a.red_div[i] = make_fastdiv(i < a.num_reduced ? static_cast<uint32_t>(red_extent[i]) : 1u);
+        if (i >= a.num_kept)
+            a.kept_src[i] = a.kept_dst[i] = 0;
+        if (i >= a.num_reduced)
+            a.red_src[i] = 0;
+    }
+    a.kept_count = static_cast<uint32_t>(kept);
+    a.red_count = static_cast<uint32_t>(red);
+    // about 2048 workgroups in all, and no group smaller than a pass of its team
+    constexpr uint64_t kTargetBlocks = 2048;
+    uint64_t groups;
+    if (plan->inner)
+        groups = std::min<uint64_t>((red + 4 * kBlockSize - 1) / (4 * kBlockSize),
+                                    std::max<uint64_t>(kTargetBlocks / std::max<uint64_t>(kept, 1), 1));
+    else
+        groups = std::min<uint64_t>(
+            (red + 15) / 16,
+            std::max<uint64_t>(kTargetBlocks / ((kept + kBlockSize - 1) / kBlockSize), 1));
+    groups = std::min<uint64_t>(std::max<uint64_t>(groups, 1), 65535);
+    a.chunk = static_cast<uint32_t>((red + groups - 1) / groups);
+    a.groups = static_cast<uint32_t>((red + a.chunk - 1) / std::max<uint32_t>(a.chunk, 1));
+    if (a.groups == 0)
+        a.groups = 1;
+    return H2X_SUCCESS;
+}
+
+template <typename T>
+int reduce_typed(const ReducePlan& plan, hipStream_t stream)
+{
+    const ReduceArgs& a = plan.args;
+    const unsigned int kept_blocks = (a.kept_count + kBlockSize - 1) / kBlockSize;
+    if (plan.inner)
+    {
+        reduce_inner_kernel<T><<<dim3(a.kept_count, a.groups), kBlockSize, 0, stream>>>(a);
+    }
+    else
+    {
+        reduce_outer_kernel<T><<<dim3(kept_blocks, a.groups), kBlockSize, 0, stream>>>(a);
+    }
+    reduce_finish_kernel<T><<<kept_blocks, kBlockSize, 0, stream>>>(a, plan.inner ? 1 : 0);
+    return launch_status();
+}
+
+} // namespace
+} // namespace h2x
+
+using namespace h2x;
+
+extern "C" int h2x_tensor_transform(h2x_transform_op op, h2x_dtype dtype, int num_tensors,
+                                    const h2x_tensor_geometry* const* geometries,
+                                    void* const* tensors, const double* params,
+                                    h2x_stream_t stream)
+{
+    const int expected = op == H2X_TRANSFORM_SCALE                ? 1
+                         : op == H2X_TRANSFORM_COPY               ? 2
+                         : op == H2X_TRANSFORM_SCALE_BIAS         ? 2
+                         : op == H2X_TRANSFORM_SUMS_TO_STATISTICS ? 4
+                                                                  : 0;
+    if (expected == 0)
+        return H2X_ERR_UNSUPPORTED;
+    if (dtype != H2X_F32 && dtype != H2X_F64)
+        return H2X_ERR_UNSUPPORTED;
+    if (num_tensors != expected || !geometries || !tensors)
+        return H2X_ERR_INVALID_ARGUMENT;
+    if (op != H2X_TRANSFORM_COPY && !params)
+        return H2X_ERR_INVALID_ARGUMENT;
+    for (int t = 0; t < num_tensors; ++t)
+    {
+        const int err = check_geometry(geometries[t]);
+        if (err)
+            return err;
+        if (geometries[t]->num_dims != geometries[0]->num_dims)
+            return H2X_ERR_INVALID_ARGUMENT;
+        for (int i = 0; i < geometries[0]->num_dims; ++i)
+            if (geometries[t]->local_shape[i] != geometries[0]->local_shape[i])
+                return H2X_ERR_INVALID_ARGUMENT;
+    }
+    // merge what is contiguous in every tensor; extent-1 dimensions vanish
+    TransformArgs a;
+    int nd = 0;
+    int64_t extent[kMaxDims];
+    uint64_t count = 1;
+    for (int i = 0; i < geometries[0]->num_dims; ++i)
+    {
+        const int64_t e = geometries[0]->local_shape[i];
+        count *= static_cast<uint64_t>(e);
+        if (e == 1)
+            continue;
+        bool merge = nd > 0;
+        for (int t = 0; merge && t < num_tensors; ++t)
+            merge = geometries[t]->strides[i] == a.stride[t][nd - 1] * extent[nd - 1];
+        if (merge)
+        {
+            extent[nd - 1] *= e;
+        }
+        else
+        {
+            extent[nd] = e;
+            for (int t = 0; t < num_tensors; ++t)
+                a.stride[t][nd] = geometries[t]->strides[i];
+            ++nd;
+        }
+    }
+    if (count == 0)
+        return H2X_SUCCESS;
+    if (count >= (1ull << 31))
+        return H2X_ERR_TOO_LARGE;
+    for (int t = 0; t < num_tensors; ++t)
+        if (!tensors[t])
+            return H2X_ERR_INVALID_ARGUMENT;
+    if (nd == 0)
+    {
+        nd = 1;
+        extent[0] = 1;
+        for (int t = 0; t < num_tensors; ++t)
+            a.stride[t][0] = 1;
+    }
+    for (int t = 0; t < kMaxTensors; ++t)
+    {
+        a.base[t] = t < num_tensors ? static_cast<char*>(tensors[t]) : nullptr;
+        for (int i = 0; i < kMaxDims; ++i)
+            if (t >= num_tensors || i >= nd)
+                a.stride[t][i] = 0;
+    }
+    for (int i = 0; i < kMaxDims; ++i)
+        a.div[i] = make_fastdiv(i < nd ? static_cast<uint32_t>(extent[i]) : 1u);
+    a.count = static_cast<uint32_t>(count);
+    a.num_dims = nd;
+    for (int i = 0; i < 4; ++i)
+        a.p[i] = params ? params[i] : 0.0;
+    return dtype == H2X_F32 ? transform_typed<float>(op, a, as_stream(stream))
+                            : transform_typed<double>(op, a, as_stream(stream));
+}
+
+extern "C" size_t h2x_tensor_reduce_sum_workspace_bytes(const h2x_tensor_geometry* src_geometry,
+                                                        const h2x_tensor_geometry* dst_geometry)
+{
+    ReducePlan plan;
+    if (plan_reduce(src_geometry, dst_geometry, &plan) != 0)
+        return 0;
+    const size_t n = static_cast<size_t>(plan.args.kept_count) * plan.args.groups * sizeof(double);
+    return (std::max<size_t>(n, 1) + 255) / 256 * 256;
+}
+
+extern "C" int h2x_tensor_reduce_sum(h2x_dtype dtype, const h2x_tensor_geometry* src_geometry,
+                                     const void* src, const h2x_tensor_geometry* dst_geometry,
+                                     void* dst, int square, void* workspace, h2x_stream_t stream)
+{
+    if (dtype != H2X_F32 && dtype != H2X_F64)
+        return H2X_ERR_UNSUPPORTED;
+    ReducePlan plan;
+    const int err = plan_reduce(src_geometry, dst_geometry, &plan);
+    if (err)
+        return err;
+    if (plan.empty || plan.args.kept_count == 0 || plan.args.red_count == 0)
+        return H2X_SUCCESS; // nothing to add: the destination keeps its values
+    if (!src || !dst || !workspace)
+        return H2X_ERR_INVALID_ARGUMENT;
+    plan.args.src = static_cast<const char*>(src);
+    plan.args.dst = static_cast<char*>(dst);
+    plan.args.partials = static_cast<double*>(workspace);
+    plan.args.square = square ? 1 : 0;
+    return dtype == H2X_F32 ? reduce_typed<float>(plan, as_stream(stream))
+                            : reduce_typed<double>(plan, as_stream(stream));
+}

@@ -300,6 +300,8 @@ int h2x_bn_backward_local(h2x_dtype dtype,
  * legacy/include/distconv/tensor/tensor.hpp:291-298) and strides[0] must be 1;
  * the data pointer that goes with it is the tensor's get_base_ptr().
  */
+/* (The transform and sum entry points further down accept any 1 to
+ * H2X_MAX_DIMS dimensions and any strides.) */
 typedef struct h2x_tensor_geometry
 {
     int32_t num_dims;
@@ -371,6 +373,71 @@ int h2x_bn_backprop2_strided(h2x_dtype dtype,
                              void* dx,
                              double epsilon,
                              h2x_stream_t stream);
+
+/* ------------------------------------------------------------------------ */
+/* Elementwise transforms and sums over dimensions                           */
+/* ------------------------------------------------------------------------ */
+
+/**
+ * The operations tensor::Transform is instantiated with on this path
+ * (legacy/include/distconv/tensor/algorithms/transform_cuda.hpp:359-693).  The
+ * reference compiles a kernel per functor; here they are named.
+ */
+typedef enum h2x_transform_op
+{
+    /** 1 tensor: x = x * params[0] (internal::ScaleFunctor, legacy/src/tensor/tensor_mpi_cuda.cu:86-98). */
+    H2X_TRANSFORM_SCALE = 0,
+    /** 2 tensors: t1 = t0. */
+    H2X_TRANSFORM_COPY = 1,
+    /** 2 tensors: t1 = params[0] * t0 + params[1] (CastScaleBias with equal types, tensor_mpi_cuda.cu:113-135). */
+    H2X_TRANSFORM_SCALE_BIAS = 2,
+    /** 4 tensors (sums -> mean, sqsums -> var, running_mean, running_var), in place, with
+     *  params[0] = num_per_sum, params[1] = decay: what h2x_bn_sums_to_statistics computes,
+     *  expressed as the four-tensor transform the reference uses
+     *  (legacy/src/dnn_backend/batchnorm.cu:288-346). */
+    H2X_TRANSFORM_SUMS_TO_STATISTICS = 3
+} h2x_transform_op;
+
+/**
+ * Applies `op` to corresponding elements of the local parts (interiors) of
+ * `num_tensors` tensors.  Each tensor comes with its own geometry: all local
+ * shapes must be equal, strides are each tensor's own (halos), the pointers
+ * are the tensors' get_base_ptr().  Here a geometry may have 1 to
+ * H2X_MAX_DIMS dimensions of any meaning and any strides.  `params` holds
+ * four doubles (may be NULL for COPY).  Replaces tensor::Transform
+ * (transform_cuda.hpp:359-693) for the named operations.
+ */
+int h2x_tensor_transform(h2x_transform_op op,
+                         h2x_dtype dtype,
+                         int num_tensors,
+                         const h2x_tensor_geometry* const* geometries,
+                         void* const* tensors,
+                         const double* params,
+                         h2x_stream_t stream);
+
+/** Bytes of device workspace h2x_tensor_reduce_sum needs for this pair of geometries (fp64 partial sums, no initialisation). */
+size_t h2x_tensor_reduce_sum_workspace_bytes(const h2x_tensor_geometry* src_geometry,
+                                             const h2x_tensor_geometry* dst_geometry);
+
+/**
+ * dst += sum of src (or of src * src when `square` is set) over every
+ * dimension in which dst has extent 1 and src has more.  Each local extent of
+ * dst must be 1 or equal to src's; src's local_shape is the region summed
+ * (the reference's local_reduction_shape).  As in the reference the
+ * destination is accumulated into, so it is zeroed by the caller first
+ * (tensor::ReduceSum and TransformReduceSum,
+ * legacy/include/distconv/tensor/algorithms/reduce_sum_cuda.hpp:56-113,388-439;
+ * the all-reduce over ranks that follows there is the caller's).  fp64
+ * accumulation in a fixed order: deterministic.
+ */
+int h2x_tensor_reduce_sum(h2x_dtype dtype,
+                          const h2x_tensor_geometry* src_geometry,
+                          const void* src,
+                          const h2x_tensor_geometry* dst_geometry,
+                          void* dst,
+                          int square,
+                          void* workspace,
+                          h2x_stream_t stream);
 
 /* ------------------------------------------------------------------------ */
 /* Channel softmax: dense [num_samples][num_channels][spatial_size] tensors,  */

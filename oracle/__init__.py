@@ -307,3 +307,56 @@ def shuffle_pack_rows4(tensor: np.ndarray, local_shape, peer_locale_shape, rank_
     lib().orc_shuffle_pack_rows4(
         _ptr(tensor), ctypes.c_int(tensor.dtype.itemsize), _i64(local_shape),
         _i64(peer_locale_shape), rlp, _ptr(buf), dpp)
+
+
+# --------------------------------------------------------------------------
+# Elementwise transforms and sums over dimensions
+# (legacy/include/distconv/tensor/algorithms/transform_cuda.hpp:359-693,
+#  reduce_sum_cuda.hpp:56-113,388-439)
+# --------------------------------------------------------------------------
+
+TRANSFORM_SCALE, TRANSFORM_COPY, TRANSFORM_SCALE_BIAS, TRANSFORM_SUMS_TO_STATISTICS = 0, 1, 2, 3
+
+
+def tensor_transform(op: int, tensors, params=()):
+    """tensor::Transform over the interiors of 1-4 tensors (numpy views of equal
+    shape, e.g. interiors of haloed arrays), in place, for the named functors:
+    ScaleFunctor (legacy/src/tensor/tensor_mpi_cuda.cu:86-98), copy,
+    CastScaleBias with equal types (tensor_mpi_cuda.cu:113-135) and the
+    sums-to-statistics functor (legacy/src/dnn_backend/batchnorm.cu:297-346).
+    Arithmetic is done in the tensors' own type, one rounding per operation."""
+    t = list(tensors)
+    dt = t[0].dtype.type
+    if op == TRANSFORM_SCALE:
+        t[0][...] = t[0] * dt(params[0])
+    elif op == TRANSFORM_COPY:
+        t[1][...] = t[0]
+    elif op == TRANSFORM_SCALE_BIAS:
+        t[1][...] = dt(params[0]) * t[0] + dt(params[1])
+    elif op == TRANSFORM_SUMS_TO_STATISTICS:
+        mean, var, rmean, rvar = t
+        shape = mean.shape
+        m, v = np.ascontiguousarray(mean).ravel(), np.ascontiguousarray(var).ravel()
+        rm, rv = np.ascontiguousarray(rmean).ravel(), np.ascontiguousarray(rvar).ravel()
+        bn_sums_to_statistics(int(params[0]), float(params[1]), m, v, rm, rv)
+        mean[...], var[...] = m.reshape(shape), v.reshape(shape)
+        rmean[...], rvar[...] = rm.reshape(shape), rv.reshape(shape)
+    else:
+        raise ValueError(op)
+
+
+def tensor_reduce_sum(src: np.ndarray, dst: np.ndarray, square: bool = False) -> None:
+    """tensor::ReduceSum / TransformReduceSum: ``dst += sum(src)`` over every
+    axis where dst has extent 1 (reduce_sum_cuda.hpp:69-113: each element is
+    added onto its destination cell; the destination is not cleared).  The sum
+    is taken in float64 and rounded once, the arithmetic the device path
+    uses; the reference accumulates floats with atomics in arrival order."""
+    assert src.ndim == dst.ndim
+    axes = tuple(i for i in range(src.ndim) if dst.shape[i] == 1 and src.shape[i] != 1)
+    for i in range(src.ndim):
+        assert dst.shape[i] in (1, src.shape[i])
+    x = src.astype(np.float64)
+    if square:
+        x = x * x
+    total = x.sum(axis=axes, keepdims=True) if axes else x
+    dst[...] = dst + total.astype(dst.dtype)
