@@ -7,6 +7,7 @@
 #include <functional>
 #include <map>
 
+#include "distconv/algorithms_mi355x.hpp"
 #include "distconv/tensor_mi355x.hpp"
 
 namespace distconv
@@ -143,10 +144,12 @@ void sums_to_statistics(index_t num_per_sum, typename Tensor::data_type decay, T
                         Tensor& global_var, Tensor& running_mean, Tensor& running_var,
                         hipStream_t stream)
 {
-    DISTCONV_CHECK_H2X(h2x_bn_sums_to_statistics(
-        Tensor::h2x_type(), static_cast<int>(global_mean.get_local_size()), num_per_sum, decay,
-        global_mean.get_base_ptr(), global_var.get_base_ptr(), running_mean.get_base_ptr(),
-        running_var.get_base_ptr(), stream));
+    // As in the reference (batchnorm.cu:317-346) this is a transform over the four
+    // per-channel tensors; the functor lives in the library.
+    tensor::Transform(global_mean, global_var, running_mean, running_var,
+                      tensor::internal::SumsToStatisticsFunctor<typename Tensor::data_type>(
+                          num_per_sum, decay),
+                      stream);
 }
 
 // batchnorm.hpp:39-49

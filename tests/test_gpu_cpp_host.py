@@ -13,7 +13,7 @@ BUILD = os.path.join(HERE, "cpp", "build")
 
 
 @pytest.mark.parametrize("name", ["test_halo_exchange_virtual", "test_shuffle_virtual",
-                                  "test_batchnorm_softmax", "test_h2_frontend"])
+                                  "test_batchnorm_softmax", "test_h2_frontend", "test_algorithms"])
 def test_cpp(name):
     exe = os.path.join(BUILD, name)
     assert os.path.exists(exe), f"{exe} is missing: run `make -C tests/cpp`"
