@@ -13,7 +13,9 @@
 // position: {Spatial..., Channel, Sample}, innermost first, is what the
 // kernels take; anything else is rejected.  Strided views are accepted where
 // the kernels have strided forms (batch-norm), contiguity is required
-// elsewhere.  There is no CPU implementation: a CPU tensor raises.
+// elsewhere.  Batch-norm and softmax have no CPU implementation: a CPU tensor
+// raises; the halo, transform and sum operators of h2/tensor_ops_mi355x.hpp
+// have both arms.
 #pragma once
 
 #include "h2/h2_mi355x.hpp"
@@ -282,6 +284,14 @@ void halo_pack_or_unpack_impl(GPUDev_t, Tensor<T>& tensor, int dim, int side, in
 
 } // namespace impl
 
+} // namespace h2
+
+// scale / copy / sums, clear_halo, halo_transfer, shuffle, instance softmax, and the CPU arms
+#include "h2/tensor_ops_mi355x.hpp"
+
+namespace h2
+{
+
 // ---- typed fronts --------------------------------------------------------------------------
 #define H2X_GPU_ONLY(tensor, call)                                                               \
     do                                                                                            \
@@ -341,15 +351,21 @@ template <typename T>
 void halo_pack(Tensor<T>& tensor, int dim, int side, int width, Tensor<T>& buffer,
                bool is_reverse = false)
 {
-    H2X_GPU_ONLY(tensor, impl::halo_pack_or_unpack_impl(DeviceT_v<Device::GPU>, tensor, dim, side,
-                                                        width, buffer, true, is_reverse, H2X_HALO_ID));
+    H2_DEVICE_DISPATCH(tensor.get_device(),
+                       impl::halo_pack_or_unpack_impl(DeviceT_v<Device::CPU>, tensor, dim, side, width,
+                                                      buffer, true, is_reverse, H2X_HALO_ID),
+                       impl::halo_pack_or_unpack_impl(DeviceT_v<Device::GPU>, tensor, dim, side, width,
+                                                      buffer, true, is_reverse, H2X_HALO_ID));
 }
 template <typename T>
 void halo_unpack(Tensor<T>& tensor, int dim, int side, int width, Tensor<T>& buffer,
                  bool is_reverse = false, int op = H2X_HALO_ID)
 {
-    H2X_GPU_ONLY(tensor, impl::halo_pack_or_unpack_impl(DeviceT_v<Device::GPU>, tensor, dim, side,
-                                                        width, buffer, false, is_reverse, op));
+    H2_DEVICE_DISPATCH(tensor.get_device(),
+                       impl::halo_pack_or_unpack_impl(DeviceT_v<Device::CPU>, tensor, dim, side, width,
+                                                      buffer, false, is_reverse, op),
+                       impl::halo_pack_or_unpack_impl(DeviceT_v<Device::GPU>, tensor, dim, side, width,
+                                                      buffer, false, is_reverse, op));
 }
 
 #undef H2X_GPU_ONLY
@@ -424,6 +440,37 @@ struct Erased
         else
             halo_unpack(as<T>(tensor), dim, side, width, as<T>(buffer), is_reverse, op);
     }
+    static void scale_(BaseTensor& t, double alpha) { scale(as<T>(t), static_cast<T>(alpha)); }
+    static void scale_bias_(const BaseTensor& src, BaseTensor& dst, double alpha, double beta)
+    {
+        scale_bias(as<T>(src), as<T>(dst), static_cast<T>(alpha), static_cast<T>(beta));
+    }
+    static void copy_values_(const BaseTensor& src, BaseTensor& dst) { copy_values(as<T>(src), as<T>(dst)); }
+    static void reduce_sum_(const BaseTensor& src, BaseTensor& dst, bool square)
+    {
+        reduce_sum(as<T>(src), as<T>(dst), square);
+    }
+    static void clear_halo_(BaseTensor& t, int dim, int width) { clear_halo(as<T>(t), dim, width); }
+    static void halo_transfer_(const BaseTensor& src, BaseTensor& dst, int dim, int src_side, int width,
+                               bool is_reverse, int op)
+    {
+        halo_transfer(as<T>(src), as<T>(dst), dim, src_side, width, is_reverse, op);
+    }
+    static void shuffle_(const ShufflePlan& plan, BaseTensor& tensor, BaseTensor& buffer, bool is_pack)
+    {
+        if (is_pack)
+            shuffle_pack(plan, as<T>(static_cast<const BaseTensor&>(tensor)), as<T>(buffer));
+        else
+            shuffle_unpack(plan, as<T>(tensor), as<T>(static_cast<const BaseTensor&>(buffer)));
+    }
+    static void softmax_instance_forward_(const BaseTensor& x, BaseTensor& y)
+    {
+        softmax_instance_forward(as<T>(x), as<T>(y));
+    }
+    static void softmax_instance_backward_(const BaseTensor& y, const BaseTensor& dy, BaseTensor& dx)
+    {
+        softmax_instance_backward(as<T>(y), as<T>(dy), as<T>(dx));
+    }
 };
 
 template <typename T>
@@ -438,6 +485,15 @@ void register_type()
     dispatch_register("softmax_channel_forward_gpu", key, &Erased<T>::softmax_forward);
     dispatch_register("softmax_channel_backward_gpu", key, &Erased<T>::softmax_backward);
     dispatch_register("halo_pack_or_unpack_gpu", key, &Erased<T>::halo);
+    dispatch_register("scale_gpu", key, &Erased<T>::scale_);
+    dispatch_register("scale_bias_gpu", key, &Erased<T>::scale_bias_);
+    dispatch_register("copy_values_gpu", key, &Erased<T>::copy_values_);
+    dispatch_register("reduce_sum_gpu", key, &Erased<T>::reduce_sum_);
+    dispatch_register("clear_halo_gpu", key, &Erased<T>::clear_halo_);
+    dispatch_register("halo_transfer_gpu", key, &Erased<T>::halo_transfer_);
+    dispatch_register("shuffle_gpu", key, &Erased<T>::shuffle_);
+    dispatch_register("softmax_instance_forward_gpu", key, &Erased<T>::softmax_instance_forward_);
+    dispatch_register("softmax_instance_backward_gpu", key, &Erased<T>::softmax_instance_backward_);
 }
 
 // Registers the float and double implementations once per process.
@@ -515,6 +571,49 @@ inline void halo_unpack(BaseTensor& tensor, int dim, int side, int width, BaseTe
     const bool is_pack = false;
     mi355x::dispatch("halo_pack_or_unpack_gpu", tensor, tensor, dim, side, width, buffer, is_pack,
                      is_reverse, op);
+}
+inline void scale(BaseTensor& t, double alpha)
+{
+    mi355x::dispatch("scale_gpu", t, t, alpha);
+}
+inline void scale_bias(const BaseTensor& src, BaseTensor& dst, double alpha, double beta)
+{
+    mi355x::dispatch("scale_bias_gpu", src, src, dst, alpha, beta);
+}
+inline void copy_values(const BaseTensor& src, BaseTensor& dst)
+{
+    mi355x::dispatch("copy_values_gpu", src, src, dst);
+}
+inline void reduce_sum(const BaseTensor& src, BaseTensor& dst, bool square = false)
+{
+    mi355x::dispatch("reduce_sum_gpu", src, src, dst, square);
+}
+inline void clear_halo(BaseTensor& t, int dim, int width)
+{
+    mi355x::dispatch("clear_halo_gpu", t, t, dim, width);
+}
+inline void halo_transfer(const BaseTensor& src, BaseTensor& dst, int dim, int src_side, int width,
+                          bool is_reverse = false, int op = H2X_HALO_ID)
+{
+    mi355x::dispatch("halo_transfer_gpu", src, src, dst, dim, src_side, width, is_reverse, op);
+}
+inline void shuffle_pack(const ShufflePlan& plan, BaseTensor& tensor, BaseTensor& buffer)
+{
+    const bool is_pack = true;
+    mi355x::dispatch("shuffle_gpu", tensor, plan, tensor, buffer, is_pack);
+}
+inline void shuffle_unpack(const ShufflePlan& plan, BaseTensor& tensor, BaseTensor& buffer)
+{
+    const bool is_pack = false;
+    mi355x::dispatch("shuffle_gpu", tensor, plan, tensor, buffer, is_pack);
+}
+inline void softmax_instance_forward(const BaseTensor& x, BaseTensor& y)
+{
+    mi355x::dispatch("softmax_instance_forward_gpu", x, x, y);
+}
+inline void softmax_instance_backward(const BaseTensor& y, const BaseTensor& dy, BaseTensor& dx)
+{
+    mi355x::dispatch("softmax_instance_backward_gpu", y, y, dy, dx);
 }
 
 } // namespace h2

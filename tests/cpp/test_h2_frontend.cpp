@@ -25,6 +25,11 @@ void orc_bn_backprop2_f32(int, int, size_t, size_t, size_t, size_t, size_t, cons
                           float);
 void orc_softmax_channel_forward_f32(int, int, size_t, const float*, float*);
 void orc_softmax_channel_backward_f32(int, int, size_t, const float*, const float*, float*);
+void orc_softmax_instance_max_f32(int, size_t, const float*, float*);
+void orc_softmax_instance_exp_f32(int, size_t, const float*, const float*, float*, float*);
+void orc_softmax_instance_normalize_f32(int, size_t, const float*, float*);
+void orc_softmax_instance_dot_f32(int, size_t, const float*, const float*, float*);
+void orc_softmax_instance_gradient_f32(int, size_t, const float*, const float*, const float*, float*);
 }
 
 using namespace h2;
@@ -311,8 +316,233 @@ static void test_errors()
     CHECK_THROWS(internal::call_dispatch_entry("probe_gpu", key, cbx, five));
 }
 
+// A strided tensor holding `values` at its elements (natural order), everything else `fill`.
+template <typename T>
+static std::vector<T> scatter_strided(const ShapeTuple& shape, const StrideTuple& strides, size_t span,
+                                      const std::vector<T>& values, T fill)
+{
+    std::vector<T> h(span, fill);
+    size_t i = 0;
+    const StrideTuple s[1] = {strides};
+    mi355x::for_each_element(shape, s, [&](const DataIndexType* o) { h[o[0]] = values[i++]; });
+    return h;
+}
+
+// Every operator of tensor_ops_mi355x.hpp on a GPU tensor and on a CPU tensor with the
+// same contents: the two arms must leave the same bits (sums: the same value to 1e-12,
+// both add in float64), and both must match plain host arithmetic.
+static void test_both_arms()
+{
+    const ComputeStream gs(Device::GPU), cs(Device::CPU);
+    const ShapeTuple shape{7, 5, 3, 2};
+    const StrideTuple halo_strides{1, 9, 9 * 8, 9 * 8 * 3}; // a 7 x 5 interior inside 9 x 8 rows
+    const size_t span = 9 * 8 * 3 * 2;
+    const DTTuple types = channel_types(4);
+    const size_t n = product<size_t>(shape);
+    std::vector<double> vals(n);
+    for (size_t i = 0; i < n; ++i)
+        vals[i] = 0.25 * (double) i - 3.0;
+    const std::vector<double> image = scatter_strided(shape, halo_strides, span, vals, -99.0);
+    double *dev_a = nullptr, *dev_b = nullptr;
+    check_hip(hipMalloc(reinterpret_cast<void**>(&dev_a), span * 8), "hipMalloc");
+    check_hip(hipMalloc(reinterpret_cast<void**>(&dev_b), n * 8), "hipMalloc");
+    std::vector<double> host_a = image, host_b(n, 0.0);
+    check_hip(hipMemcpy(dev_a, image.data(), span * 8, hipMemcpyHostToDevice), "upload");
+    Tensor<double> ga(Device::GPU, dev_a, shape, types, halo_strides, gs);
+    Tensor<double> gb(Device::GPU, dev_b, shape, types, get_contiguous_strides(shape), gs);
+    Tensor<double> ca(Device::CPU, host_a.data(), shape, types, halo_strides, cs);
+    Tensor<double> cb(Device::CPU, host_b.data(), shape, types, get_contiguous_strides(shape), cs);
+    auto same = [&](const char* what) {
+        std::vector<double> a(span), b(n);
+        check_hip(hipDeviceSynchronize(), "sync");
+        check_hip(hipMemcpy(a.data(), dev_a, span * 8, hipMemcpyDeviceToHost), "download");
+        check_hip(hipMemcpy(b.data(), dev_b, n * 8, hipMemcpyDeviceToHost), "download");
+        if (std::memcmp(a.data(), host_a.data(), span * 8) != 0 || std::memcmp(b.data(), host_b.data(), n * 8) != 0)
+        {
+            std::printf("FAILED: GPU and CPU arms differ after %s\n", what);
+            std::exit(1);
+        }
+    };
+    scale(ga, 2.0);
+    scale(ca, 2.0);
+    same("scale");
+    for (size_t i = 0; i < span; ++i)
+        CHECK(host_a[i] == (image[i] == -99.0 ? -99.0 : 2.0 * image[i])); // the gaps are not touched
+    copy_values(ga, gb);
+    copy_values(ca, cb);
+    same("copy_values");
+    for (size_t i = 0; i < n; ++i)
+        CHECK(host_b[i] == 2.0 * vals[i]);
+    scale_bias(ga, gb, 0.5, 1.0);
+    scale_bias(ca, cb, 0.5, 1.0);
+    same("scale_bias");
+    for (size_t i = 0; i < n; ++i)
+        CHECK(host_b[i] == vals[i] + 1.0);
+    // sums over space and samples into a per-channel tensor, through the type-erased front too
+    const ShapeTuple rshape{1, 1, 3, 1};
+    Tensor<double> gr(Device::GPU, rshape, types, gs);
+    std::vector<double> host_r(3, 10.0);
+    upload(gr, host_r);
+    Tensor<double> cr(Device::CPU, host_r.data(), rshape, types, get_contiguous_strides(rshape), cs);
+    const BaseTensor& bga = ga;
+    BaseTensor& bgr = gr;
+    reduce_sum(bga, bgr, true);
+    reduce_sum(ca, cr, true);
+    const std::vector<double> got_r = download(gr);
+    for (int c = 0; c < 3; ++c)
+    {
+        double want = 10.0;
+        for (int s = 0; s < 2; ++s)
+            for (int i = 0; i < 35; ++i)
+            {
+                const double x = 2.0 * vals[(s * 3 + c) * 35 + i];
+                want += x * x;
+            }
+        CHECK(std::fabs(got_r[c] - want) <= 1e-12 * want && std::fabs(host_r[c] - want) <= 1e-12 * want);
+    }
+    // clear_halo, halo pack / unpack and halo_transfer on contiguous tensors whose shape includes the halo
+    const ShapeTuple hshape{10, 6, 3, 2};
+    const size_t ht = product<size_t>(hshape);
+    std::vector<double> h1(ht), h2v(ht);
+    for (size_t i = 0; i < ht; ++i)
+    {
+        h1[i] = 1.0 + (double) i;
+        h2v[i] = -2.0 * (double) i;
+    }
+    std::vector<double> c1 = h1, c2 = h2v, cbuf(ht, 0.0); // room for the largest strip
+    Tensor<double> g1(Device::GPU, hshape, types, gs), g2(Device::GPU, hshape, types, gs);
+    Tensor<double> gbuf(Device::GPU, ShapeTuple{(DimType) ht}, DTTuple{DT::Any}, gs);
+    upload(g1, h1);
+    upload(g2, h2v);
+    upload(gbuf, cbuf);
+    Tensor<double> t1(Device::CPU, c1.data(), hshape, types, get_contiguous_strides(hshape), cs);
+    Tensor<double> t2(Device::CPU, c2.data(), hshape, types, get_contiguous_strides(hshape), cs);
+    Tensor<double> tbuf(Device::CPU, cbuf.data(), ShapeTuple{(DimType) ht}, DTTuple{DT::Any}, StrideTuple{1}, cs);
+    auto same_halo = [&](const char* what) {
+        const std::vector<double> a = download(g1), b = download(g2), c = download(gbuf);
+        if (a != c1 || b != c2 || c != cbuf)
+        {
+            std::printf("FAILED: GPU and CPU arms differ after %s\n", what);
+            std::exit(1);
+        }
+    };
+    clear_halo(g2, 1, 1);
+    clear_halo(t2, 1, 1);
+    same_halo("clear_halo");
+    for (size_t i = 0; i < ht; ++i)
+    {
+        const size_t h = (i / 10) % 6;
+        CHECK(c2[i] == ((h == 0 || h == 5) ? 0.0 : h2v[i]));
+    }
+    for (int width : {1, 2})
+        for (int dim : {0, 1, 2})
+        {
+            if (2 * width > hshape[dim])
+                continue;
+            halo_pack(g1, dim, H2X_RHS, width, gbuf);
+            halo_pack(t1, dim, H2X_RHS, width, tbuf);
+            halo_unpack(g2, dim, H2X_LHS, width, gbuf);
+            halo_unpack(t2, dim, H2X_LHS, width, tbuf);
+            same_halo("halo pack + unpack");
+            halo_pack(g1, dim, H2X_LHS, width, gbuf, true);
+            halo_pack(t1, dim, H2X_LHS, width, tbuf, true);
+            halo_unpack(g2, dim, H2X_RHS, width, gbuf, true, H2X_HALO_SUM);
+            halo_unpack(t2, dim, H2X_RHS, width, tbuf, true, H2X_HALO_SUM);
+            same_halo("reverse halo pack + SUM unpack");
+            halo_transfer(g1, g2, dim, H2X_RHS, width);
+            halo_transfer(t1, t2, dim, H2X_RHS, width);
+            same_halo("halo_transfer");
+            halo_transfer(g2, g1, dim, H2X_LHS, width, true, H2X_HALO_MAX);
+            halo_transfer(t2, t1, dim, H2X_LHS, width, true, H2X_HALO_MAX);
+            same_halo("reverse halo_transfer with MAX");
+        }
+    // a transfer equals pack on the source + unpack on the destination
+    {
+        std::vector<double> ref = c2;
+        Tensor<double> tr(Device::CPU, ref.data(), hshape, types, get_contiguous_strides(hshape), cs);
+        halo_pack(t1, 0, H2X_LHS, 1, tbuf);
+        halo_unpack(tr, 0, H2X_RHS, 1, tbuf);
+        halo_transfer(t1, t2, 0, H2X_LHS, 1);
+        CHECK(ref == c2);
+    }
+    CHECK_THROWS(halo_transfer(g1, t2, 0, H2X_LHS, 1));   // tensors on different devices
+    Tensor<double> bad(Device::CPU, ShapeTuple{1, 2, 3, 1}, types, cs);
+    CHECK_THROWS(reduce_sum(ca, bad));                    // extent 2 is neither 1 nor 5
+    check_hip(hipFree(dev_a), "hipFree");
+    check_hip(hipFree(dev_b), "hipFree");
+}
+
+// shuffle pack / unpack of one rank through a ShufflePlan: a 8 x 6 x 2 x 2 local tensor cut
+// for a 2 x 2 peer grid; the buffer holds the four boxes one after the other, each in its
+// own natural order (legacy/src/tensor/shuffle_mpi_cuda.cu:42-98).
+static void test_shuffle()
+{
+    const ComputeStream gs(Device::GPU);
+    const ShapeTuple shape{8, 6, 2, 2};
+    const size_t n = product<size_t>(shape);
+    const std::vector<int32_t> limits{4, 8, 3, 6, 2, 2};
+    const std::vector<int32_t> displs{0, 48, 96, 144};
+    ShufflePlan plan(shape, get_contiguous_strides(shape), ShapeTuple{2, 2, 1, 1}, limits, displs, 4);
+    std::vector<float> h(n);
+    for (size_t i = 0; i < n; ++i)
+        h[i] = (float) i;
+    Tensor<float> t(Device::GPU, shape, channel_types(4), gs), back(Device::GPU, shape, channel_types(4), gs);
+    Tensor<float> buf(Device::GPU, ShapeTuple{(DimType) n}, DTTuple{DT::Any}, gs);
+    upload(t, h);
+    upload(back, std::vector<float>(n, -1.0f));
+    shuffle_pack(plan, t, buf);
+    const std::vector<float> packed = download(buf);
+    size_t o = 0;
+    for (int ph = 0; ph < 2; ++ph)          // peers in rank order: dimension 0 of the grid fastest
+        for (int pw = 0; pw < 2; ++pw)
+        {
+            o = displs[ph * 2 + pw];
+            for (int s = 0; s < 2; ++s)
+                for (int c = 0; c < 2; ++c)
+                    for (int y = 0; y < 3; ++y)
+                        for (int x = 0; x < 4; ++x)
+                            CHECK(packed[o++] == h[((s * 2 + c) * 6 + ph * 3 + y) * 8 + pw * 4 + x]);
+        }
+    BaseTensor &bt = back, &bb = buf;
+    shuffle_unpack(plan, bt, bb);           // type-erased front
+    CHECK(download(back) == h);
+    Tensor<float> cpu(Device::CPU, shape, channel_types(4)), cbuf(Device::CPU, ShapeTuple{(DimType) n}, DTTuple{DT::Any});
+    CHECK_THROWS(shuffle_pack(plan, cpu, cbuf));   // no CPU implementation
+}
+
+static void test_softmax_instance()
+{
+    const ShapeTuple shape{9, 7, 5, 3};
+    const size_t total = product<size_t>(shape), size = total / 3;
+    const ComputeStream stream(Device::GPU);
+    Tensor<float> x(Device::GPU, shape, channel_types(4), stream), y(Device::GPU, shape, channel_types(4), stream),
+        dy(Device::GPU, shape, channel_types(4), stream), dx(Device::GPU, shape, channel_types(4), stream);
+    const std::vector<float> hx = randn(total, 5, 2.0f), hdy = randn(total, 6);
+    upload(x, hx);
+    upload(dy, hdy);
+    softmax_instance_forward(x, y);
+    const BaseTensor &by = y, &bdy = dy;
+    BaseTensor& bdx = dx;
+    softmax_instance_backward(by, bdy, bdx);
+    std::vector<float> wy(total), wdx(total), smax(3), sexp(3), sdp(3);
+    orc_softmax_instance_max_f32(3, size, hx.data(), smax.data());
+    orc_softmax_instance_exp_f32(3, size, hx.data(), smax.data(), wy.data(), sexp.data());
+    orc_softmax_instance_normalize_f32(3, size, sexp.data(), wy.data());
+    const std::vector<float> gy = download(y);
+    orc_softmax_instance_dot_f32(3, size, gy.data(), hdy.data(), sdp.data());
+    orc_softmax_instance_gradient_f32(3, size, gy.data(), hdy.data(), sdp.data(), wdx.data());
+    CHECK(max_rel(gy, wy) <= 1e-5);
+    // dx = y * (dy - dp) cancels: compare against the scale of its terms
+    const std::vector<float> gdx = download(dx);
+    for (size_t i = 0; i < total; ++i)
+        CHECK(std::fabs(gdx[i] - wdx[i]) <= 1e-5 * (std::fabs(gy[i] * hdy[i]) + std::fabs(gy[i])));
+}
+
 int main()
 {
+    test_both_arms();
+    test_shuffle();
+    test_softmax_instance();
     test_batchnorm(ShapeTuple{14, 14, 8, 4});
     test_batchnorm(ShapeTuple{6, 5, 7, 3, 2});
     test_batchnorm(ShapeTuple{33, 5, 2}); // one spatial dimension, odd length
