@@ -6,14 +6,16 @@ One "step" is one pass of the path BASELINE.json's metric is quoted on:
   * one full halo exchange (pack + unpack, 3 dimension phases, width 1) of a
     periodic 2 x 2 x 2 grid of virtual ranks, each N1 C32 128^3 fp32 (config 2).
 `value` is the algorithmic bytes of a step divided by its wall time, inputs
-resident in HBM.  The other BASELINE configs (2-D batch-norm forward, channel
-softmax, shuffle) are timed once each and reported under "breakdown".
+resident in HBM.  Every BASELINE config, the exchange's phases and the
+follow-on operators are timed separately under "breakdown" (GPU time through
+HIP-graph replay, and the eager Python figure beside it where it differs).
 
 Prints ONE JSON line.  `--gpus N` with N > 1 exits: this build runs on one GPU.
 """
 from __future__ import annotations
 
 import argparse
+import hashlib
 import json
 import os
 import statistics
@@ -33,12 +35,14 @@ def _gbs(nbytes: float, ms: float) -> float:
 
 
 def _time_events(fn, iters: int, warmup: int, inner: int = 4):
-    """Median and minimum milliseconds of one fn() measured with events on the
-    current stream (the stream every kernel of fn is launched on).  `inner`
+    """Median and minimum milliseconds of one eager fn() measured with events on
+    the current stream (the stream every kernel of fn is launched on).  `inner`
     calls are issued back to back between the two events so that the launch
     latency of a call is hidden behind the execution of the previous one -- the
     reference's harness hides it with a spin kernel
-    (legacy/benchmarks/distconv_benchmark_bn.cpp:254-295)."""
+    (legacy/benchmarks/distconv_benchmark_bn.cpp:254-295).  Calls shorter than
+    their own Python + launch cost (a few tens of microseconds) are bound by
+    the host here; _time_graph gives their GPU time."""
     import torch
     for _ in range(warmup):
         fn()
@@ -52,6 +56,33 @@ def _time_events(fn, iters: int, warmup: int, inner: int = 4):
         e1.record()
         e1.synchronize()
         times.append(e0.elapsed_time(e1) / inner)
+    return statistics.median(times), min(times)
+
+
+def _time_graph(fn, iters: int, warmup: int, inner: int = 4):
+    """Median and minimum milliseconds of one fn() with `inner` calls captured
+    into a HIP graph and the graph replayed between two events: the GPU's time
+    for the launches, free of host enqueue cost."""
+    import torch
+    for _ in range(max(warmup, 1)):
+        fn()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for _ in range(inner):
+            fn()
+    for _ in range(2):
+        graph.replay()
+    torch.cuda.synchronize()
+    times = []
+    for _ in range(iters):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        graph.replay()
+        e1.record()
+        e1.synchronize()
+        times.append(e0.elapsed_time(e1) / inner)
+    del graph
     return statistics.median(times), min(times)
 
 
@@ -75,17 +106,26 @@ def _time_events_cold(fn, flush, iters: int, warmup: int):
 
 
 class BatchNormWorkload:
-    """BatchNormalization forward + backward on one rank."""
+    """BatchNormalization forward + backward on one rank.  `overlap` puts a
+    halo of that width on every spatial dimension (the strided kernels)."""
 
-    def __init__(self, shape_np, seed):
+    def __init__(self, shape_np, seed, overlap: int = 0, fuse_local: bool = True):
         import torch
         from dihydrogen_amd.layers import BatchNormalization
         from dihydrogen_amd.tensor import Distribution, LocaleVirtual, Tensor
         g = torch.Generator(device="cuda").manual_seed(seed)
         nd = len(shape_np)
         c = shape_np[1]
-        dist = Distribution.make_localized_distribution(nd)
-        mk = lambda: Tensor(list(shape_np[::-1]), LocaleVirtual(0, 1), dist).allocate()
+        if overlap:
+            # a distribution split over every spatial dimension gives the tensor its halos; one
+            # virtual rank of it is enough to run the kernels on a haloed shard of this local size
+            locale = [2] * (nd - 2) + [1, 1]
+            dist = Distribution.make_overlapped_distribution(locale, [overlap] * (nd - 2) + [0, 0])
+            gshape = [2 * e for e in shape_np[:1:-1]] + [shape_np[1], shape_np[0]]
+            mk = lambda: Tensor(gshape, LocaleVirtual(0, 2 ** (nd - 2)), dist).allocate()
+        else:
+            dist = Distribution.make_localized_distribution(nd)
+            mk = lambda: Tensor(list(shape_np[::-1]), LocaleVirtual(0, 1), dist).allocate()
         self.x, self.y, self.dy, self.dx = mk(), mk(), mk(), mk()
         self.x.data.normal_(0, 1, generator=g)
         self.dy.data.normal_(0, 1, generator=g)
@@ -94,12 +134,15 @@ class BatchNormWorkload:
         self.mean, self.var = torch.empty(c, device="cuda"), torch.empty(c, device="cuda")
         self.rm, self.rv = torch.zeros(c, device="cuda"), torch.ones(c, device="cuda")
         self.grads = [torch.empty(c, device="cuda") for _ in range(4)]
-        self.bn = BatchNormalization(nd, 0.9, 1e-5)
+        self.bn = BatchNormalization(nd, 0.9, 1e-5, fuse_local=fuse_local)
         self.elems = self.x.get_local_size()
 
     def forward(self):
         self.bn.forward(self.x, self.mean, self.var, self.rm, self.rv, self.scale, self.bias,
                         self.y, True)
+
+    def backward(self):
+        self.bn.backward(self.x, self.dy, self.mean, self.var, self.scale, *self.grads, self.dx)
 
     def backward_reduce(self):
         self.bn.backward_stage1(self.x, self.dy, self.mean, self.var, self.scale, *self.grads)
@@ -108,10 +151,6 @@ class BatchNormWorkload:
     def backward_apply(self):
         self.bn.backward_stage2(self.x, self.dy, self.mean, self.var, self.scale, self.grads[2],
                                 self.grads[3], self.dx)
-
-    def backward(self):
-        self.backward_reduce()
-        self.backward_apply()
 
 
 class HaloWorkload:
@@ -139,7 +178,7 @@ class HaloWorkload:
 
 
 class SoftmaxWorkload:
-    def __init__(self, shape_np, seed):
+    def __init__(self, shape_np, seed, instance: bool = False):
         import torch
         from dihydrogen_amd.layers import Softmax, SoftmaxMode
         from dihydrogen_amd.tensor import Distribution, LocaleVirtual, Tensor
@@ -150,7 +189,7 @@ class SoftmaxWorkload:
         self.x.data.normal_(0, 2, generator=g)  # sigma = 2
         self.dy.data.normal_(0, 1, generator=g)
         self.sm = Softmax()
-        self.sm.setup(self.x, SoftmaxMode.CHANNEL)
+        self.sm.setup(self.x, SoftmaxMode.INSTANCE if instance else SoftmaxMode.CHANNEL)
         self.elems = self.x.get_local_size()
 
     def forward(self):
@@ -161,16 +200,16 @@ class SoftmaxWorkload:
 
 
 class ShuffleWorkload:
-    """Sample-parallel (N over 4 ranks) <-> spatial-parallel (H/2 x W/2)."""
+    """Sample-parallel (N over `ranks` ranks) <-> spatial-parallel (H x W grid)."""
 
-    def __init__(self, gshape, seed):
+    def __init__(self, gshape, seed, ranks=4, grid=(2, 2)):
         import torch
         from dihydrogen_amd.layers import TensorShufflerVirtual
         from dihydrogen_amd.tensor import Distribution, LocaleVirtual, Tensor
         g = torch.Generator(device="cuda").manual_seed(seed)
-        sd, dd = Distribution([1, 1, 1, 4]), Distribution([2, 2, 1, 1])
-        self.src = [Tensor(gshape, LocaleVirtual(r, 4), sd).allocate() for r in range(4)]
-        self.dst = [Tensor(gshape, LocaleVirtual(r, 4), dd).allocate() for r in range(4)]
+        sd, dd = Distribution([1, 1, 1, ranks]), Distribution([grid[0], grid[1], 1, 1])
+        self.src = [Tensor(gshape, LocaleVirtual(r, ranks), sd).allocate() for r in range(ranks)]
+        self.dst = [Tensor(gshape, LocaleVirtual(r, ranks), dd).allocate() for r in range(ranks)]
         for t in self.src:
             t.data.uniform_(-1, 1, generator=g)
         self.sh = TensorShufflerVirtual(self.src, self.dst)
@@ -185,71 +224,152 @@ class ShuffleWorkload:
         self.sh.shuffle_backward()
 
 
-def cpu_baseline(repeats: int = 9):
-    """The CPU oracle (this repository's restatement of the reference kernels;
+def _cpu_model() -> str:
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_baseline(repeats: int = 5):
+    """The CPU oracle (this repository's restatement of the reference kernels:
     the reference has no CPU implementation of batch-norm, softmax or halo
-    packing) on the same step: config 3 batch-norm forward+backward plus the
-    config 2 exchange for 2 of the 8 virtual ranks' worth of faces."""
+    packing, and its CPU shuffler is restated too) timed on the host cores, per
+    BASELINE config, on bounded samples that are stated with each figure."""
     import numpy as np
     import oracle
+    from oracle import geometry as G
     lib = oracle.lib()
     lib.orc_num_threads.restype = __import__("ctypes").c_int
     threads = lib.orc_num_threads()
     rng = np.random.default_rng(SEED)
+
+    def med(fn):
+        """Median of at least `repeats` runs and at least a second of them."""
+        fn()
+        ts = []
+        while len(ts) < repeats or (sum(ts) < 1.0 and len(ts) < 200):
+            t0 = time.perf_counter()
+            fn()
+            ts.append(time.perf_counter() - t0)
+        return statistics.median(ts)
+
+    def entry(nbytes, elems, seconds, sample):
+        return {"GB/s": nbytes / seconds / 1e9, "Gelem/s": elems / seconds / 1e9, "seconds": seconds,
+                "bytes": nbytes, "sample": sample}
+
+    configs = {}
+    # C1: 2-D batch-norm forward, in full
+    x1 = rng.standard_normal((8, 64, 56, 56), dtype=np.float32)
+    sc, bi = rng.uniform(0.5, 1.5, 64).astype(np.float32), (0.1 * rng.standard_normal(64)).astype(np.float32)
+    t = med(lambda: oracle.bn_forward(x1, sc, bi, np.zeros(64, np.float32), np.ones(64, np.float32)))
+    configs["C1_bn2d_fwd"] = entry(3 * x1.size * 4, x1.size, t, "in full")
+    # C3: 3-D batch-norm forward + backward, in full
     shp = (4, 64, 64, 64, 64)
-    x = rng.standard_normal(shp, dtype=np.float32)
-    dy = rng.standard_normal(shp, dtype=np.float32)
-    scale = rng.uniform(0.5, 1.5, 64).astype(np.float32)
-    bias = (0.1 * rng.standard_normal(64)).astype(np.float32)
+    x3 = rng.standard_normal(shp, dtype=np.float32)
+    dy3 = rng.standard_normal(shp, dtype=np.float32)
+
+    def c3():
+        y, mean, var = oracle.bn_forward(x3, sc, bi, np.zeros(64, np.float32), np.ones(64, np.float32))
+        oracle.bn_backward(x3, dy3, mean, var, sc)
+
+    t3 = med(c3)
+    configs["C3_bn3d_fwd_bwd"] = entry(8 * x3.size * 4, x3.size, t3, "in full")
+    del x3, dy3
+    # C2: halo pack + unpack of all 6 faces, 2 of the 8 ranks
     halo_ranks = 2
     fields = [rng.uniform(-1, 1, (1, 32, 130, 130, 130)).astype(np.float32) for _ in range(halo_ranks)]
     bufs = {d: np.empty(oracle.halo_size((130, 130, 130, 32, 1), d, 1), np.float32) for d in range(3)}
-    bn_bytes = 8 * x.size * 4
-    halo_bytes = halo_ranks * 3 * 2 * 2 * 2 * bufs[0].size * 4
 
-    def step():
-        rm, rv = np.zeros(64, np.float32), np.ones(64, np.float32)
-        y, mean, var = oracle.bn_forward(x, scale, bias, rm, rv)
-        oracle.bn_backward(x, dy, mean, var, scale)
+    def c2():
         for f in fields:
             for d in range(3):
                 for side in (0, 1):
                     oracle.halo_pack_or_unpack(f, d, side, 1, bufs[d], True)
                     oracle.halo_pack_or_unpack(f, d, side, 1, bufs[d], False)
 
-    step()
-    times = []
-    for _ in range(repeats):
-        t0 = time.perf_counter()
-        step()
-        times.append(time.perf_counter() - t0)
-    t = statistics.median(times)
+    t2 = med(c2)
+    halo_bytes = halo_ranks * 3 * 2 * 2 * 2 * bufs[0].size * 4
+    configs["C2_halo"] = entry(halo_bytes, halo_ranks * 12 * bufs[0].size, t2,
+                               f"{halo_ranks} of 8 ranks, all 6 faces each, pack + unpack")
+    del fields
+    # C4: channel softmax forward + backward, in full
+    x4 = (2 * rng.standard_normal((16, 21, 256, 256), dtype=np.float32))
+    dy4 = rng.standard_normal((16, 21, 256, 256), dtype=np.float32)
+
+    def c4():
+        y = oracle.softmax_channel_forward(x4)
+        oracle.softmax_channel_backward(y, dy4)
+
+    t4 = med(c4)
+    configs["C4_softmax_fwd_bwd"] = entry(5 * x4.size * 4, x4.size, t4, "in full")
+    del x4, dy4
+    # C5: the shuffler's pack + unpack of one direction.  Generic per-element path (single-threaded,
+    # as the reference's: shuffle_mpi.hpp:688-706,851-872) on one of the four ranks; OpenMP row-copy
+    # path (shuffle_mpi.hpp:708-849,874-947) on all four.
+    shape5, n5 = (128, 128, 64, 32), 4
+    src_g = [G.TensorGeom(shape5, G.Dist((1, 1, 1, 4), (1, 1, 1, 4), [0] * 4), r) for r in range(n5)]
+    dst_g = [G.TensorGeom(shape5, G.Dist((2, 2, 1, 1), (2, 2, 1, 1), [0] * 4), r) for r in range(n5)]
+    # every rank has arrays of its own, as in a real job: nothing is shared through the caches
+    fields5 = [rng.uniform(-1, 1, src_g[r].local_size).astype(np.float32) for r in range(n5)]
+    bufs5 = [np.empty(src_g[r].local_size, np.float32) for r in range(n5)]
+    outs5 = [np.empty(dst_g[r].local_size, np.float32) for r in range(n5)]
+    field = fields5[0]
+    tables = []
+    for r in range(n5):
+        _, sd, _, rd = G.counts_and_displs(src_g[r], dst_g[r])
+        tables.append((G.rank_limits(src_g[r], dst_g[r]), sd, G.rank_limits(dst_g[r], src_g[r]), rd))
+
+    def generic(r):
+        lim, sd, lim_d, rd = tables[r]
+        field, buf, out = fields5[r], bufs5[r], outs5[r]
+        oracle.shuffle_pack_or_unpack(field, src_g[r].local_shape, src_g[r].strides(), (2, 2, 1, 1), lim, buf, sd, True)
+        oracle.shuffle_pack_or_unpack(out, dst_g[r].local_shape, dst_g[r].strides(), (1, 1, 1, 4), lim_d, buf, rd, False)
+
+    def rows():
+        for r in range(n5):
+            lim, sd, lim_d, rd = tables[r]
+            field, buf, out = fields5[r], bufs5[r], outs5[r]
+            oracle.shuffle_rows(field, src_g[r].local_shape, src_g[r].strides(), (2, 2, 1, 1), lim, buf, sd, True)
+            oracle.shuffle_rows(out, dst_g[r].local_shape, dst_g[r].strides(), (1, 1, 1, 4), lim_d, buf, rd, False)
+
+    t0 = time.perf_counter()
+    generic(0)
+    tg = time.perf_counter() - t0
+    per_rank = 4 * field.size * 4  # pack read + write, unpack read + write
+    configs["C5_shuffle_generic"] = entry(per_rank, field.size, tg,
+                                          "1 of 4 ranks, forward direction, per-element path on one thread (one run)")
+    tr = med(rows)
+    configs["C5_shuffle_row_copy"] = entry(n5 * per_rank, n5 * field.size, tr,
+                                           "all 4 ranks, forward direction, OpenMP row-copy path")
+    # the step the headline value is quoted on: C3 in full + C2 scaled to its 2-rank sample
+    step_bytes = 8 * 67108864 * 4 + halo_bytes
     return {
-        "value": (bn_bytes + halo_bytes) / t / 1e9,
+        "value": step_bytes / (t3 + t2) / 1e9,
         "unit": "GB/s",
         "cores": threads,
         "kind": "port",
-        "sample": (f"config 3 batch-norm fwd+bwd in full (67108864 elems) + config 2 exchange of "
-                   f"{halo_ranks} of 8 ranks; median of {repeats} runs, {t:.3f} s each; "
-                   f"gcc -O3 -fopenmp, OMP threads = {threads}"),
+        "cpu_model": _cpu_model(),
+        "sample": (f"config 3 batch-norm fwd+bwd in full + config 2 exchange of {halo_ranks} of 8 ranks; "
+                   f"medians of {repeats} runs ({t3:.3f} s + {t2:.3f} s); gcc -O3 -fopenmp, "
+                   f"OMP threads = {threads}"),
+        "configs": configs,
     }
 
 
-# HBM traffic per launch measured with rocprofv3 --pmc (profiles/bench_pmc_traffic.txt):
-# FETCH_SIZE and WRITE_SIZE in KiB per dispatch; FETCH_SIZE reads 0.5x for full-line
-# streaming reads on this stack (calibrated there on a copy of known size), WRITE_SIZE 1.0x.
-PMC_KIB = {  # label -> (FETCH_SIZE KiB, fetch scale, WRITE_SIZE KiB) per launch
-    "bn_sums": (131095, 2.0, 128),
-    "bn_apply": (131102, 2.0, 262162),
-    "bn_backprop1": (262182, 2.0, 128),
-    "bn_backprop2": (262178, 2.0, 262144),
-    "halo_dim0_pack": (154900, 2.0, 16900),    # 8 faces per launch, two launches per step
-    "halo_dim0_unpack": (8503, 2.0, 135200),
-    "halo_dim1_pack": (21017, 2.0, 33800),
-    "halo_dim1_unpack": (16954, 2.0, 37365),
-    "halo_dim2_pack": (17048, 2.0, 33800),
-    "halo_dim2_unpack": (16956, 2.0, 35112),
-}
+# HBM-side traffic per launch measured with rocprofv3 --pmc (profiles/bench_pmc_traffic.txt):
+# request counters between the L2 and the fabric, converted to bytes there
+# (TCC_EA0_RDREQ, TCC_EA0_RDREQ_32B, TCC_BUBBLE; TCC_EA0_WRREQ, TCC_EA0_WRREQ_64B).
+# label -> (bytes read, bytes written) per launch
+PMC_TRAFFIC = {}
+# sha256 of the kernel sources the table was measured with (see kernel_sources_sha()); with other
+# sources the traffic fields are omitted
+PMC_SOURCES_SHA = ""
+PMC_COMMIT = ""
 
 KERNEL_OF = {
     "bn_sums": "bn_sums_kernel<float,4> (+bn_finish_kernel<float,2>)",
@@ -257,20 +377,32 @@ KERNEL_OF = {
     "bn_apply": "bn_apply_kernel<float,4>",
     "bn_backprop1": "bn_backprop1_kernel<float,4> (+bn_finish_kernel<float,4>)",
     "bn_backprop2": "bn_backprop2_kernel<float,4>",
-    "halo_dim0_pack": "box_copy_kernel<u32,1,OpId,sparse>",
-    "halo_dim0_unpack": "box_copy_kernel<u32,1,OpId,sparse>",
-    "halo_dim1_pack": "box_copy_kernel<u32,2,OpId>",
-    "halo_dim1_unpack": "box_copy_kernel<u32,2,OpId>",
-    "halo_dim2_pack": "box_copy_kernel<u32,4,OpId>",
-    "halo_dim2_unpack": "box_copy_kernel<u32,4,OpId>",
+    "halo_dim0_pack": "box_copy_kernel<u32,1,OpId,sparse,pack>",
+    "halo_dim0_unpack": "box_copy_kernel<u32,1,OpId,sparse,unpack>",
+    "halo_dim1_pack": "box_copy_kernel<u32,4,OpId,dense,pack>",
+    "halo_dim1_unpack": "box_copy_kernel<u32,4,OpId,dense,unpack>",
+    "halo_dim2_pack": "box_copy_kernel<u32,4,OpId,dense,pack>",
+    "halo_dim2_unpack": "box_copy_kernel<u32,4,OpId,dense,unpack>",
 }
+
+
+def kernel_sources_sha() -> str:
+    """Hash of the HIP sources of libh2x.so: ties measured-traffic constants to
+    the kernels they were measured on."""
+    h = hashlib.sha256()
+    d = os.path.join(ROOT, "dihydrogen_amd", "csrc")
+    for name in sorted(os.listdir(d)):
+        if name.endswith((".hip", ".hpp")):
+            with open(os.path.join(d, name), "rb") as f:
+                h.update(name.encode() + b"\0" + f.read())
+    return h.hexdigest()[:16]
 
 
 def dim0_study():
     """The dimension-0 phase of the config 2 exchange (one 4-byte element per
     520-byte row and side) as a rate of memory transactions: every packed
     element costs the fetch of a 128-byte line (two neighbouring rows' ends
-    share one), every unpacked element a 32-byte masked write.  Timed for
+    share one), every unpacked row seam an 8-byte partial write.  Timed for
     launch groups of 2, 4 and 8 ranks, pack and unpack alone and together, and
     for the tensor-to-tensor form."""
     from dihydrogen_amd import capi
@@ -280,7 +412,7 @@ def dim0_study():
     xch, dt = halo.xch, halo.ranks[0].h2x_dtype
     rows = 130 * 130 * 32                      # rows of one rank
     lines_per_rank = rows * (1 + 12 / 128)     # one line per row pair end, 12 bytes apart: 9 % straddle
-    writes_per_rank = 2 * rows
+    seams_per_rank = rows
     ident = HaloExchangeAccumOp.ID
 
     def faces(group, is_pack):
@@ -288,33 +420,32 @@ def dim0_study():
         for r in group:
             for side in (capi.LHS, capi.RHS):
                 peer = xch.find_peer_rank(r, 0, side)
-                buf = xch._recv_buffer(peer, 0, capi.LHS if side == capi.RHS else capi.RHS) if is_pack \
-                    else xch._recv_buffer(r, 0, side)
-                out.append(xch._face(r, 0, side, 1, buf, is_pack, False, ident))
+                buf = xch.recv_buffer(peer, 0, capi.LHS if side == capi.RHS else capi.RHS) if is_pack \
+                    else xch.recv_buffer(r, 0, side)
+                out.append(xch.make_face(r, 0, side, 1, buf, is_pack, False, ident))
         return (capi.HaloFace * len(out))(*out)
 
     def launch(arr):
         capi.check(lib.h2x_halo_pack_or_unpack_batched(dt, arr, len(arr), None), "halo")
 
-    result = {"rows_per_rank": rows, "lines_per_rank": int(lines_per_rank), "writes_per_rank": writes_per_rank,
+    result = {"rows_per_rank": rows, "lines_per_rank": int(lines_per_rank), "seam_writes_per_rank": seams_per_rank,
               "groups": {}}
     for size in (2, 4, 8):
         groups = [list(range(g, g + size)) for g in range(0, 8, size)]
         packs = [faces(g, True) for g in groups]
         unpacks = [faces(g, False) for g in groups]
-        t_pack = _time_events(lambda: [launch(a) for a in packs], 10, 3, inner=2)[0]
-        t_unpack = _time_events(lambda: [launch(a) for a in unpacks], 10, 3, inner=2)[0]
-        t_both = _time_events(lambda: [(launch(p), launch(u)) for p, u in zip(packs, unpacks)], 10, 3, inner=2)[0]
+        t_pack = _time_graph(lambda: [launch(a) for a in packs], 10, 3, inner=2)[0]
+        t_unpack = _time_graph(lambda: [launch(a) for a in unpacks], 10, 3, inner=2)[0]
+        t_both = _time_graph(lambda: [(launch(p), launch(u)) for p, u in zip(packs, unpacks)], 10, 3, inner=2)[0]
         result["groups"][str(size)] = {
             "pack_us": t_pack * 1e3, "unpack_us": t_unpack * 1e3, "pack_then_unpack_us": t_both * 1e3,
             "pack_Glines_per_s": 8 * lines_per_rank / (t_pack * 1e-3) / 1e9,
             "pack_line_traffic_GB/s": 8 * lines_per_rank * 128 / (t_pack * 1e-3) / 1e9,
-            "unpack_Gwrites_per_s": 8 * writes_per_rank / (t_unpack * 1e-3) / 1e9,
+            "unpack_Gseams_per_s": 8 * seams_per_rank / (t_unpack * 1e-3) / 1e9,
         }
     ov = [1, 0, 0, 0, 0]
-    t_fused = _time_events(lambda: xch.exchange(ov, ov, ov, ov, fused=True), 10, 3, inner=2)[0]
+    t_fused = _time_graph(lambda: xch.exchange(ov, ov, ov, ov, fused=True), 10, 3, inner=2)[0]
     result["fused_us"] = t_fused * 1e3
-    result["fused_Gtransactions_per_s"] = 8 * (lines_per_rank + writes_per_rank) / (t_fused * 1e-3) / 1e9
     return result
 
 
@@ -327,8 +458,12 @@ def main() -> int:
     ap.add_argument("--no-breakdown", action="store_true")
     ap.add_argument("--dim0-study", action="store_true",
                     help="instead of the benchmark: the innermost-dimension halo phase alone, by number of "
-                         "ranks per launch group, as cache lines and masked writes per second")
+                         "ranks per launch group, as cache lines and seam writes per second")
+    ap.add_argument("--sources-sha", action="store_true", help="print the hash of the kernel sources and exit")
     args = ap.parse_args()
+    if args.sources_sha:
+        print(kernel_sources_sha())
+        return 0
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (virtual ranks share it); "
               f"--gpus {args.gpus} is not supported", file=sys.stderr)
@@ -357,8 +492,8 @@ def main() -> int:
                   "bn_backprop2": 3 * S3 * 4}
     faces_per_launch = {}  # halo label -> faces in one launch (the exchange may split a phase)
 
-    # Every launch of the step is bracketed by a pair of events on the stream it is
-    # launched on (torch's current stream, whose handle the C ABI receives).
+    # Every launch is bracketed by a pair of events on the stream it is launched on
+    # (torch's current stream, whose handle the C ABI receives).
     events = {}
     recording = [False]
     only = [None]  # labels to instrument; None = all
@@ -381,8 +516,16 @@ def main() -> int:
     nps = b._num_per_sum(bn3.x)
 
     def step():
+        """The timed step: the layer's own forward() and backward() (two launches each: the
+        second kernel of each finishes the first one's channel sums) and the exchange."""
+        bn3.forward()
+        bn3.backward()
+        halo.run()
+
+    def step_staged():
+        """The same work with the staged batch-norm entry points (what a rank that all-reduces
+        between the stages runs), every launch labelled: the per-launch table."""
         timed("bn_sums", lambda: b.forward_stage1(bn3.x, bn3.mean, bn3.var, True))
-        b.forward_allreduce(bn3.mean, bn3.var, True)
         timed("bn_statistics", lambda: b.sums_to_statistics(nps, bn3.mean, bn3.var, bn3.rm, bn3.rv))
         timed("bn_apply", lambda: b.batch_normalization(bn3.x, bn3.mean, bn3.var, bn3.scale, bn3.bias, bn3.y))
         timed("bn_backprop1", bn3.backward_reduce)
@@ -399,10 +542,13 @@ def main() -> int:
     # warm-up, with every launch bracketed by events: finds the dominant kernel
     recording[0] = True
     for _ in range(max(args.warmup, 1)):
-        step()
+        step_staged()
     torch.cuda.synchronize()
     share0 = kernel_share(events, max(args.warmup, 1))
     dominant = max(share0, key=share0.get)
+    events.clear()
+    step()  # the fused entry points once, untimed (first-use allocations)
+    torch.cuda.synchronize()
     events.clear()
 
     # timed region: only the dominant kernel's launches carry events
@@ -420,24 +566,25 @@ def main() -> int:
     # a second, fully instrumented pass for the per-launch table
     only[0] = None
     for _ in range(args.steps):
-        step()
+        step_staged()
     torch.cuda.synchronize()
     recording[0] = False
     halo.xch.launch_hook = None
     for label, pairs in dominant_events.items():
         events[label] = pairs  # the dominant kernel's figures come from the timed region
 
+    sources_sha = kernel_sources_sha()
+    traffic_valid = bool(PMC_TRAFFIC) and sources_sha == PMC_SOURCES_SHA
     launches = {}
     for label, pairs in events.items():
         samples = [e0.elapsed_time(e1) for e0, e1 in pairs]
         # the dominant kernel's figure is the average over the timed region; the other launches come
         # from the instrumented pass, where the median keeps a late host enqueue out of the figure
         ms = statistics.mean(samples) if label in dominant_events else statistics.median(samples)
-        fetch_kib, scale, write_kib = PMC_KIB.get(label, (0, 0.0, 0))
         launches[label] = {
             "kernel": KERNEL_OF[label], "avg_launch_ms": ms, "algorithmic_bytes": algo_bytes[label],
             "GB/s": _gbs(algo_bytes[label], ms), "frac": _gbs(algo_bytes[label], ms) / HBM_PEAK_GBS,
-            "traffic": int((fetch_kib * scale + write_kib) * 1024) if label in PMC_KIB else None,
+            "traffic": sum(PMC_TRAFFIC[label]) if traffic_valid and label in PMC_TRAFFIC else None,
         }
         if label in faces_per_launch:
             launches[label]["faces"] = faces_per_launch[label]
@@ -446,76 +593,123 @@ def main() -> int:
     share = {}
     for label, v in launches.items():
         share.setdefault(v["kernel"], []).append(label)
-    dl = share[dominant]
+    dl = [l for l in share[dominant] if l in dominant_events] or share[dominant]
     d_ms = statistics.mean(launches[l]["avg_launch_ms"] for l in dl)
     d_bytes = statistics.mean(launches[l]["algorithmic_bytes"] for l in dl)
-    d_traffic = statistics.mean(launches[l]["traffic"] for l in dl)
+    d_traffic = (statistics.mean(launches[l]["traffic"] for l in dl)
+                 if all(launches[l]["traffic"] is not None for l in dl) else None)
     roofline = {
         "kernel": dominant, "launches_per_step": dl, "bound": "hbm",
         "achieved": _gbs(d_bytes, d_ms), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-        "frac": _gbs(d_bytes, d_ms) / HBM_PEAK_GBS, "traffic": int(d_traffic),
+        "frac": _gbs(d_bytes, d_ms) / HBM_PEAK_GBS,
+        "traffic": int(d_traffic) if d_traffic is not None else None,
         "avg_launch_ms": d_ms, "algorithmic_bytes": int(d_bytes),
-        "traffic_GB/s": _gbs(d_traffic, d_ms),
+        # the same launch priced by the bytes the memory system moved for it
+        "traffic_GB/s": _gbs(d_traffic, d_ms) if d_traffic is not None else None,
+        "frac_of_peak_in_traffic": _gbs(d_traffic, d_ms) / HBM_PEAK_GBS if d_traffic is not None else None,
+        "traffic_source": (f"rocprofv3 --pmc, profiles/bench_pmc_traffic.txt @ {PMC_COMMIT}, kernel sources "
+                           f"{PMC_SOURCES_SHA}" if traffic_valid else
+                           f"omitted: kernel sources {sources_sha} differ from the profiled {PMC_SOURCES_SHA or 'none'}"),
     }
 
     breakdown = {}
     if not args.no_breakdown:
         it, wu = 20, 5
 
-        def entry(nbytes, elems, med, mn):
-            return {"bytes": nbytes, "ms_median": med, "ms_min": mn, "GB/s": _gbs(nbytes, med),
-                    "frac_of_peak": _gbs(nbytes, med) / HBM_PEAK_GBS, "Gelem/s": elems / (med * 1e-3) / 1e9}
+        def entry(nbytes, elems, fn, inner=4, eager=True):
+            med, mn = _time_graph(fn, it, wu, inner)
+            e = {"bytes": nbytes, "ms_median": med, "ms_min": mn, "GB/s": _gbs(nbytes, med),
+                 "frac_of_peak": _gbs(nbytes, med) / HBM_PEAK_GBS, "Gelem/s": elems / (med * 1e-3) / 1e9,
+                 "timing": "HIP-graph replay (GPU time)"}
+            if eager:
+                e["ms_eager_median"] = _time_events(fn, it, wu, inner)[0]
+            return e
 
-        breakdown["C3_bn3d_fwd"] = entry(3 * S3 * 4, S3, *_time_events(bn3.forward, it, wu))
-        breakdown["C3_bn3d_bwd"] = entry(5 * S3 * 4, S3, *_time_events(bn3.backward, it, wu))
-        breakdown["C3_bn3d_fwd_bwd"] = entry(
-            8 * S3 * 4, S3, *_time_events(lambda: (bn3.forward(), bn3.backward()), it, wu))
-        breakdown["C2_halo_8ranks"] = entry(halo.bytes, halo.elems, *_time_events(halo.run, it, wu))
+        breakdown["C3_bn3d_fwd"] = entry(3 * S3 * 4, S3, bn3.forward)
+        breakdown["C3_bn3d_bwd"] = entry(5 * S3 * 4, S3, bn3.backward)
+        breakdown["C3_bn3d_fwd_bwd"] = entry(8 * S3 * 4, S3, lambda: (bn3.forward(), bn3.backward()), inner=2)
+        bn3.bn.fuse_local = False
+        breakdown["C3_bn3d_fwd_bwd_staged"] = entry(8 * S3 * 4, S3, lambda: (bn3.forward(), bn3.backward()), inner=2)
+        bn3.bn.fuse_local = True
+        breakdown["C2_halo_8ranks"] = entry(halo.bytes, halo.elems, halo.run, inner=2)
         for d, name in enumerate(("dim0_W", "dim1_H", "dim2_D")):
             ov = [1 if k == d else 0 for k in range(5)]
             fn = lambda ov=ov: halo.xch.exchange(ov, ov, ov, ov)
-            breakdown[f"C2_halo_{name}"] = entry(halo.bytes // 3, halo.elems // 3, *_time_events(fn, it, wu))
+            breakdown[f"C2_halo_{name}"] = entry(halo.bytes // 3, halo.elems // 3, fn)
         # the same exchange as tensor-to-tensor transfers (no buffers): half the bytes per strip
-        breakdown["C2_halo_8ranks_fused"] = entry(
-            halo.bytes // 2, halo.elems // 2, *_time_events(lambda: halo.xch.exchange(fused=True), it, wu))
+        breakdown["C2_halo_8ranks_fused"] = entry(halo.bytes // 2, halo.elems // 2,
+                                                  lambda: halo.xch.exchange(fused=True), inner=2)
         for d, name in enumerate(("dim0_W", "dim1_H", "dim2_D")):
             ov = [1 if k == d else 0 for k in range(5)]
             fn = lambda ov=ov: halo.xch.exchange(ov, ov, ov, ov, fused=True)
-            breakdown[f"C2_halo_{name}_fused"] = entry(halo.bytes // 6, halo.elems // 6,
-                                                       *_time_events(fn, it, wu))
+            breakdown[f"C2_halo_{name}_fused"] = entry(halo.bytes // 6, halo.elems // 6, fn)
+        # follow-on rows at the config 2 shape: clear_halo of all three dimensions on every rank
+        # (writes only), and the reverse exchange that adds halo contributions onto the interiors
+        from dihydrogen_amd.layers import HaloExchangeAccumOp
+
+        def clear_all():
+            for d in range(3):
+                halo.xch.clear_halo(d)
+
+        breakdown["C2_clear_halo_8ranks"] = entry(halo.bytes // 4, halo.elems // 2, clear_all, inner=2)
+        # pack: read + write; accumulating unpack: read buffer, read + write tensor -> 5/4 of the forward bytes
+        breakdown["C2_halo_reverse_sum_8ranks"] = entry(
+            halo.bytes * 5 // 4, halo.elems,
+            lambda: halo.xch.exchange(is_reverse=True, op=HaloExchangeAccumOp.SUM), inner=2)
         yard_x, yard_y = bn3.x.data, bn3.y.data
-        breakdown["yardstick_torch_copy_268MB"] = entry(
-            2 * S3 * 4, S3, *_time_events(lambda: yard_y.copy_(yard_x), it, wu))
+        breakdown["yardstick_torch_copy_268MB"] = entry(2 * S3 * 4, S3, lambda: yard_y.copy_(yard_x), eager=False)
         del bn3, halo, b, yard_x, yard_y
+        torch.cuda.empty_cache()
+        # strided batch-norm: the config 3 shard with a halo of 1 on all three spatial dimensions
+        bn3h = BatchNormWorkload((4, 64, 64, 64, 64), SEED + 6, overlap=1)
+        breakdown["C3_bn3d_haloed_fwd_bwd"] = entry(8 * bn3h.elems * 4, bn3h.elems,
+                                                    lambda: (bn3h.forward(), bn3h.backward()), inner=2)
+        del bn3h
         torch.cuda.empty_cache()
         # configs 1 and 4 fit in the memory-side cache: warm = back to back, cold = after a 512 MB read
         evict = torch.empty(1 << 27, device="cuda").fill_(1.0)
         flush = lambda: evict.sum()
         bn1 = BatchNormWorkload((8, 64, 56, 56), SEED + 1)
-        breakdown["C1_bn2d_fwd_warm"] = entry(3 * bn1.elems * 4, bn1.elems, *_time_events(bn1.forward, it, wu))
-        breakdown["C1_bn2d_fwd_cold"] = entry(3 * bn1.elems * 4, bn1.elems,
-                                              *_time_events_cold(bn1.forward, flush, it, wu))
+        breakdown["C1_bn2d_fwd"] = entry(3 * bn1.elems * 4, bn1.elems, bn1.forward)
+        med, mn = _time_events_cold(bn1.forward, flush, it, wu)
+        breakdown["C1_bn2d_fwd_cold"] = {
+            "bytes": 3 * bn1.elems * 4, "ms_median": med, "ms_min": mn, "GB/s": _gbs(3 * bn1.elems * 4, med),
+            "frac_of_peak": _gbs(3 * bn1.elems * 4, med) / HBM_PEAK_GBS,
+            "timing": "events around one eager call after a cache-evicting read (2 launches)"}
+        bn1.bn.fuse_local = False
+        breakdown["C1_bn2d_fwd_staged"] = entry(3 * bn1.elems * 4, bn1.elems, bn1.forward)
         del bn1
         sm = SoftmaxWorkload((16, 21, 256, 256), SEED + 4)
         sm.forward()
-        breakdown["C4_softmax_fwd"] = entry(2 * sm.elems * 4, sm.elems, *_time_events(sm.forward, it, wu))
-        breakdown["C4_softmax_bwd"] = entry(3 * sm.elems * 4, sm.elems, *_time_events(sm.backward, it, wu))
-        breakdown["C4_softmax_fwd_cold"] = entry(2 * sm.elems * 4, sm.elems,
-                                                 *_time_events_cold(sm.forward, flush, it, wu))
-        breakdown["C4_softmax_bwd_cold"] = entry(3 * sm.elems * 4, sm.elems,
-                                                 *_time_events_cold(sm.backward, flush, it, wu))
-        del sm, evict
+        breakdown["C4_softmax_fwd"] = entry(2 * sm.elems * 4, sm.elems, sm.forward)
+        breakdown["C4_softmax_bwd"] = entry(3 * sm.elems * 4, sm.elems, sm.backward)
+        for name, fn, nb in (("fwd", sm.forward, 2), ("bwd", sm.backward, 3)):
+            med, mn = _time_events_cold(fn, flush, it, wu)
+            breakdown[f"C4_softmax_{name}_cold"] = {
+                "bytes": nb * sm.elems * 4, "ms_median": med, "ms_min": mn, "GB/s": _gbs(nb * sm.elems * 4, med),
+                "frac_of_peak": _gbs(nb * sm.elems * 4, med) / HBM_PEAK_GBS,
+                "timing": "events around one eager call after a cache-evicting read"}
+        del sm
+        # instance-mode softmax at the same shape: forward reads x twice and y once and writes y twice
+        # (max, exp, normalise), backward reads y and dy twice and writes dx
+        smi = SoftmaxWorkload((16, 21, 256, 256), SEED + 4, instance=True)
+        smi.forward()
+        breakdown["C4_softmax_instance_fwd"] = entry(5 * smi.elems * 4, smi.elems, smi.forward)
+        breakdown["C4_softmax_instance_bwd"] = entry(5 * smi.elems * 4, smi.elems, smi.backward)
+        del smi, evict
+        torch.cuda.empty_cache()
         shf = ShuffleWorkload((128, 128, 64, 32), SEED + 5)
-        breakdown["C5_shuffle_fwd"] = entry(4 * shf.elems * 4, shf.elems, *_time_events(shf.forward, it, wu))
-        breakdown["C5_shuffle_bwd"] = entry(4 * shf.elems * 4, shf.elems, *_time_events(shf.backward, it, wu))
-
-        def round_trip():
-            shf.forward()
-            shf.backward()
-
+        breakdown["C5_shuffle_fwd"] = entry(4 * shf.elems * 4, shf.elems, shf.forward)
+        breakdown["C5_shuffle_bwd"] = entry(4 * shf.elems * 4, shf.elems, shf.backward)
         breakdown["C5_shuffle_round_trip"] = entry(8 * shf.elems * 4, 2 * shf.elems,
-                                                   *_time_events(round_trip, it, wu))
+                                                   lambda: (shf.forward(), shf.backward()), inner=2)
         del shf
+        torch.cuda.empty_cache()
+        # the same tensor between 16 ranks: 256 boxes a direction, one launch each for pack and unpack
+        shf16 = ShuffleWorkload((128, 128, 64, 32), SEED + 5, ranks=16, grid=(4, 4))
+        breakdown["C5_shuffle_16ranks_round_trip"] = entry(8 * shf16.elems * 4, 2 * shf16.elems,
+                                                           lambda: (shf16.forward(), shf16.backward()), inner=2)
+        del shf16
         torch.cuda.empty_cache()
 
     out = {
@@ -540,6 +734,7 @@ def main() -> int:
         },
         "frac_of_hbm_peak": value / HBM_PEAK_GBS,
         "elements_per_s": step_elems / (ms_per_step * 1e-3),
+        "kernel_sources": sources_sha,
         "roofline": roofline,
         "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline(),
         "launches": launches,

@@ -429,7 +429,9 @@ class HaloExchangeVirtual:
         was reallocated gets new tables."""
         return tuple(t.get_buffer() if t.data is not None else 0 for t in self.tensors)
 
-    def _recv_buffer(self, rank: int, dim: int, side: int) -> torch.Tensor:
+    def recv_buffer(self, rank: int, dim: int, side: int) -> torch.Tensor:
+        """The buffer rank `rank` unpacks its (dim, side) halo from -- and its
+        neighbour on that side packs into (get_recv_buffer, halo_exchange_cuda.hpp:277-283)."""
         key = (rank, dim, side)
         if key not in self._recv:
             t = self.tensors[rank]
@@ -437,7 +439,9 @@ class HaloExchangeVirtual:
             self._recv[key] = torch.zeros(max(n, 1), dtype=t.dtype, device=t.device)
         return self._recv[key]
 
-    def _face(self, rank, dim, side, width, buf, is_pack, is_reverse, op) -> capi.HaloFace:
+    def make_face(self, rank, dim, side, width, buf, is_pack, is_reverse, op) -> capi.HaloFace:
+        """One h2x_halo_face of rank `rank`: what pack_dim / unpack_dim pass down
+        (halo_exchange_cuda.hpp:365-393)."""
         t = self.tensors[rank]
         f = capi.HaloFace()
         f.tensor = t.get_buffer()
@@ -483,11 +487,11 @@ class HaloExchangeVirtual:
                         w_send = width_rhs_send if side == capi.RHS else width_lhs_send
                         w_recv = width_rhs_recv if side == capi.RHS else width_lhs_recv
                         if w_send > 0:
-                            dst = self._recv_buffer(peer, dim, capi.LHS if side == capi.RHS else capi.RHS)
-                            packs.append(self._face(r, dim, side, w_send, dst, True, is_reverse, op))
+                            dst = self.recv_buffer(peer, dim, capi.LHS if side == capi.RHS else capi.RHS)
+                            packs.append(self.make_face(r, dim, side, w_send, dst, True, is_reverse, op))
                         if w_recv > 0 and not skip_unpack:
-                            src = self._recv_buffer(r, dim, side)
-                            unpacks.append(self._face(r, dim, side, w_recv, src, False, is_reverse, op))
+                            src = self.recv_buffer(r, dim, side)
+                            unpacks.append(self.make_face(r, dim, side, w_recv, src, False, is_reverse, op))
                 # the face tables depend only on the arguments and on the tensors'
                 # addresses (part of the key): build them once
                 cached.append(tuple((capi.HaloFace * len(f))(*f) if f else None for f in (packs, unpacks)))

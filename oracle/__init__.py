@@ -360,3 +360,17 @@ def tensor_reduce_sum(src: np.ndarray, dst: np.ndarray, square: bool = False) ->
         x = x * x
     total = x.sum(axis=axes, keepdims=True) if axes else x
     dst[...] = dst + total.astype(dst.dtype)
+
+
+def shuffle_rows(tensor: np.ndarray, local_shape, strides, peer_locale_shape, rank_limits,
+                 buf: np.ndarray, displs, is_pack: bool) -> None:
+    """Row-copy pack / unpack of any rank (the reference's OpenMP memcpy paths,
+    legacy/include/distconv/tensor/shuffle_mpi.hpp:708-849,874-947); plain
+    rank limits only; requires strides[0] == 1."""
+    nd = len(local_shape)
+    assert strides[0] == 1
+    rl, rlp = _i32arr(rank_limits)
+    dp, dpp = _i32arr(displs)
+    lib().orc_shuffle_rows(
+        _ptr(tensor), ctypes.c_int(nd), ctypes.c_int(tensor.dtype.itemsize), _i64(local_shape),
+        _i64(strides), _i64(peer_locale_shape), rlp, _ptr(buf), dpp, ctypes.c_int(int(is_pack)))

@@ -217,3 +217,81 @@ void orc_shuffle_pack_rows4(const void* tensor, int elem_size, const int64_t* lo
         }
     }
 }
+
+/*
+ * Row-copy pack (is_pack = 1) or unpack (0) for tensors of any rank up to
+ * ORC_MAX_DIMS: the structure shared by the reference's CPU fast paths
+ * pack_sample_to_spatial4 / 5 (legacy/include/distconv/tensor/shuffle_mpi.hpp:708-849),
+ * unpack_sample_to_spatial (:874-879, one memcpy when nothing is cut) and
+ * unpack_sample_to_spatial_halo4 / 5 (:881-947): OpenMP over all outer
+ * indices, every innermost row cut at the peer grid's limits along dimension
+ * 0 and each piece moved with memcpy; the tensor side is addressed through
+ * `strides`, so a haloed destination works as in the _halo variants.  (The
+ * reference's _halo5 declares its stride array with four entries and indexes
+ * it with five, :919-941; the evident five-dimensional loop is restated.)
+ * Cuts follow rank_limits, so uneven splits equal orc_shuffle_pack_or_unpack
+ * on the same tables (checked in the tests).
+ */
+void orc_shuffle_rows(void* tensor, int nd, int elem_size, const int64_t* local_shape,
+                      const int64_t* strides, const int64_t* peer_locale_shape,
+                      const int32_t* rank_limits, void* buf, const int32_t* displs, int is_pack)
+{
+    size_t outer = 1;
+    for (int i = 1; i < nd; ++i)
+        outer *= (size_t) local_shape[i];
+    if (outer == 0 || local_shape[0] == 0)
+        return;
+    const int32_t* lim[ORC_MAX_DIMS];
+    int rl = 0;
+    for (int i = 0; i < nd; ++i)
+    {
+        lim[i] = rank_limits + rl;
+        rl += (int) peer_locale_shape[i];
+    }
+    char* tp = (char*) tensor;
+    char* bp = (char*) buf;
+#pragma omp parallel for schedule(static)
+    for (long long o = 0; o < (long long) outer; ++o)
+    {
+        /* outer index -> (i1 .. i_{nd-1}); peer slab and offset inside it per dimension */
+        size_t rem = (size_t) o, toff = 0;
+        int64_t rank_outer = 0, rank_stride = peer_locale_shape[0];
+        int64_t in_slab[ORC_MAX_DIMS], slab_extent[ORC_MAX_DIMS];
+        for (int i = 1; i < nd; ++i)
+        {
+            const int64_t idx = (int64_t) (rem % (size_t) local_shape[i]);
+            rem /= (size_t) local_shape[i];
+            toff += (size_t) idx * (size_t) strides[i];
+            int j = 0;
+            while (idx >= lim[i][j])
+                ++j;
+            const int64_t base = j ? lim[i][j - 1] : 0;
+            in_slab[i] = idx - base;
+            slab_extent[i] = lim[i][j] - base;
+            rank_outer += j * rank_stride;
+            rank_stride *= peer_locale_shape[i];
+        }
+        int64_t w0 = 0;
+        for (int jw = 0; jw < (int) peer_locale_shape[0]; ++jw)
+        {
+            const int64_t ew = lim[0][jw] - w0;
+            if (ew > 0)
+            {
+                /* natural order of the intersection box: dimension 0 fastest */
+                size_t poff = 0, lin = (size_t) ew;
+                for (int i = 1; i < nd; ++i)
+                {
+                    poff += (size_t) in_slab[i] * lin;
+                    lin *= (size_t) slab_extent[i];
+                }
+                char* t = tp + (toff + (size_t) w0 * (size_t) strides[0]) * (size_t) elem_size;
+                char* b = bp + ((size_t) displs[jw + rank_outer] + poff) * (size_t) elem_size;
+                if (is_pack)
+                    memcpy(b, t, (size_t) ew * (size_t) elem_size);
+                else
+                    memcpy(t, b, (size_t) ew * (size_t) elem_size);
+            }
+            w0 = lim[0][jw];
+        }
+    }
+}

@@ -149,3 +149,44 @@ def test_row_copy_pack_equals_generic_pack():
             c = np.zeros(s.local_size, np.float32)
             oracle.shuffle_pack_or_unpack(field, s.local_shape, s.strides(), dst_g[r].dist.locale_shape, lim, c, sd, True, parallel=True)
             assert np.array_equal(a, c)
+
+
+def test_row_copy_of_any_rank_equals_the_generic_path():
+    """orc_shuffle_rows (the structure of pack_sample_to_spatial4/5 and
+    unpack_sample_to_spatial[_halo4/5], shuffle_mpi.hpp:708-849,874-947) against
+    the per-element pack / unpack on the same tables: 4-D and 5-D, uneven splits,
+    and a haloed destination for the unpack (rows land inside the halo frame,
+    the frame itself is not touched)."""
+    cases = [
+        ((8, 8, 2, 4), (1, 1, 1, 4), (2, 2, 1, 1), None),
+        ((11, 7, 3, 5), (1, 1, 1, 4), (2, 2, 1, 1), None),
+        ((8, 8, 2, 4), (1, 1, 1, 4), (2, 2, 1, 1), (1, 1, 0, 0)),
+        ((6, 8, 4, 2, 4), (1, 1, 1, 1, 4), (1, 2, 2, 1, 1), (0, 1, 1, 0, 0)),
+        ((7, 5, 6, 3, 8), (1, 1, 1, 1, 8), (2, 2, 2, 1, 1), None),
+    ]
+    for shape, sl, dl, halo in cases:
+        nd, n = len(shape), int(np.prod(sl))
+        src_g = [G.TensorGeom(shape, G.Dist(sl, sl, [0] * nd), r) for r in range(n)]
+        dst_g = [G.TensorGeom(shape, G.Dist(dl, dl, list(halo) if halo else [0] * nd), r) for r in range(n)]
+        for r in range(n):
+            s, d = src_g[r], dst_g[r]
+            rng = np.random.default_rng(100 + r)
+            # pack on the source side
+            field = rng.standard_normal(s.real_size).astype(np.float32)
+            lim = G.rank_limits(s, d)
+            _, sd, _, rd = G.counts_and_displs(s, d)
+            a, b = np.zeros(s.local_size, np.float32), np.zeros(s.local_size, np.float32)
+            base = s.base_offset()
+            oracle.shuffle_pack_or_unpack(field[base:], s.local_shape, s.strides(), d.dist.locale_shape, lim, a, sd, True)
+            oracle.shuffle_rows(field[base:], s.local_shape, s.strides(), d.dist.locale_shape, lim, b, sd, True)
+            assert np.array_equal(a, b)
+            # unpack on the destination side (haloed or not)
+            lim_d = G.rank_limits(d, s)
+            buf = rng.standard_normal(d.local_size).astype(np.float32)
+            t1 = np.full(d.real_size, -5.0, np.float32)
+            t2 = t1.copy()
+            base = d.base_offset()
+            oracle.shuffle_pack_or_unpack(t1[base:], d.local_shape, d.strides(), s.dist.locale_shape, lim_d, buf, rd, False)
+            oracle.shuffle_rows(t2[base:], d.local_shape, d.strides(), s.dist.locale_shape, lim_d, buf, rd, False)
+            assert np.array_equal(t1, t2)
+            assert (t2 == -5.0).sum() == d.real_size - d.local_size   # only the interior was written
