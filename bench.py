@@ -405,6 +405,8 @@ def dim0_study():
     share one), every unpacked row seam an 8-byte partial write.  Timed for
     launch groups of 2, 4 and 8 ranks, pack and unpack alone and together, and
     for the tensor-to-tensor form."""
+    import ctypes
+    import torch
     from dihydrogen_amd import capi
     from dihydrogen_amd.layers import HaloExchangeAccumOp
     lib = capi.load()
@@ -426,7 +428,9 @@ def dim0_study():
         return (capi.HaloFace * len(out))(*out)
 
     def launch(arr):
-        capi.check(lib.h2x_halo_pack_or_unpack_batched(dt, arr, len(arr), None), "halo")
+        # on torch's current stream (the capture stream while a graph is recorded)
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        capi.check(lib.h2x_halo_pack_or_unpack_batched(dt, arr, len(arr), stream), "halo")
 
     result = {"rows_per_rank": rows, "lines_per_rank": int(lines_per_rank), "seam_writes_per_rank": seams_per_rank,
               "groups": {}}
@@ -449,6 +453,35 @@ def dim0_study():
     return result
 
 
+def halo_sweep():
+    """How the rate of a dense halo phase grows with the bytes one launch moves:
+    the dimension-1 and dimension-2 phases (one pack launch + one unpack launch,
+    16 faces each) of the config 2 grid at 2 ... 128 channels, and beside each
+    two plain device-to-device copies of the same bytes.  A phase that tracks
+    the copies is bound by how fast a launch of that size fills and drains the
+    chip, not by its access pattern."""
+    import torch
+    rows = []
+    for channels in (2, 4, 8, 16, 32, 64, 128):
+        halo = HaloWorkload(128, channels, SEED + 2)
+        launch_bytes = halo.bytes // 6  # one launch: 16 faces read and written
+        n = launch_bytes // 8           # floats one plain copy moves (read + write = launch_bytes)
+        a = torch.empty(2, n, device="cuda").normal_()
+        b = torch.empty(2, n, device="cuda")
+        row = {"channels": channels, "bytes_per_launch": launch_bytes}
+        t = _time_graph(lambda: (b[0].copy_(a[0]), b[1].copy_(a[1])), 20, 5)[0]
+        row["copy_pair_us"], row["copy_pair_GB/s"] = t * 1e3, _gbs(2 * launch_bytes, t)
+        for d, name in ((1, "dim1"), (2, "dim2")):
+            ov = [1 if k == d else 0 for k in range(5)]
+            t = _time_graph(lambda ov=ov: halo.xch.exchange(ov, ov, ov, ov), 20, 5)[0]
+            row[f"{name}_us"], row[f"{name}_GB/s"] = t * 1e3, _gbs(2 * launch_bytes, t)
+            row[f"{name}_vs_copy"] = row["copy_pair_us"] / (t * 1e3)
+        rows.append(row)
+        del halo, a, b
+        torch.cuda.empty_cache()
+    return {"peak_GB/s": HBM_PEAK_GBS, "rows": rows}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -459,6 +492,9 @@ def main() -> int:
     ap.add_argument("--dim0-study", action="store_true",
                     help="instead of the benchmark: the innermost-dimension halo phase alone, by number of "
                          "ranks per launch group, as cache lines and seam writes per second")
+    ap.add_argument("--halo-sweep", action="store_true",
+                    help="instead of the benchmark: the dimension-1 and -2 halo phases of the config 2 grid for "
+                         "growing channel counts, beside plain copies of the same bytes per launch")
     ap.add_argument("--sources-sha", action="store_true", help="print the hash of the kernel sources and exit")
     args = ap.parse_args()
     if args.sources_sha:
@@ -479,6 +515,10 @@ def main() -> int:
 
     if args.dim0_study:
         print(json.dumps(dim0_study()))
+        return 0
+
+    if args.halo_sweep:
+        print(json.dumps(halo_sweep()))
         return 0
 
     bn3 = BatchNormWorkload((4, 64, 64, 64, 64), SEED + 3)
@@ -532,19 +572,21 @@ def main() -> int:
         timed("bn_backprop2", bn3.backward_apply)
         halo.run()
 
-    def kernel_share(evs, steps):
+    def kernel_share(evs):
+        """Milliseconds per step by kernel: median launch time x launches per step."""
         tot = {}
         for label, pairs in evs.items():
-            ms = sum(e0.elapsed_time(e1) for e0, e1 in pairs) / steps  # per step, all launches
+            per_step = 16 // faces_per_launch[label] if label in faces_per_launch else 1
+            ms = statistics.median(e0.elapsed_time(e1) for e0, e1 in pairs) * per_step
             tot[KERNEL_OF[label]] = tot.get(KERNEL_OF[label], 0.0) + ms
         return tot
 
     # warm-up, with every launch bracketed by events: finds the dominant kernel
     recording[0] = True
-    for _ in range(max(args.warmup, 1)):
+    for _ in range(max(args.warmup, 3)):
         step_staged()
     torch.cuda.synchronize()
-    share0 = kernel_share(events, max(args.warmup, 1))
+    share0 = kernel_share(events)
     dominant = max(share0, key=share0.get)
     events.clear()
     step()  # the fused entry points once, untimed (first-use allocations)

@@ -26,6 +26,7 @@
 #include "h2x_copy_kernel.hpp"
 
 #include <algorithm>
+#include <cstdlib>
 #include <cstring>
 #include <new>
 #include <vector>
@@ -220,6 +221,33 @@ bool box_is_sparse(const HostBox& h, int elem_size)
                     : (h.stride[0] != 1 && h.extent[0] > 1);
 }
 
+// Two boxes of identical geometry whose origins are `delta` elements apart
+// share no element if, with every stride a multiple of the row pitch, the
+// shift within a row is at least one run and at most a pitch less one run.
+// (A sufficient test: false means "not known to be disjoint".)
+bool translated_boxes_are_disjoint(const HostBox& h, int64_t delta)
+{
+    int64_t run = 1, pitch = 0;
+    int first = 0;
+    if (h.stride[0] == 1)
+    {
+        run = h.extent[0];
+        first = 1;
+    }
+    for (int i = first; i < h.nd; ++i)
+        if (h.extent[i] > 1)
+            pitch = pitch == 0 ? std::llabs(h.stride[i]) : std::min<int64_t>(pitch, std::llabs(h.stride[i]));
+    if (delta < 0)
+        delta = -delta;
+    if (pitch == 0) // a single run
+        return delta >= run;
+    for (int i = first; i < h.nd; ++i)
+        if (h.extent[i] > 1 && h.stride[i] % pitch != 0)
+            return false;
+    const int64_t shift = delta % pitch;
+    return shift >= run && shift <= pitch - run;
+}
+
 bool same_geometry(const HostBox& a, const HostBox& b)
 {
     if (a.nd != b.nd || a.count != b.count)
@@ -245,7 +273,7 @@ void fill_box(Box* b, const HostBox& h)
     b->ragged = 0;
     b->seam = 0;
     b->deep = h.nd > 3;
-    b->reserved = 0;
+    b->disjoint = 0;
     b->tensor2 = nullptr;
     b->buffer2 = nullptr;
 }
@@ -336,6 +364,7 @@ struct Launcher
             // (the RHS and the LHS halo cell at a row seam): unpacked in one store
             first.seam = box_mode == kUnpack && v == 1 && h.nd == 1
                          && tptr + elem_size == first.tensor + h.stride[0] * elem_size;
+            first.disjoint = translated_boxes_are_disjoint(h, (tptr - first.tensor) / elem_size);
             return H2X_SUCCESS;
         }
         if (batch.num_boxes == kMaxBoxes

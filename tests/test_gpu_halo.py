@@ -117,6 +117,43 @@ def test_both_faces_of_the_innermost_dimension_in_one_call(op, dtype, oracle_mod
             assert np.array_equal(bd[side].cpu().numpy(), b_o[side])
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("op", [1, 2, 3])
+@pytest.mark.parametrize("real_np,width", [((2, 3, 7, 9), 1), ((2, 3, 7, 3), 1), ((2, 2, 5, 6), 2),
+                                           ((2, 2, 5, 7), 2), ((1, 2, 3, 130), 1)])
+def test_reverse_accumulation_of_both_faces_in_one_call(real_np, width, op, dtype, oracle_mod):
+    """Reverse unpack (halo contributions folded into the interior strips) of
+    the LHS and RHS face of dimension 0 by one batched call.  With an interior
+    as narrow as the strip the two strips are the same cells, with one cell
+    more they overlap in part: every cell must then receive both contributions,
+    as the oracle's two unpacks one after the other give them."""
+    import torch
+    from dihydrogen_amd import capi
+    lib = capi.load()
+    shape = real_np[::-1]
+    rng = np.random.default_rng(29 + op + width)
+    t = rng.uniform(-1, 1, real_np).astype(dtype)
+    n = oracle_mod.halo_size(shape, 0, width)
+    bufs = [rng.uniform(-1, 1, n).astype(dtype) for _ in range(2)]
+    h2x_dt = capi.F32 if dtype == np.float32 else capi.F64
+    t_o = t.copy()
+    for side in (0, 1):
+        oracle_mod.halo_pack_or_unpack(t_o, 0, side, width, bufs[side], False, True, op)
+    td = torch.from_numpy(t).cuda()
+    bd = [torch.from_numpy(b).cuda() for b in bufs]
+    faces = (capi.HaloFace * 2)()
+    for side in (0, 1):
+        f = faces[side]
+        f.tensor, f.buffer = td.data_ptr(), bd[side].data_ptr()
+        for i, e in enumerate(shape):
+            f.real_shape[i] = e
+        f.num_dims, f.dim, f.side, f.width = len(shape), 0, side, width
+        f.inner, f.is_pack, f.op = 1, 0, op
+    capi.check(lib.h2x_halo_pack_or_unpack_batched(h2x_dt, faces, 2, None))
+    torch.cuda.synchronize()
+    assert np.array_equal(td.cpu().numpy(), t_o)
+
+
 def _exchange_case(shape, locale, overlap, periodic, oracle_mod, widths=None, dtype=np.float32,
                    fused=False):
     """Runs the exchange on the GPU and on the CPU oracle; returns both."""
