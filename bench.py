@@ -361,15 +361,27 @@ def cpu_baseline(repeats: int = 5):
     }
 
 
-# HBM-side traffic per launch measured with rocprofv3 --pmc (profiles/bench_pmc_traffic.txt):
-# request counters between the L2 and the fabric, converted to bytes there
-# (TCC_EA0_RDREQ, TCC_EA0_RDREQ_32B, TCC_BUBBLE; TCC_EA0_WRREQ, TCC_EA0_WRREQ_64B).
+# Traffic between the L2 and the memory fabric per launch, measured with rocprofv3 --pmc
+# (profiles/bench_pmc_traffic.txt): read bytes = 128 x TCC_EA0_RDREQ_128B + 64 x TCC_EA0_RDREQ_64B
+# + 32 x TCC_EA0_RDREQ_32B, written bytes = 64 x TCC_EA0_WRREQ_64B + 32 x (TCC_EA0_WRREQ -
+# TCC_EA0_WRREQ_64B), request counts summed over the L2 channels, per dispatch.
 # label -> (bytes read, bytes written) per launch
-PMC_TRAFFIC = {}
-# sha256 of the kernel sources the table was measured with (see kernel_sources_sha()); with other
-# sources the traffic fields are omitted
-PMC_SOURCES_SHA = ""
-PMC_COMMIT = ""
+PMC_TRAFFIC = {
+    "bn_sums": (268459008, 131072),
+    "bn_apply": (268465664, 268480640),
+    "bn_backprop1": (536912384, 131104),
+    "bn_backprop2": (536905728, 268435456),
+    "halo_dim0_pack": (149722656, 8652800),    # 4 faces (2 ranks) a launch, four launches a step
+    "halo_dim0_unpack": (9217808, 43264000),
+    "halo_dim1_pack": (42624768, 34611200),
+    "halo_dim1_unpack": (34637568, 36216480),
+    "halo_dim2_pack": (34694400, 34611200),
+    "halo_dim2_unpack": (34637568, 34619456),
+}
+# sha256 (first 16 hex digits) of the kernel sources the table was measured with, see
+# kernel_sources_sha(); with other sources the traffic fields are omitted
+PMC_SOURCES_SHA = "b1c21b63828c3eb0"
+PMC_COMMIT = "c41ee01"
 
 KERNEL_OF = {
     "bn_sums": "bn_sums_kernel<float,4> (+bn_finish_kernel<float,2>)",
