@@ -249,10 +249,11 @@ def cpu_baseline(repeats: int = 5):
     rng = np.random.default_rng(SEED)
 
     def med(fn):
-        """Median of at least `repeats` runs and at least a second of them."""
+        """Median of at least `repeats` runs and at least two seconds of them
+        (about 15 s of CPU work over all configs)."""
         fn()
         ts = []
-        while len(ts) < repeats or (sum(ts) < 1.0 and len(ts) < 200):
+        while len(ts) < repeats or (sum(ts) < 2.0 and len(ts) < 2000):
             t0 = time.perf_counter()
             fn()
             ts.append(time.perf_counter() - t0)
@@ -354,8 +355,9 @@ def cpu_baseline(repeats: int = 5):
         "cores": threads,
         "kind": "port",
         "cpu_model": _cpu_model(),
+        "logical_cpus": os.cpu_count(),
         "sample": (f"config 3 batch-norm fwd+bwd in full + config 2 exchange of {halo_ranks} of 8 ranks; "
-                   f"medians of {repeats} runs ({t3:.3f} s + {t2:.3f} s); gcc -O3 -fopenmp, "
+                   f"medians of at least {repeats} runs and 2 s each ({t3:.3f} s + {t2:.3f} s a run); gcc -O3 -fopenmp, "
                    f"OMP threads = {threads}"),
         "configs": configs,
     }
