@@ -712,6 +712,15 @@ def main() -> int:
         breakdown["C2_halo_reverse_sum_8ranks"] = entry(
             halo.bytes * 5 // 4, halo.elems,
             lambda: halo.xch.exchange(is_reverse=True, op=HaloExchangeAccumOp.SUM), inner=2)
+        # tensor::Transform / ReduceSum at the config 3 shape: scale in place (read + write), copy into a
+        # second tensor (read + write), per-channel sums and sums of squares (one read each)
+        from dihydrogen_amd import layers as L
+        from dihydrogen_amd.tensor import Distribution as _D, LocaleVirtual as _LV, Tensor as _T
+        breakdown["C3_transform_scale"] = entry(2 * S3 * 4, S3, lambda: L.transform(capi.TRANSFORM_SCALE, [bn3.y], [1.0]))
+        breakdown["C3_transform_copy"] = entry(2 * S3 * 4, S3, lambda: L.transform(capi.TRANSFORM_COPY, [bn3.x, bn3.y]))
+        stat = _T([1, 1, 1, 64, 1], _LV(0, 1), _D.make_localized_distribution(5)).allocate()
+        breakdown["C3_reduce_sum_per_channel"] = entry(S3 * 4, S3, lambda: L.reduce_sum(bn3.x, stat))
+        breakdown["C3_reduce_sqsum_per_channel"] = entry(S3 * 4, S3, lambda: L.reduce_sum(bn3.x, stat, square=True))
         yard_x, yard_y = bn3.x.data, bn3.y.data
         breakdown["yardstick_torch_copy_268MB"] = entry(2 * S3 * 4, S3, lambda: yard_y.copy_(yard_x), eager=False)
         del bn3, halo, b, yard_x, yard_y

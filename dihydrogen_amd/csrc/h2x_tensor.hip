@@ -63,14 +63,59 @@ __device__ __forceinline__ void sums_to_statistics(T& mean, T& var, T& rmean, T&
     rvar = fma_t(decay, rvar, (T(1) - decay) * v);
 }
 
+// One element of one operation; pointers to the element in each tensor.
 template <typename T, int OP>
+__device__ __forceinline__ void transform_element(T* const (&v)[4], const double (&p)[4])
+{
+    if constexpr (OP == H2X_TRANSFORM_SCALE)
+    {
+        *v[0] = *v[0] * static_cast<T>(p[0]); // internal::ScaleFunctor, tensor_mpi_cuda.cu:86-92
+    }
+    else if constexpr (OP == H2X_TRANSFORM_COPY)
+    {
+        *v[1] = *v[0];
+    }
+    else if constexpr (OP == H2X_TRANSFORM_SCALE_BIAS)
+    {
+        // CastScaleBiasFuctor with equal types: dst = alpha * src + beta (tensor_mpi_cuda.cu:113-128)
+        *v[1] = static_cast<T>(p[0]) * *v[0] + static_cast<T>(p[1]);
+    }
+    else
+    {
+        T m = *v[0], var = *v[1], rm = *v[2], rv = *v[3];
+        if (p[0] == 0.0) // nothing was counted: batchnorm.cu:337-345
+        {
+            *v[1] = T(1);
+        }
+        else
+        {
+            sums_to_statistics(m, var, rm, rv, static_cast<T>(p[0]), static_cast<T>(p[1]));
+            *v[0] = m;
+            *v[1] = var;
+            *v[2] = rm;
+            *v[3] = rv;
+        }
+    }
+}
+
+// A thread owns VEC neighbouring elements of the innermost merged dimension
+// (VEC > 1: that dimension is contiguous in every tensor and a multiple of VEC
+// long, so a vector never leaves its row; rows of haloed tensors start on any
+// element, hence vector types aligned to one element).  Tensors that are only
+// read come in as one vector load, tensors that are written leave as one vector
+// store; a tensor that is only written (the destination of a copy or of
+// scale + bias) is stored past the caches.
+template <typename T, int OP, int VEC>
 __global__ __launch_bounds__(kBlockSize) void transform_kernel(const TransformArgs a)
 {
     constexpr int N = OP == H2X_TRANSFORM_SCALE ? 1 : OP == H2X_TRANSFORM_SUMS_TO_STATISTICS ? 4 : 2;
-    for (uint64_t i = blockIdx.x * static_cast<uint64_t>(kBlockSize) + threadIdx.x; i < a.count;
+    constexpr bool kStreamOut = OP == H2X_TRANSFORM_COPY || OP == H2X_TRANSFORM_SCALE_BIAS;
+    typedef T Vec __attribute__((ext_vector_type(VEC), aligned(sizeof(T))));
+    const uint64_t vectors = a.count / VEC;
+    for (uint64_t i = blockIdx.x * static_cast<uint64_t>(kBlockSize) + threadIdx.x; i < vectors;
          i += static_cast<uint64_t>(gridDim.x) * kBlockSize)
     {
-        uint32_t rem = static_cast<uint32_t>(i);
+        uint32_t rem = static_cast<uint32_t>(i * VEC);
         int64_t off[N];
 #pragma unroll
         for (int t = 0; t < N; ++t)
@@ -92,37 +137,48 @@ __global__ __launch_bounds__(kBlockSize) void transform_kernel(const TransformAr
                     off[t] += static_cast<int64_t>(idx) * a.stride[t][d];
             }
         }
-        T* p[N];
+        if constexpr (VEC == 1)
+        {
+            T* v[4] = {nullptr, nullptr, nullptr, nullptr};
 #pragma unroll
-        for (int t = 0; t < N; ++t)
-            p[t] = reinterpret_cast<T*>(a.base[t]) + off[t];
-        if constexpr (OP == H2X_TRANSFORM_SCALE)
-        {
-            *p[0] = *p[0] * static_cast<T>(a.p[0]); // internal::ScaleFunctor, tensor_mpi_cuda.cu:86-92
-        }
-        else if constexpr (OP == H2X_TRANSFORM_COPY)
-        {
-            *p[1] = *p[0];
-        }
-        else if constexpr (OP == H2X_TRANSFORM_SCALE_BIAS)
-        {
-            // CastScaleBiasFuctor with equal types: dst = alpha * src + beta (tensor_mpi_cuda.cu:113-128)
-            *p[1] = static_cast<T>(a.p[0]) * *p[0] + static_cast<T>(a.p[1]);
+            for (int t = 0; t < N; ++t)
+                v[t] = reinterpret_cast<T*>(a.base[t]) + off[t];
+            transform_element<T, OP>(v, a.p);
         }
         else
         {
-            T m = *p[0], v = *p[1], rm = *p[2], rv = *p[3];
-            if (a.p[0] == 0.0) // nothing was counted: batchnorm.cu:337-345
+            Vec reg[N];
+#pragma unroll
+            for (int t = 0; t < N; ++t)
+                if (!(kStreamOut && t == 1))
+                    reg[t] = *reinterpret_cast<const Vec*>(reinterpret_cast<const T*>(a.base[t]) + off[t]);
+            T lane[4][VEC];
+#pragma unroll
+            for (int j = 0; j < VEC; ++j)
             {
-                *p[1] = T(1);
+                T* v[4] = {nullptr, nullptr, nullptr, nullptr};
+#pragma unroll
+                for (int t = 0; t < N; ++t)
+                {
+                    lane[t][j] = (kStreamOut && t == 1) ? T(0) : reg[t][j];
+                    v[t] = &lane[t][j];
+                }
+                transform_element<T, OP>(v, a.p);
             }
-            else
+#pragma unroll
+            for (int t = 0; t < N; ++t)
             {
-                sums_to_statistics(m, v, rm, rv, static_cast<T>(a.p[0]), static_cast<T>(a.p[1]));
-                *p[0] = m;
-                *p[1] = v;
-                *p[2] = rm;
-                *p[3] = rv;
+                if (OP != H2X_TRANSFORM_SCALE && OP != H2X_TRANSFORM_SUMS_TO_STATISTICS && t == 0)
+                    continue; // the source of a copy is not written
+                Vec out;
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+                    out[j] = lane[t][j];
+                Vec* const dst = reinterpret_cast<Vec*>(reinterpret_cast<T*>(a.base[t]) + off[t]);
+                if constexpr (kStreamOut)
+                    __builtin_nontemporal_store(out, dst);
+                else
+                    *dst = out;
             }
         }
     }
@@ -173,10 +229,14 @@ __device__ __forceinline__ int64_t chain(uint32_t i, int nd, const FastDiv* div,
 }
 
 // The innermost dimension is reduced: a workgroup adds one group of one output
-// element's addends; neighbouring threads read neighbouring addends.
-template <typename T>
+// element's addends; neighbouring threads read neighbouring addends, VEC at a
+// time (VEC > 1: the innermost reduced dimension is contiguous and a multiple of
+// VEC long, and so is the group size), four loads in flight per thread.
+template <typename T, int VEC>
 __global__ __launch_bounds__(kBlockSize) void reduce_inner_kernel(const ReduceArgs a)
 {
+    typedef T Vec __attribute__((ext_vector_type(VEC), aligned(sizeof(T))));
+    constexpr int kInFlight = 4;
     __shared__ double lds[kWavesPerBlock];
     const uint32_t k = blockIdx.x, g = blockIdx.y;
     const T* src = reinterpret_cast<const T*>(a.src)
@@ -184,11 +244,32 @@ __global__ __launch_bounds__(kBlockSize) void reduce_inner_kernel(const ReduceAr
     const uint32_t begin = g * a.chunk;
     const uint32_t end = begin + a.chunk < a.red_count ? begin + a.chunk : a.red_count;
     double acc[1] = {0.0};
-    for (uint32_t r = begin + threadIdx.x; r < end; r += kBlockSize)
-    {
-        const double x = static_cast<double>(
-            src[chain(r, a.num_reduced, a.red_div, a.red_src, nullptr, nullptr)]);
+    auto add = [&](T v) {
+        const double x = static_cast<double>(v);
         acc[0] += a.square ? x * x : x;
+    };
+    constexpr uint32_t kStep = kBlockSize * VEC;
+    uint32_t r = begin + threadIdx.x * VEC;
+    for (; r + (kInFlight - 1) * kStep < end; r += kInFlight * kStep)
+    {
+        Vec v[kInFlight];
+#pragma unroll
+        for (int u = 0; u < kInFlight; ++u)
+            v[u] = *reinterpret_cast<const Vec*>(
+                src + chain(r + u * kStep, a.num_reduced, a.red_div, a.red_src, nullptr, nullptr));
+#pragma unroll
+        for (int u = 0; u < kInFlight; ++u)
+#pragma unroll
+            for (int j = 0; j < VEC; ++j)
+                add(v[u][j]);
+    }
+    for (; r < end; r += kStep)
+    {
+        const Vec v = *reinterpret_cast<const Vec*>(
+            src + chain(r, a.num_reduced, a.red_div, a.red_src, nullptr, nullptr));
+#pragma unroll
+        for (int j = 0; j < VEC; ++j)
+            add(v[j]);
     }
     block_sum<1>(acc, lds);
     if (threadIdx.x == 0)
@@ -246,28 +327,41 @@ int check_geometry(const h2x_tensor_geometry* g)
     return H2X_SUCCESS;
 }
 
-template <typename T>
-int transform_typed(int op, const TransformArgs& a, hipStream_t stream)
+template <typename T, int VEC>
+int transform_vec(int op, const TransformArgs& a, hipStream_t stream)
 {
+    const uint64_t vectors = a.count / VEC;
     const unsigned int blocks =
-        static_cast<unsigned int>(std::min<uint64_t>((a.count + kBlockSize - 1) / kBlockSize, 65536));
+        static_cast<unsigned int>(std::min<uint64_t>((vectors + kBlockSize - 1) / kBlockSize, 1u << 20));
     switch (op)
     {
     case H2X_TRANSFORM_SCALE:
-        transform_kernel<T, H2X_TRANSFORM_SCALE><<<blocks, kBlockSize, 0, stream>>>(a);
+        transform_kernel<T, H2X_TRANSFORM_SCALE, VEC><<<blocks, kBlockSize, 0, stream>>>(a);
         break;
     case H2X_TRANSFORM_COPY:
-        transform_kernel<T, H2X_TRANSFORM_COPY><<<blocks, kBlockSize, 0, stream>>>(a);
+        transform_kernel<T, H2X_TRANSFORM_COPY, VEC><<<blocks, kBlockSize, 0, stream>>>(a);
         break;
     case H2X_TRANSFORM_SCALE_BIAS:
-        transform_kernel<T, H2X_TRANSFORM_SCALE_BIAS><<<blocks, kBlockSize, 0, stream>>>(a);
+        transform_kernel<T, H2X_TRANSFORM_SCALE_BIAS, VEC><<<blocks, kBlockSize, 0, stream>>>(a);
         break;
     case H2X_TRANSFORM_SUMS_TO_STATISTICS:
-        transform_kernel<T, H2X_TRANSFORM_SUMS_TO_STATISTICS><<<blocks, kBlockSize, 0, stream>>>(a);
+        transform_kernel<T, H2X_TRANSFORM_SUMS_TO_STATISTICS, VEC><<<blocks, kBlockSize, 0, stream>>>(a);
         break;
     default: return H2X_ERR_UNSUPPORTED;
     }
     return launch_status();
+}
+
+// 16-byte vectors when the innermost merged dimension is contiguous in every
+// tensor and a multiple of the vector long; element by element otherwise.
+template <typename T>
+int transform_typed(int op, int num_tensors, const TransformArgs& a, hipStream_t stream)
+{
+    constexpr int kVec = 16 / sizeof(T);
+    bool vec = a.div[0].divisor % kVec == 0;
+    for (int t = 0; t < num_tensors; ++t)
+        vec = vec && a.stride[t][0] == 1;
+    return vec ? transform_vec<T, kVec>(op, a, stream) : transform_vec<T, 1>(op, a, stream);
 }
 
 // How a sum is cut up.  Shared by the entry point and the workspace query.
@@ -275,10 +369,12 @@ struct ReducePlan
 {
     ReduceArgs args;
     bool inner = false; // the innermost dimension with more than one element is reduced
+    int vec = 1;        // elements per load of the inner reduction (a multiple divides every group)
     bool empty = false; // nothing to add
 };
 
-int plan_reduce(const h2x_tensor_geometry* src, const h2x_tensor_geometry* dst, ReducePlan* plan)
+int plan_reduce(const h2x_tensor_geometry* src, const h2x_tensor_geometry* dst, int max_vec,
+                ReducePlan* plan)
 {
     int err = check_geometry(src);
     if (!err)
@@ -346,8 +442,8 @@ int plan_reduce(const h2x_tensor_geometry* src, const h2x_tensor_geometry* dst, 
     }
     a.kept_count = static_cast<uint32_t>(kept);
     a.red_count = static_cast<uint32_t>(red);
-    // about 2048 workgroups in all, and no group smaller than a pass of its team
-    constexpr uint64_t kTargetBlocks = 2048;
+    // about 4096 workgroups in all, and no group smaller than four passes of its team
+    constexpr uint64_t kTargetBlocks = 4096;
     uint64_t groups;
     if (plan->inner)
         groups = std::min<uint64_t>((red + 4 * kBlockSize - 1) / (4 * kBlockSize),
@@ -358,6 +454,14 @@ int plan_reduce(const h2x_tensor_geometry* src, const h2x_tensor_geometry* dst, 
             std::max<uint64_t>(kTargetBlocks / ((kept + kBlockSize - 1) / kBlockSize), 1));
     groups = std::min<uint64_t>(std::max<uint64_t>(groups, 1), 65535);
     a.chunk = static_cast<uint32_t>((red + groups - 1) / groups);
+    // 16-byte loads: the innermost reduced dimension is contiguous and a multiple of
+    // the vector long; groups then start and end on whole vectors
+    plan->vec = 1;
+    if (plan->inner && a.num_reduced > 0 && a.red_src[0] == 1 && red_extent[0] % max_vec == 0)
+    {
+        plan->vec = max_vec;
+        a.chunk = (a.chunk + max_vec - 1) / max_vec * max_vec;
+    }
     a.groups = static_cast<uint32_t>((red + a.chunk - 1) / std::max<uint32_t>(a.chunk, 1));
     if (a.groups == 0)
         a.groups = 1;
@@ -371,7 +475,11 @@ int reduce_typed(const ReducePlan& plan, hipStream_t stream)
     const unsigned int kept_blocks = (a.kept_count + kBlockSize - 1) / kBlockSize;
     if (plan.inner)
     {
-        reduce_inner_kernel<T><<<dim3(a.kept_count, a.groups), kBlockSize, 0, stream>>>(a);
+        constexpr int kVec = 16 / sizeof(T);
+        if (plan.vec == kVec)
+            reduce_inner_kernel<T, kVec><<<dim3(a.kept_count, a.groups), kBlockSize, 0, stream>>>(a);
+        else
+            reduce_inner_kernel<T, 1><<<dim3(a.kept_count, a.groups), kBlockSize, 0, stream>>>(a);
     }
     else
     {
@@ -468,15 +576,17 @@ extern "C" int h2x_tensor_transform(h2x_transform_op op, h2x_dtype dtype, int nu
     a.num_dims = nd;
     for (int i = 0; i < 4; ++i)
         a.p[i] = params ? params[i] : 0.0;
-    return dtype == H2X_F32 ? transform_typed<float>(op, a, as_stream(stream))
-                            : transform_typed<double>(op, a, as_stream(stream));
+    return dtype == H2X_F32 ? transform_typed<float>(op, num_tensors, a, as_stream(stream))
+                            : transform_typed<double>(op, num_tensors, a, as_stream(stream));
 }
 
 extern "C" size_t h2x_tensor_reduce_sum_workspace_bytes(const h2x_tensor_geometry* src_geometry,
                                                         const h2x_tensor_geometry* dst_geometry)
 {
+    // rounding the group size up to whole vectors can only lower the number of
+    // groups, so the plan without vectors bounds both element types
     ReducePlan plan;
-    if (plan_reduce(src_geometry, dst_geometry, &plan) != 0)
+    if (plan_reduce(src_geometry, dst_geometry, 1, &plan) != 0)
         return 0;
     const size_t n = static_cast<size_t>(plan.args.kept_count) * plan.args.groups * sizeof(double);
     return (std::max<size_t>(n, 1) + 255) / 256 * 256;
@@ -489,7 +599,7 @@ extern "C" int h2x_tensor_reduce_sum(h2x_dtype dtype, const h2x_tensor_geometry*
     if (dtype != H2X_F32 && dtype != H2X_F64)
         return H2X_ERR_UNSUPPORTED;
     ReducePlan plan;
-    const int err = plan_reduce(src_geometry, dst_geometry, &plan);
+    const int err = plan_reduce(src_geometry, dst_geometry, dtype == H2X_F32 ? 4 : 2, &plan);
     if (err)
         return err;
     if (plan.empty || plan.args.kept_count == 0 || plan.args.red_count == 0)

@@ -259,6 +259,61 @@ class BatchNormalization:
                                     d_input)
 
 
+def _local_geometry(t: Tensor, region: Optional[Sequence[int]] = None) -> capi.TensorGeometry:
+    """Local shape (or a region of it that starts at the first interior element)
+    and the strides of the real allocation."""
+    g = capi.TensorGeometry()
+    nd = t.get_num_dims()
+    g.num_dims = nd
+    strides = t.get_strides()
+    for i in range(nd):
+        g.local_shape[i] = t.local_shape[i] if region is None else region[i]
+        g.strides[i] = strides[i]
+    return g
+
+
+def transform(op: int, tensors: Sequence[Tensor], params: Sequence[float] = (),
+              stream: Optional[torch.cuda.Stream] = None) -> None:
+    """tensor::Transform over the interiors of 1-4 tensors of equal local shape
+    (legacy/include/distconv/tensor/algorithms/transform_cuda.hpp:359-693) for the
+    functors the library names: capi.TRANSFORM_SCALE (t *= p0), TRANSFORM_COPY
+    (t1 = t0), TRANSFORM_SCALE_BIAS (t1 = p0 * t0 + p1), TRANSFORM_SUMS_TO_STATISTICS
+    (mean, var, running_mean, running_var; p0 = count, p1 = decay)."""
+    n = len(tensors)
+    for t in tensors:
+        if list(t.local_shape) != list(tensors[0].local_shape):
+            raise ValueError("tensors of a transform must have the same local shape")  # :383-390
+    if tensors[0].get_local_size() == 0:
+        return
+    geoms = [_local_geometry(t) for t in tensors]
+    gp = (ctypes.POINTER(capi.TensorGeometry) * n)(*[ctypes.pointer(g) for g in geoms])
+    tp = (ctypes.c_void_p * n)(*[t.get_base_ptr() for t in tensors])
+    pp = (ctypes.c_double * 4)(*(list(params) + [0.0] * (4 - len(params))))
+    capi.check(capi.load().h2x_tensor_transform(op, tensors[0].h2x_dtype, n, gp, tp, pp, _stream_handle(stream)),
+               "tensor transform")
+
+
+_reduce_workspaces = {}
+
+
+def reduce_sum(src: Tensor, dst: Tensor, square: bool = False, region: Optional[Sequence[int]] = None,
+               stream: Optional[torch.cuda.Stream] = None) -> None:
+    """tensor::ReduceSum / TransformReduceSum (reduce_sum_cuda.hpp:388-439,
+    transform_reduce_sum_cuda.hpp:17-87): dst += sum of src (of its squares) over
+    every dimension along which dst's local extent is 1.  The sum over ranks that
+    the reference ends with (reduce_sum_cuda.hpp:186-192) is the caller's."""
+    lib = capi.load()
+    gs, gd = _local_geometry(src, region), _local_geometry(dst)
+    need = lib.h2x_tensor_reduce_sum_workspace_bytes(ctypes.byref(gs), ctypes.byref(gd))
+    key = torch.cuda.current_stream().cuda_stream if stream is None else stream.cuda_stream
+    ws = _reduce_workspaces.get(key)
+    if ws is None or ws.numel() < need:
+        ws = _reduce_workspaces[key] = torch.empty(max(need, 256), dtype=torch.uint8, device="cuda")
+    capi.check(lib.h2x_tensor_reduce_sum(src.h2x_dtype, ctypes.byref(gs), ctypes.c_void_p(src.get_base_ptr()),
+                                         ctypes.byref(gd), ctypes.c_void_p(dst.get_base_ptr()), int(square),
+                                         ctypes.c_void_p(ws.data_ptr()), _stream_handle(stream)), "tensor reduce_sum")
+
+
 class SoftmaxMode(Enum):
     """legacy/include/distconv/base.hpp (SoftmaxMode)."""
     INSTANCE = 0

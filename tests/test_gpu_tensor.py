@@ -53,7 +53,9 @@ def _transform(op, arrays, geoms, bases, params, dtype):
 @pytest.mark.parametrize("local,halos", [((2, 3, 5, 7), ((0, 0, 0, 0), (0, 0, 1, 2))),
                                          ((1, 4, 3, 6, 8), ((0, 0, 1, 1, 1), (0, 0, 0, 0, 0))),
                                          ((5, 1, 1, 9), ((0, 0, 0, 3), (0, 0, 0, 0))),
-                                         ((64, 33), ((0, 0), (1, 0)))])
+                                         ((64, 33), ((0, 0), (1, 0))),
+                                         ((2, 3, 4, 8), ((0, 0, 1, 1), (0, 0, 0, 2))),
+                                         ((3, 2, 5, 64), ((0, 0, 0, 0), (0, 0, 1, 0)))])
 def test_transforms_match_oracle(local, halos, dtype, oracle_mod):
     from dihydrogen_amd import capi
     rng = np.random.default_rng(11)
@@ -128,6 +130,8 @@ REDUCE_CASES = [
     ((2, 3, 4, 40, 50), (0, 0, 1, 1, 1), (0, 2, 3, 4)),
     ((6, 5, 2000), (0, 0, 0), (0,)),
     ((6, 5, 2000), (0, 0, 3), (1, 2)),
+    ((2, 3, 4, 6, 8), (0, 0, 1, 1, 1), (0, 2, 3, 4)),   # rows of whole 16-byte vectors that start on any element
+    ((2, 3, 1100, 4), (0, 0, 1, 1), (0, 2, 3)),         # more than one group per output, groups of whole vectors
 ]
 
 
