@@ -382,7 +382,7 @@ PMC_TRAFFIC = {
 }
 # sha256 (first 16 hex digits) of the kernel sources the table was measured with, see
 # kernel_sources_sha(); with other sources the traffic fields are omitted
-PMC_SOURCES_SHA = "b1c21b63828c3eb0"
+PMC_SOURCES_SHA = "963f41d071a7202b"
 PMC_COMMIT = "c41ee01"
 
 KERNEL_OF = {
@@ -400,15 +400,18 @@ KERNEL_OF = {
 }
 
 
+# the sources of the kernels of the step (batch-norm and box copy), whose traffic PMC_TRAFFIC holds
+STEP_KERNEL_SOURCES = ("h2x_bn.hip", "h2x_copy.hip", "h2x_copy_acc.hip", "h2x_copy_kernel.hpp", "h2x_device.hpp")
+
+
 def kernel_sources_sha() -> str:
-    """Hash of the HIP sources of libh2x.so: ties measured-traffic constants to
-    the kernels they were measured on."""
+    """Hash of the HIP sources of the step's kernels: ties the measured-traffic
+    constants to the kernels they were measured on."""
     h = hashlib.sha256()
     d = os.path.join(ROOT, "dihydrogen_amd", "csrc")
-    for name in sorted(os.listdir(d)):
-        if name.endswith((".hip", ".hpp")):
-            with open(os.path.join(d, name), "rb") as f:
-                h.update(name.encode() + b"\0" + f.read())
+    for name in STEP_KERNEL_SOURCES:
+        with open(os.path.join(d, name), "rb") as f:
+            h.update(name.encode() + b"\0" + f.read())
     return h.hexdigest()[:16]
 
 
