@@ -124,7 +124,7 @@ def test_backward_matches_oracle(shape, oracle_mod):
 
 @pytest.mark.parametrize("dtype", ["float32", "float64"])
 @pytest.mark.parametrize("shape", [(8, 64, 56, 56), (2, 3, 4, 5), (3, 5, 7, 9, 11), (64, 32, 7, 7), (1, 1, 1, 1),
-                                   (2, 4, 40, 40, 40), (1, 300, 3, 3)])
+                                   (2, 4, 40, 40, 40), (1, 300, 3, 3), (3, 20, 37, 37), (2, 16, 8, 16, 16), (1, 24, 2, 1024)])
 def test_two_launch_forward_and_backward_equal_the_staged_calls(shape, dtype):
     """forward()/backward() of a single rank finish the channel sums inside the
     normalising / input-gradient kernel (h2x_bn_forward_local, _backward_local);
