@@ -298,7 +298,7 @@ __global__ __launch_bounds__(kBlockSize) void reduce_outer_kernel(const ReduceAr
     a.partials[static_cast<size_t>(g) * a.kept_count + k] = acc;
 }
 
-// dst[k] += sum over the groups, in group order.
+// dst[k] += sum over the groups, in group order: a thread per output element.
 template <typename T>
 __global__ __launch_bounds__(kBlockSize) void reduce_finish_kernel(const ReduceArgs a, int inner)
 {
@@ -313,6 +313,28 @@ __global__ __launch_bounds__(kBlockSize) void reduce_finish_kernel(const ReduceA
     chain(k, a.num_kept, a.kept_div, a.kept_src, a.kept_dst, &dst_off);
     T* p = reinterpret_cast<T*>(a.dst) + dst_off;
     *p = *p + static_cast<T>(t);
+}
+
+// The same for few outputs with many groups each: a workgroup per output element;
+// thread t adds groups t, t + 256, ..., the workgroup combines its threads in the
+// fixed order of block_sum.
+template <typename T>
+__global__ __launch_bounds__(kBlockSize) void reduce_finish_wide_kernel(const ReduceArgs a, int inner)
+{
+    __shared__ double lds[kWavesPerBlock];
+    const uint32_t k = blockIdx.x;
+    double t[1] = {0.0};
+    for (uint32_t g = threadIdx.x; g < a.groups; g += kBlockSize)
+        t[0] += inner ? a.partials[static_cast<size_t>(k) * a.groups + g]
+                      : a.partials[static_cast<size_t>(g) * a.kept_count + k];
+    block_sum<1>(t, lds);
+    if (threadIdx.x == 0)
+    {
+        int64_t dst_off;
+        chain(k, a.num_kept, a.kept_div, a.kept_src, a.kept_dst, &dst_off);
+        T* p = reinterpret_cast<T*>(a.dst) + dst_off;
+        *p = *p + static_cast<T>(t[0]);
+    }
 }
 
 // ---- host ---------------------------------------------------------------------
@@ -485,7 +507,10 @@ int reduce_typed(const ReducePlan& plan, hipStream_t stream)
     {
         reduce_outer_kernel<T><<<dim3(kept_blocks, a.groups), kBlockSize, 0, stream>>>(a);
     }
-    reduce_finish_kernel<T><<<kept_blocks, kBlockSize, 0, stream>>>(a, plan.inner ? 1 : 0);
+    if (a.groups >= 16 && a.kept_count <= 4096)
+        reduce_finish_wide_kernel<T><<<a.kept_count, kBlockSize, 0, stream>>>(a, plan.inner ? 1 : 0);
+    else
+        reduce_finish_kernel<T><<<kept_blocks, kBlockSize, 0, stream>>>(a, plan.inner ? 1 : 0);
     return launch_status();
 }
 

@@ -212,6 +212,7 @@ static int test_statistics()
 
 int main()
 {
+    std::setvbuf(stdout, nullptr, _IONBF, 0); // what was printed survives a crash
     int errors = 0;
     const Shape s4({12, 10, 3, 4});
     const Distribution plain = Distribution::make_distribution(Shape({2, 2, 1, 1}));

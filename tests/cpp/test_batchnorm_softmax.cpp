@@ -251,6 +251,7 @@ static int test_bn_haloed()
 
 int main()
 {
+    std::setvbuf(stdout, nullptr, _IONBF, 0); // what was printed survives a crash
     int errors = 0;
     errors += test_bn_haloed();
     {

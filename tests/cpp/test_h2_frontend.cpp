@@ -540,16 +540,25 @@ static void test_softmax_instance()
 
 int main()
 {
-    test_both_arms();
-    test_shuffle();
-    test_softmax_instance();
-    test_batchnorm(ShapeTuple{14, 14, 8, 4});
-    test_batchnorm(ShapeTuple{6, 5, 7, 3, 2});
-    test_batchnorm(ShapeTuple{33, 5, 2}); // one spatial dimension, odd length
-    test_strided_view();
-    test_softmax();
-    test_halo();
-    test_errors();
+    std::setvbuf(stdout, nullptr, _IONBF, 0); // what was printed survives a crash
+#define RUN(call)                                                                                  \
+    do                                                                                             \
+    {                                                                                              \
+        std::printf("%s\n", #call);                                                                \
+        call;                                                                                      \
+    } while (0)
+    RUN(test_both_arms());
+    RUN(test_shuffle());
+    RUN(test_softmax_instance());
+    RUN(test_batchnorm(ShapeTuple{14, 14, 8, 4}));
+    RUN(test_batchnorm(ShapeTuple{6, 5, 7, 3, 2}));
+    RUN(test_batchnorm(ShapeTuple{33, 5, 2})); // one spatial dimension, odd length
+    RUN(test_strided_view());
+    RUN(test_softmax());
+    RUN(test_halo());
+    RUN(test_errors());
+#undef RUN
+    check_hip(hipDeviceSynchronize(), "sync");
     std::printf("test_h2_frontend: ok\n");
     return 0;
 }

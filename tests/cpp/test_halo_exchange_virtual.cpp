@@ -90,6 +90,7 @@ static int run_case(const Shape& shape, const Shape& locale, const IntVector& ov
 
 int main()
 {
+    std::setvbuf(stdout, nullptr, _IONBF, 0); // what was printed survives a crash
     int errors = 0;
     for (bool periodic : {false, true})
     {

@@ -57,6 +57,7 @@ static int run_case(const Shape& shape, const Distribution& sd, const Distributi
 
 int main()
 {
+    std::setvbuf(stdout, nullptr, _IONBF, 0); // what was printed survives a crash
     int errors = 0;
     const Shape s4({8, 8, 2, 4});
     const IntVector none(4, 0);

@@ -20,4 +20,4 @@ def test_cpp(name):
     print("running", exe, flush=True)
     r = subprocess.run([exe], capture_output=True, text=True, timeout=110)
     print(r.stdout[-2000:], r.stderr[-2000:])
-    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    assert r.returncode == 0, f"exit status {r.returncode}\n" + r.stdout[-2000:] + r.stderr[-2000:]
