@@ -202,12 +202,14 @@ class SoftmaxWorkload:
 class ShuffleWorkload:
     """Sample-parallel (N over `ranks` ranks) <-> spatial-parallel (H x W grid)."""
 
-    def __init__(self, gshape, seed, ranks=4, grid=(2, 2)):
+    def __init__(self, gshape, seed, ranks=4, grid=(2, 2), dst_overlap=0):
         import torch
         from dihydrogen_amd.layers import TensorShufflerVirtual
         from dihydrogen_amd.tensor import Distribution, LocaleVirtual, Tensor
         g = torch.Generator(device="cuda").manual_seed(seed)
-        sd, dd = Distribution([1, 1, 1, ranks]), Distribution([grid[0], grid[1], 1, 1])
+        sd = Distribution([1, 1, 1, ranks])
+        dd = (Distribution.make_overlapped_distribution([grid[0], grid[1], 1, 1], [dst_overlap, dst_overlap, 0, 0])
+              if dst_overlap else Distribution([grid[0], grid[1], 1, 1]))
         self.src = [Tensor(gshape, LocaleVirtual(r, ranks), sd).allocate() for r in range(ranks)]
         self.dst = [Tensor(gshape, LocaleVirtual(r, ranks), dd).allocate() for r in range(ranks)]
         for t in self.src:
@@ -772,6 +774,13 @@ def main() -> int:
         breakdown["C5_shuffle_round_trip"] = entry(8 * shf.elems * 4, 2 * shf.elems,
                                                    lambda: (shf.forward(), shf.backward()), inner=2)
         del shf
+        torch.cuda.empty_cache()
+        # the spatial side with a halo of 1 (what a convolution behind the shuffle needs): the unpack
+        # writes rows of 64 floats into rows of 66, the backward pack reads them
+        shfh = ShuffleWorkload((128, 128, 64, 32), SEED + 5, dst_overlap=1)
+        breakdown["C5_shuffle_haloed_dst_round_trip"] = entry(8 * shfh.elems * 4, 2 * shfh.elems,
+                                                              lambda: (shfh.forward(), shfh.backward()), inner=2)
+        del shfh
         torch.cuda.empty_cache()
         # the same tensor between 16 ranks: 256 boxes a direction, one launch each for pack and unpack
         shf16 = ShuffleWorkload((128, 128, 64, 32), SEED + 5, ranks=16, grid=(4, 4))
