@@ -1,7 +1,8 @@
 """Runs the C++ tests of the host-side layer (tests/cpp) on the GPU.
 
 The binaries are built beforehand by __graft_entry__.build() (make -C tests/cpp);
-each returns 0 when every check passed."""
+each returns 0 when every check passed.  Each runs in a process of its own beside
+this one; the file is named to be collected after the in-process GPU tests."""
 import os
 import subprocess
 
