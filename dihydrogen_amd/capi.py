@@ -135,6 +135,8 @@ SIGNATURES = {
     "h2x_softmax_instance_exp": (c_int, [c_int, c_int, c_size_t, c_void_p, c_void_p, c_void_p, c_void_p,
                                          c_void_p, c_void_p]),
     "h2x_softmax_instance_normalize": (c_int, [c_int, c_int, c_size_t, c_void_p, c_void_p, c_void_p]),
+    "h2x_softmax_instance_forward_local": (c_int, [c_int, c_int, c_size_t, c_void_p, c_void_p, c_void_p, c_void_p,
+                                                   c_void_p, c_void_p]),
     "h2x_softmax_instance_dot": (c_int, [c_int, c_int, c_size_t, c_void_p, c_void_p, c_void_p, c_void_p,
                                          c_void_p]),
     "h2x_softmax_instance_gradient": (c_int, [c_int, c_int, c_size_t, c_void_p, c_void_p, c_void_p,

@@ -485,7 +485,8 @@ enum InstReduce : int
 {
     kInstMax = 0,   // max x                       -> T partial
     kInstExpSum = 1, // y = exp(x - max); sum y     -> double partial
-    kInstDot = 2     // sum y * dy                  -> double partial
+    kInstDot = 2,    // sum y * dy                  -> double partial
+    kInstSumExp = 3  // sum exp(x - max), y untouched -> double partial
 };
 
 // One pass over the chunk [begin, end) of sample n.  a: x (max, exp) or y (dot);
@@ -504,7 +505,7 @@ __global__ __launch_bounds__(kBlockSize) void softmax_inst_reduce_kernel(
     const T* ap = a + static_cast<size_t>(n) * sample_size;
     const T* bp = MODE == kInstDot ? b + static_cast<size_t>(n) * sample_size : nullptr;
     T* op = MODE == kInstExpSum ? out + static_cast<size_t>(n) * sample_size : nullptr;
-    const T shift = MODE == kInstExpSum ? sample_param[n] : T(0);
+    const T shift = (MODE == kInstExpSum || MODE == kInstSumExp) ? sample_param[n] : T(0);
     constexpr size_t kStride = static_cast<size_t>(kBlockSize) * VEC;
 
     T mx = Limits<T>::min_normal; // softmax.cu:88-99: the maximum starts at min_normal
@@ -531,7 +532,7 @@ __global__ __launch_bounds__(kBlockSize) void softmax_inst_reduce_kernel(
                     {
                         mx = va[u][j] >= mx ? va[u][j] : mx;
                     }
-                    else if constexpr (MODE == kInstExpSum)
+                    else if constexpr (MODE == kInstExpSum || MODE == kInstSumExp)
                     {
                         const T e = exp_t(va[u][j] - shift);
                         va[u][j] = e;
@@ -605,12 +606,22 @@ __global__ __launch_bounds__(kBlockSize) void softmax_inst_finish_kernel(
     }
 }
 
-// y = max(y / sum, sqrt(min_normal))  (SoftmaxOp, softmax.cu:424-435) or
-// dx = y > sqrt(min_normal) ? y * (dy - dp) : 0  (bp_compute_func, :483-500)
-template <typename T, int VEC, bool BACKWARD>
+// kMapNormalize: y = max(y / sum, sqrt(min_normal))  (SoftmaxOp, softmax.cu:424-435);
+// kMapGradient:  dx = y > sqrt(min_normal) ? y * (dy - dp) : 0  (bp_compute_func, :483-500);
+// kMapFromInput: y = max(exp(x - max) / sum, sqrt(min_normal)): the exponentials are
+// made again from x instead of being read back (the same bits: the same function of
+// the same arguments), for samples that are whole on this rank.
+enum InstMap : int
+{
+    kMapNormalize = 0,
+    kMapGradient = 1,
+    kMapFromInput = 2
+};
+
+template <typename T, int VEC, int KIND>
 __global__ __launch_bounds__(kBlockSize) void softmax_inst_map_kernel(
-    const T* y_in, const T* __restrict__ dy, const T* __restrict__ sample_param, T* out,
-    size_t sample_size, T min_output)
+    const T* y_in, const T* __restrict__ dy, const T* __restrict__ sample_param,
+    const T* __restrict__ sample_shift, T* out, size_t sample_size, T min_output)
 {
     using P = Pack<T, VEC>;
     const int n = blockIdx.y;
@@ -620,7 +631,7 @@ __global__ __launch_bounds__(kBlockSize) void softmax_inst_map_kernel(
     const size_t off = static_cast<size_t>(n) * sample_size + i;
     const T p = sample_param[n];
     P v = P::load(y_in + off);
-    if constexpr (BACKWARD)
+    if constexpr (KIND == kMapGradient)
     {
         const P g = P::load(dy + off);
 #pragma unroll
@@ -629,10 +640,14 @@ __global__ __launch_bounds__(kBlockSize) void softmax_inst_map_kernel(
     }
     else
     {
+        T shift = T(0);
+        if constexpr (KIND == kMapFromInput)
+            shift = sample_shift[n];
 #pragma unroll
         for (int j = 0; j < VEC; ++j)
         {
-            const T r = v[j] / p;
+            const T e = KIND == kMapFromInput ? exp_t(v[j] - shift) : v[j];
+            const T r = e / p;
             v[j] = r > min_output ? r : min_output;
         }
     }
@@ -686,22 +701,38 @@ int inst_reduce(int n, size_t sample_size, const void* a, const void* b, void* o
     return launch_status();
 }
 
-template <typename T, bool BACKWARD>
-int inst_map(int n, size_t sample_size, const void* y, const void* dy, const void* param, void* out,
-             hipStream_t st)
+template <typename T, int KIND>
+int inst_map(int n, size_t sample_size, const void* y, const void* dy, const void* param,
+             const void* shift, void* out, hipStream_t st)
 {
     constexpr int kFull = 16 / sizeof(T);
     const int v = vector_width<T>(sample_size, kFull, {y, dy ? dy : y, out});
     const T min_output = inst_min_output<T>();
     if (v == kFull)
-        softmax_inst_map_kernel<T, kFull, BACKWARD><<<pixel_grid(sample_size, kFull, n), kBlockSize, 0, st>>>(
+        softmax_inst_map_kernel<T, kFull, KIND><<<pixel_grid(sample_size, kFull, n), kBlockSize, 0, st>>>(
             static_cast<const T*>(y), static_cast<const T*>(dy), static_cast<const T*>(param),
-            static_cast<T*>(out), sample_size, min_output);
+            static_cast<const T*>(shift), static_cast<T*>(out), sample_size, min_output);
     else
-        softmax_inst_map_kernel<T, 1, BACKWARD><<<pixel_grid(sample_size, 1, n), kBlockSize, 0, st>>>(
+        softmax_inst_map_kernel<T, 1, KIND><<<pixel_grid(sample_size, 1, n), kBlockSize, 0, st>>>(
             static_cast<const T*>(y), static_cast<const T*>(dy), static_cast<const T*>(param),
-            static_cast<T*>(out), sample_size, min_output);
+            static_cast<const T*>(shift), static_cast<T*>(out), sample_size, min_output);
     return launch_status();
+}
+
+// Forward pass of samples that are whole on this rank: maximum, sum of the
+// exponentials (y is not written), y from x: 4 tensor passes instead of 5.
+template <typename T>
+int inst_forward_local(int n, size_t sample_size, const void* x, void* y, void* sample_max,
+                       void* sample_exp, void* workspace, hipStream_t st)
+{
+    int err = inst_reduce<T, kInstMax>(n, sample_size, x, nullptr, nullptr, nullptr, sample_max,
+                                       workspace, st);
+    // `y` takes part in the choice of the vector width only, as in the staged call,
+    // so that the sum is cut up and added in the same order
+    if (!err)
+        err = inst_reduce<T, kInstSumExp>(n, sample_size, x, nullptr, y, sample_max, sample_exp,
+                                          workspace, st);
+    return err ? err : inst_map<T, kMapFromInput>(n, sample_size, x, nullptr, sample_exp, sample_max, y, st);
 }
 
 bool inst_bad(int num_samples, size_t sample_size)
@@ -809,10 +840,10 @@ extern "C" int h2x_softmax_instance_normalize(h2x_dtype dtype, int num_samples, 
 {
     if (!sample_exp || !y)
         return num_samples == 0 || sample_size == 0 ? H2X_SUCCESS : H2X_ERR_INVALID_ARGUMENT;
-    H2X_INST_ENTRY((inst_map<float, false>(num_samples, sample_size, y, nullptr, sample_exp, y,
-                                           as_stream(stream))),
-                   (inst_map<double, false>(num_samples, sample_size, y, nullptr, sample_exp, y,
-                                            as_stream(stream))));
+    H2X_INST_ENTRY((inst_map<float, kMapNormalize>(num_samples, sample_size, y, nullptr, sample_exp,
+                                                   nullptr, y, as_stream(stream))),
+                   (inst_map<double, kMapNormalize>(num_samples, sample_size, y, nullptr, sample_exp,
+                                                    nullptr, y, as_stream(stream))));
 }
 
 extern "C" int h2x_softmax_instance_dot(h2x_dtype dtype, int num_samples, size_t sample_size,
@@ -833,8 +864,21 @@ extern "C" int h2x_softmax_instance_gradient(h2x_dtype dtype, int num_samples, s
 {
     if (!y || !dy || !sample_dp || !dx)
         return num_samples == 0 || sample_size == 0 ? H2X_SUCCESS : H2X_ERR_INVALID_ARGUMENT;
-    H2X_INST_ENTRY((inst_map<float, true>(num_samples, sample_size, y, dy, sample_dp, dx,
-                                          as_stream(stream))),
-                   (inst_map<double, true>(num_samples, sample_size, y, dy, sample_dp, dx,
-                                           as_stream(stream))));
+    H2X_INST_ENTRY((inst_map<float, kMapGradient>(num_samples, sample_size, y, dy, sample_dp, nullptr,
+                                                  dx, as_stream(stream))),
+                   (inst_map<double, kMapGradient>(num_samples, sample_size, y, dy, sample_dp, nullptr,
+                                                   dx, as_stream(stream))));
+}
+
+extern "C" int h2x_softmax_instance_forward_local(h2x_dtype dtype, int num_samples,
+                                                  size_t sample_size, const void* x, void* y,
+                                                  void* sample_max, void* sample_exp,
+                                                  void* workspace, h2x_stream_t stream)
+{
+    if (!x || !y || !sample_max || !sample_exp || !workspace)
+        return num_samples == 0 || sample_size == 0 ? H2X_SUCCESS : H2X_ERR_INVALID_ARGUMENT;
+    H2X_INST_ENTRY((inst_forward_local<float>(num_samples, sample_size, x, y, sample_max, sample_exp,
+                                              workspace, as_stream(stream))),
+                   (inst_forward_local<double>(num_samples, sample_size, x, y, sample_max, sample_exp,
+                                               workspace, as_stream(stream))));
 }

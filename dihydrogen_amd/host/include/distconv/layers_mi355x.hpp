@@ -513,6 +513,14 @@ public:
         const size_t size = spatial * c;
         T* scalars = per_sample<T>(n);
         T *smax = scalars, *sexp = scalars + n;
+        if (!m_allreducer)
+        {
+            // every sample is whole on this rank: the stages need not be separate calls
+            DISTCONV_CHECK_H2X(h2x_softmax_instance_forward_local(dt, n, size, x.get_const_base_ptr(),
+                                                                  y.get_base_ptr(), smax, sexp,
+                                                                  workspace(n), m_stream));
+            return 0;
+        }
         DISTCONV_CHECK_H2X(h2x_softmax_instance_max(dt, n, size, x.get_const_base_ptr(), smax,
                                                     workspace(n), m_stream));
         if (m_allreducer)

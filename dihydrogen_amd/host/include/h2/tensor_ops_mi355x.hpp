@@ -421,12 +421,10 @@ void softmax_instance_forward_impl(GPUDev_t, const Tensor<T>& x, Tensor<T>& y)
     void* ws = mi355x::stream_scratch(s, h2x_softmax_instance_workspace_bytes(n), 2);
     T* scalars = static_cast<T*>(mi355x::stream_scratch(s, 2 * n * sizeof(T), 3));
     const h2x_dtype dt = mi355x::dtype_of<T>();
-    mi355x::check(h2x_softmax_instance_max(dt, n, size, x.const_data(), scalars, ws, s), "softmax max");
-    mi355x::check(h2x_softmax_instance_exp(dt, n, size, x.const_data(), scalars, y.data(), scalars + n,
-                                           ws, s),
-                  "softmax exp");
-    mi355x::check(h2x_softmax_instance_normalize(dt, n, size, scalars + n, y.data(), s),
-                  "softmax normalize");
+    // an h2 tensor is one rank's whole tensor: no all-reduce between the stages
+    mi355x::check(h2x_softmax_instance_forward_local(dt, n, size, x.const_data(), y.data(), scalars,
+                                                     scalars + n, ws, s),
+                  "softmax instance forward");
 }
 template <typename T>
 void softmax_instance_backward_impl(GPUDev_t, const Tensor<T>& y, const Tensor<T>& dy, Tensor<T>& dx)

@@ -364,6 +364,12 @@ class Softmax:
         dt, size, ws = x.h2x_dtype, c * s, self._workspace(n)
         smax = torch.empty(n, dtype=x.dtype, device=x.device)
         sexp = torch.empty(n, dtype=x.dtype, device=x.device)
+        if self.allreduce is None:
+            # every sample is whole on this rank: the stages need not be separate calls
+            capi.check(self._lib.h2x_softmax_instance_forward_local(
+                dt, n, size, _ptr(x.get_base_ptr()), _ptr(y.get_base_ptr()), _ptr(smax), _ptr(sexp), _ptr(ws), st),
+                "softmax instance forward")
+            return 0
         capi.check(self._lib.h2x_softmax_instance_max(dt, n, size, _ptr(x.get_base_ptr()), _ptr(smax),
                                                       _ptr(ws), st), "softmax instance max")
         if self.allreduce:

@@ -495,6 +495,18 @@ int h2x_softmax_instance_exp(h2x_dtype dtype, int num_samples, size_t sample_siz
 int h2x_softmax_instance_normalize(h2x_dtype dtype, int num_samples, size_t sample_size,
                                    const void* sample_exp, void* y, h2x_stream_t stream);
 
+/**
+ * The three forward stages for samples that are whole on this rank (no
+ * all-reduce between them, softmax.hpp:52-62 with one process per sample): what
+ * h2x_softmax_instance_max, _exp and _normalize leave in y, sample_max and
+ * sample_exp, bit for bit, in four passes over the tensors instead of five: the
+ * exponentials are summed without being stored and made again from x when y is
+ * written.  The staged entry points remain for samples spread over ranks.
+ */
+int h2x_softmax_instance_forward_local(h2x_dtype dtype, int num_samples, size_t sample_size,
+                                       const void* x, void* y, void* sample_max, void* sample_exp,
+                                       void* workspace, h2x_stream_t stream);
+
 /** sample_dp[n] = sum_i y * dy: bp_dotproduct, softmax.cu:458-481. */
 int h2x_softmax_instance_dot(h2x_dtype dtype, int num_samples, size_t sample_size, const void* y,
                              const void* dy, void* sample_dp, void* workspace, h2x_stream_t stream);

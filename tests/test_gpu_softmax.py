@@ -202,3 +202,38 @@ def test_instance_mode_split_sample_allreduce(oracle_mod):
     torch.cuda.synchronize()
     got = np.concatenate([ys[0].real_view().cpu().numpy(), ys[1].real_view().cpu().numpy()], axis=2)
     assert max_rel(got, want) <= TOL
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("shape", INSTANCE_CASES + [(3, 1031)])
+def test_instance_forward_in_four_passes_equals_the_staged_calls(shape, dtype):
+    """h2x_softmax_instance_forward_local (whole samples on this rank: the exponentials are
+    summed without being stored and made again from x) against the three staged calls:
+    y, the per-sample maxima and the per-sample sums must agree bit for bit."""
+    import torch
+    from dihydrogen_amd import capi
+    lib = capi.load()
+    rng = np.random.default_rng(5)
+    x = (2.0 * rng.standard_normal(shape)).astype(dtype)
+    n, size = shape[0], int(np.prod(shape[1:]))
+    dt = capi.F32 if dtype == np.float32 else capi.F64
+    xd = torch.from_numpy(x).cuda()
+    ws = torch.empty(lib.h2x_softmax_instance_workspace_bytes(n), dtype=torch.uint8, device="cuda")
+    tdt = torch.float32 if dtype == np.float32 else torch.float64
+    outs = []
+    for local in (True, False):
+        y = torch.full(shape, float("nan"), dtype=tdt, device="cuda")
+        mx = torch.full((n,), float("nan"), dtype=tdt, device="cuda")
+        ex = torch.full((n,), float("nan"), dtype=tdt, device="cuda")
+        if local:
+            capi.check(lib.h2x_softmax_instance_forward_local(dt, n, size, xd.data_ptr(), y.data_ptr(), mx.data_ptr(),
+                                                              ex.data_ptr(), ws.data_ptr(), None))
+        else:
+            capi.check(lib.h2x_softmax_instance_max(dt, n, size, xd.data_ptr(), mx.data_ptr(), ws.data_ptr(), None))
+            capi.check(lib.h2x_softmax_instance_exp(dt, n, size, xd.data_ptr(), mx.data_ptr(), y.data_ptr(),
+                                                    ex.data_ptr(), ws.data_ptr(), None))
+            capi.check(lib.h2x_softmax_instance_normalize(dt, n, size, ex.data_ptr(), y.data_ptr(), None))
+        torch.cuda.synchronize()
+        outs.append([t.cpu().numpy() for t in (y, mx, ex)])
+    for name, a, b in zip(("y", "sample_max", "sample_exp"), *outs):
+        assert np.array_equal(a, b), name
