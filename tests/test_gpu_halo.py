@@ -390,6 +390,39 @@ def test_clear_halo(oracle_mod):
         assert np.array_equal(f, want)
 
 
+@pytest.mark.parametrize("shape,locale,overlap", [((32, 31, 4, 8), (2, 2, 1, 1), (1, 2, 0, 0)),
+                                                  ((12, 9, 10, 3, 2), (2, 1, 2, 1, 1), (2, 0, 1, 0, 0))])
+def test_clear_halo_one_dimension_at_a_time(shape, locale, overlap):
+    """The reference's own check (legacy/tests/tensor/test_tensor_mpi_cuda.cu:162-231): fill
+    with 1, clear the halo of ONE dimension, and every cell whose index along that
+    dimension lies in the halo is 0, every other cell - the halos of the other
+    dimensions included - still 1."""
+    import torch
+    from dihydrogen_amd.layers import HaloExchangeVirtual
+    from dihydrogen_amd.tensor import Distribution, LocaleVirtual, Tensor
+    n = int(np.prod(locale))
+    dist = Distribution.make_overlapped_distribution(locale, overlap)
+    tensors = [Tensor(shape, LocaleVirtual(r, n), dist).allocate() for r in range(n)]
+    xch = HaloExchangeVirtual(tensors)
+    for d in range(len(shape)):
+        for t in tensors:
+            t.data.fill_(1.0)
+        xch.clear_halo(d)
+        torch.cuda.synchronize()
+        for t in tensors:
+            f = t.real_view().cpu().numpy()
+            want = np.ones_like(f)
+            ov = t.overlap[d]
+            if ov:
+                axis = len(shape) - 1 - d
+                idx = [slice(None)] * len(shape)
+                idx[axis] = slice(0, ov)
+                want[tuple(idx)] = 0
+                idx[axis] = slice(f.shape[axis] - ov, None)
+                want[tuple(idx)] = 0
+            assert np.array_equal(f, want), (d, t.locale.get_rank() if hasattr(t, "locale") else None)
+
+
 def test_zero_width_is_noop():
     import torch
     from dihydrogen_amd import capi
