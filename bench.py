@@ -154,9 +154,9 @@ class BatchNormWorkload:
 
 
 class HaloWorkload:
-    """Halo exchange of a periodic 2 x 2 x 2 grid of virtual ranks."""
+    """Halo exchange of a 2 x 2 x 2 grid of virtual ranks (periodic unless said otherwise)."""
 
-    def __init__(self, local_spatial, channels, seed):
+    def __init__(self, local_spatial, channels, seed, periodic=True):
         import torch
         from dihydrogen_amd.layers import HaloExchangeVirtual
         from dihydrogen_amd.tensor import Distribution, LocaleVirtual, Tensor
@@ -167,7 +167,7 @@ class HaloWorkload:
         self.ranks = [Tensor(gshape, LocaleVirtual(r, 8), dist).allocate() for r in range(8)]
         for t in self.ranks:
             t.interior_view().uniform_(-1, 1, generator=g)
-        self.xch = HaloExchangeVirtual(self.ranks, periodic=True)
+        self.xch = HaloExchangeVirtual(self.ranks, periodic=periodic)
         face = (local_spatial + 2) ** 2 * channels
         # per rank: 3 dims x 2 sides x (pack: read+write, unpack: read+write) x 4 bytes
         self.bytes = 8 * 3 * 2 * 2 * 2 * face * 4
@@ -713,6 +713,9 @@ def main() -> int:
                 halo.xch.clear_halo(d)
 
         breakdown["C2_clear_halo_8ranks"] = entry(halo.bytes // 4, halo.elems // 2, clear_all, inner=2)
+        # the same strips cleared by one batched call (3 launches instead of 24)
+        breakdown["C2_clear_halos_batched_8ranks"] = entry(halo.bytes // 4, halo.elems // 2, halo.xch.clear_halos,
+                                                          inner=2)
         # pack: read + write; accumulating unpack: read buffer, read + write tensor -> 5/4 of the forward bytes
         breakdown["C2_halo_reverse_sum_8ranks"] = entry(
             halo.bytes * 5 // 4, halo.elems,
@@ -726,9 +729,25 @@ def main() -> int:
         stat = _T([1, 1, 1, 64, 1], _LV(0, 1), _D.make_localized_distribution(5)).allocate()
         breakdown["C3_reduce_sum_per_channel"] = entry(S3 * 4, S3, lambda: L.reduce_sum(bn3.x, stat))
         breakdown["C3_reduce_sqsum_per_channel"] = entry(S3 * 4, S3, lambda: L.reduce_sum(bn3.x, stat, square=True))
+        # what a convolution does before it runs (convolution.hpp:400-411): clear the halos, exchange.
+        # Bytes: the exchange's; the clearing is overhead.  On the periodic grid every strip is overwritten
+        # by the exchange, on the open one half of them.
+        breakdown["C2_clear_then_exchange"] = entry(halo.bytes, halo.elems,
+                                                    lambda: (halo.xch.clear_halos(), halo.run()), inner=2)
+        breakdown["C2_clear_unfilled_then_exchange"] = entry(
+            halo.bytes, halo.elems, lambda: (halo.xch.clear_halos(only_unfilled=True), halo.run()), inner=2)
         yard_x, yard_y = bn3.x.data, bn3.y.data
         breakdown["yardstick_torch_copy_268MB"] = entry(2 * S3 * 4, S3, lambda: yard_y.copy_(yard_x), eager=False)
         del bn3, halo, b, yard_x, yard_y
+        torch.cuda.empty_cache()
+        # the same on an open (non-periodic) 2 x 2 x 2 grid: every rank has a neighbour on 3 of its 6 sides
+        halo_open = HaloWorkload(128, 32, SEED + 2, periodic=False)
+        breakdown["C2open_clear_then_exchange"] = entry(halo_open.bytes // 2, halo_open.elems // 2,
+                                                        lambda: (halo_open.xch.clear_halos(), halo_open.run()), inner=2)
+        breakdown["C2open_clear_unfilled_then_exchange"] = entry(
+            halo_open.bytes // 2, halo_open.elems // 2,
+            lambda: (halo_open.xch.clear_halos(only_unfilled=True), halo_open.run()), inner=2)
+        del halo_open
         torch.cuda.empty_cache()
         # strided batch-norm: the config 3 shard with a halo of 1 on all three spatial dimensions
         bn3h = BatchNormWorkload((4, 64, 64, 64, 64), SEED + 6, overlap=1)

@@ -146,6 +146,7 @@ SIGNATURES = {
                                         c_int, c_void_p, c_int, c_int, c_int, c_void_p]),
     "h2x_halo_pack_or_unpack_batched": (c_int, [c_int, POINTER(HaloFace), c_int, c_void_p]),
     "h2x_halo_clear": (c_int, [c_int, c_void_p, c_int, POINTER(c_int64), c_int, c_int, c_void_p]),
+    "h2x_halo_clear_batched": (c_int, [c_int, POINTER(HaloFace), c_int, c_void_p]),
     "h2x_halo_exchange_fused": (c_int, [c_int, POINTER(HaloTransfer), c_int, c_void_p]),
     "h2x_shuffle_plan_create": (c_int, [POINTER(ShuffleGeometry), POINTER(c_void_p)]),
     "h2x_shuffle_plan_destroy": (c_int, [c_void_p]),

@@ -577,6 +577,40 @@ extern "C" int h2x_halo_clear(h2x_dtype dtype, void* tensor, int num_dims,
     return l.flush();
 }
 
+extern "C" int h2x_halo_clear_batched(h2x_dtype dtype, const h2x_halo_face* faces, int num_faces,
+                                      h2x_stream_t stream)
+{
+    const int es = elem_size_of(dtype);
+    if (es == 0)
+        return H2X_ERR_UNSUPPORTED;
+    if (num_faces < 0 || (num_faces > 0 && !faces))
+        return H2X_ERR_INVALID_ARGUMENT;
+    // validate everything before anything is launched
+    BoxList boxes(num_faces);
+    for (int i = 0; i < num_faces; ++i)
+    {
+        const int err = halo_box(faces[i], &boxes[i]);
+        if (err != 0)
+            return err;
+        if (boxes[i].count > 0 && !faces[i].tensor)
+            return H2X_ERR_INVALID_ARGUMENT;
+        if (boxes[i].count >= (1ll << 31))
+            return H2X_ERR_TOO_LARGE;
+    }
+    // sparse strips first, then the others: boxes of one kind share launches
+    Launcher l(as_stream(stream), es, dtype, H2X_HALO_ID);
+    for (int pass = 0; pass < 2; ++pass)
+        for (int i = 0; i < num_faces; ++i)
+        {
+            if (boxes[i].count == 0 || box_is_sparse(boxes[i], es) != (pass == 0))
+                continue;
+            const int err = l.add(boxes[i], faces[i].tensor, nullptr, kClear);
+            if (err != 0)
+                return err;
+        }
+    return l.flush();
+}
+
 extern "C" int h2x_halo_exchange_fused(h2x_dtype dtype, const h2x_halo_transfer* transfers,
                                        int num_transfers, h2x_stream_t stream)
 {

@@ -384,6 +384,51 @@ public:
         }
     }
 
+    // Tensor::clear_halo for every dimension that has a halo, on every rank, in
+    // batched launches: the loop that precedes the forward exchange in
+    // Convolution::forward (convolution.hpp:400-411).  only_unfilled: only the
+    // sides without a neighbour are cleared.  A full-width exchange() that
+    // follows overwrites every other halo strip completely (a strip spans the
+    // whole real extent of the other dimensions), and the stale values it moves
+    // into corner cells in the meantime are themselves overwritten by a later
+    // dimension's phase -- neighbours along one dimension sit at the same
+    // position of every other dimension, so a corner that no later phase fills
+    // receives cleared cells -- so the tensors end up exactly as after clearing
+    // everything first.
+    void clear_halos(hipStream_t stream, bool only_unfilled = false)
+    {
+        std::vector<h2x_halo_face> faces;
+        for (auto& r : m_ranks)
+        {
+            auto& t = r->get_tensor();
+            if (t.get_local_size() == 0)
+                continue;
+            for (int d = 0; d < t.get_num_dims(); ++d)
+            {
+                const int width = t.get_halo_width(d);
+                if (width == 0)
+                    continue;
+                for (Side side : SIDES)
+                {
+                    if (only_unfilled && r->get_peer(d, side) != kProcNull)
+                        continue;
+                    h2x_halo_face f = {};
+                    f.tensor = t.get_buffer();
+                    for (int i = 0; i < t.get_num_dims(); ++i)
+                        f.real_shape[i] = static_cast<int64_t>(t.get_local_real_shape()[i]);
+                    f.num_dims = t.get_num_dims();
+                    f.dim = d;
+                    f.side = static_cast<int>(side);
+                    f.width = width;
+                    faces.push_back(f);
+                }
+            }
+        }
+        if (!faces.empty())
+            DISTCONV_CHECK_H2X(h2x_halo_clear_batched(TensorType::h2x_type(), faces.data(),
+                                                      static_cast<int>(faces.size()), stream));
+    }
+
     // The exchange of all dimensions with every strip moved straight from the
     // neighbour's tensor into this rank's (one launch per dimension and group
     // of ranks, no buffers).  The tensors end up as after exchange().

@@ -677,6 +677,44 @@ class HaloExchangeVirtual:
                        "clear_halo")
 
 
+    def clear_halos(self, only_unfilled: bool = False) -> None:
+        """clear_halo of every dimension that has a halo, on every rank, in batched
+        launches: the loop that precedes the forward exchange in Convolution::forward
+        (legacy/include/distconv/dnn_backend/convolution.hpp:400-411).
+
+        ``only_unfilled``: only the sides without a neighbour are cleared.  A
+        full-width ``exchange()`` that follows overwrites every other halo strip
+        completely (a strip spans the whole real extent of the other dimensions);
+        the stale values it moves into corner cells on the way are overwritten by a
+        later dimension's phase, and a corner that no later phase fills receives
+        cleared cells, because neighbours along one dimension sit at the same
+        position of every other dimension.  The tensors end up exactly as after
+        clearing everything first."""
+        key = ("clear", only_unfilled, self._addresses())
+        if key not in self._faces:
+            faces = []
+            for r, t in enumerate(self.tensors):
+                if t.get_local_size() == 0:
+                    continue
+                for d in range(self.nd):
+                    if t.overlap[d] == 0:
+                        continue
+                    for side in (capi.LHS, capi.RHS):
+                        if only_unfilled and self.find_peer_rank(r, d, side) is not None:
+                            continue
+                        f = capi.HaloFace()
+                        f.tensor = t.get_buffer()
+                        for i, e in enumerate(t.local_real_shape):
+                            f.real_shape[i] = e
+                        f.num_dims, f.dim, f.side, f.width, f.inner = self.nd, d, side, t.overlap[d], 0
+                        faces.append(f)
+            self._faces[key] = (capi.HaloFace * len(faces))(*faces)
+        arr = self._faces[key]
+        if len(arr):
+            capi.check(self._lib.h2x_halo_clear_batched(self.tensors[0].h2x_dtype, arr, len(arr),
+                                                        _stream_handle(self.stream)), "clear_halos")
+
+
 class TensorShufflerVirtual:
     """TensorMPICUDAShuffler for all virtual ranks of a (src, dst) pair of
     distributed tensors (legacy/include/distconv/tensor/shuffle_mpi_cuda.hpp:14-512,

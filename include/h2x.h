@@ -583,6 +583,23 @@ int h2x_halo_pack_or_unpack_batched(h2x_dtype dtype,
                                     h2x_stream_t stream);
 
 /**
+ * tensor[strip] = 0 for every face of `faces` (tensor, real_shape, num_dims, dim,
+ * side, width and inner are read; inner = 0 names the halo strip), any number of
+ * tensors, dimensions and sides, in as few launches as the kinds of strips allow
+ * (one for the strips of the innermost dimension, one per 16 of the others).
+ * What a loop of TensorImplHelper::clear_halo over dimensions and tensors does
+ * (legacy/src/tensor/tensor_mpi_cuda.cu:14-84; the loop:
+ * legacy/include/distconv/dnn_backend/convolution.hpp:400-411), and its building
+ * block where only some sides need clearing: a side whose neighbour will
+ * overwrite the whole strip in the exchange that follows need not be cleared.
+ * `faces` is host memory, read before return.
+ */
+int h2x_halo_clear_batched(h2x_dtype dtype,
+                           const h2x_halo_face* faces,
+                           int num_faces,
+                           h2x_stream_t stream);
+
+/**
  * tensor[strip] = 0 for the outer strips of `dim` on both sides, width =
  * the real halo width.  Replaces TensorImplHelper::clear_halo
  * (legacy/src/tensor/tensor_mpi_cuda.cu:14-84).

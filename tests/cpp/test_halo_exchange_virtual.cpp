@@ -8,7 +8,9 @@ enum Mode
 {
     kBuffers,        // pack, unpack through receive buffers, one stream
     kFused,          // tensor-to-tensor transfers
-    kBoundaryStreams // the reference's driver signature with two boundary streams per dimension
+    kBoundaryStreams, // the reference's driver signature with two boundary streams per dimension
+    kClearBatched,    // pack, unpack; the halos cleared by one batched call for all ranks and dimensions
+    kClearUnfilled    // pack, unpack; only the halo strips without a neighbour cleared beforehand
 };
 
 static int run_case(const Shape& shape, const Shape& locale, const IntVector& overlap, bool periodic,
@@ -27,9 +29,13 @@ static int run_case(const Shape& shape, const Shape& locale, const IntVector& ov
         ptrs.push_back(ranks.back().get());
     }
     HaloExchangeVirtual<float> xch(ptrs, periodic);
-    for (int d = 0; d < nd; ++d) // Convolution clears the halo before every exchange
-        for (auto* t : ptrs)
-            t->clear_halo(d, nullptr);
+    // Convolution clears the halo before every exchange (the fields carry -1 there)
+    if (mode == kClearBatched || mode == kClearUnfilled)
+        xch.clear_halos(nullptr, mode == kClearUnfilled);
+    else
+        for (int d = 0; d < nd; ++d)
+            for (auto* t : ptrs)
+                t->clear_halo(d, nullptr);
     if (mode == kFused)
     {
         xch.exchange_fused(nullptr);
@@ -104,6 +110,13 @@ int main()
         errors += run_case(Shape({8, 10, 12, 3, 2}), Shape({2, 2, 2, 1, 1}), IntVector({1, 1, 1, 0, 0}), periodic, kFused);
         errors += run_case(Shape({8, 10, 12, 3, 2}), Shape({2, 2, 2, 1, 1}), IntVector({1, 1, 1, 0, 0}), periodic,
                            kBoundaryStreams);
+        // the clearing batched, and cut down to the strips the exchange does not overwrite
+        for (Mode m : {kClearBatched, kClearUnfilled})
+        {
+            errors += run_case(Shape({13, 11, 3, 2}), Shape({3, 2, 1, 1}), IntVector({1, 2, 0, 0}), periodic, m);
+            errors += run_case(Shape({8, 10, 12, 3, 2}), Shape({2, 2, 2, 1, 1}), IntVector({1, 1, 1, 0, 0}), periodic, m);
+            errors += run_case(Shape({9, 12, 12, 3, 2}), Shape({1, 3, 2, 1, 1}), IntVector({0, 2, 1, 0, 0}), periodic, m);
+        }
     }
     // reverse exchange with SUM: transfers and pack + unpack leave the same tensors
     {

@@ -435,3 +435,48 @@ def test_zero_width_is_noop():
                                        None) == -1
     torch.cuda.synchronize()
     assert (t == 1).all()
+
+
+@pytest.mark.parametrize("periodic", [False, True])
+@pytest.mark.parametrize("shape,locale,overlap", [((10, 8, 6, 2, 1), (2, 2, 2, 1, 1), (1, 2, 1, 0, 0)),
+                                                  ((12, 9, 4, 3), (3, 2, 1, 1), (2, 1, 0, 0)),
+                                                  ((130, 6, 5, 2), (2, 1, 1, 1), (1, 0, 0, 0))])
+def test_batched_clear_and_clearing_only_what_the_exchange_leaves(shape, locale, overlap, periodic):
+    """clear_halos() (one batched call for all ranks, dimensions and sides) equals
+    clear_halo(dim) rank by rank; and clear_halos(only_unfilled=True) followed by a
+    full-width exchange leaves every tensor - corners and the halos at the edge of a
+    non-periodic grid included - bit for bit as clearing everything and then
+    exchanging, from halos poisoned with different values on every rank."""
+    import torch
+    from dihydrogen_amd.layers import HaloExchangeVirtual
+    from dihydrogen_amd.tensor import Distribution, LocaleVirtual, Tensor
+    n = int(np.prod(locale))
+    dist = Distribution.make_overlapped_distribution(locale, overlap)
+    rng = np.random.default_rng(3)
+
+    def make():
+        ts = [Tensor(shape, LocaleVirtual(r, n), dist).allocate() for r in range(n)]
+        g = np.random.default_rng(11)
+        for t in ts:
+            t.real_view().copy_(torch.from_numpy(g.uniform(1, 2, tuple(t.real_view().shape)).astype(np.float32)))
+        return ts
+
+    a, b = make(), make()
+    xa, xb = HaloExchangeVirtual(a, periodic=periodic), HaloExchangeVirtual(b, periodic=periodic)
+    for d in range(len(shape)):
+        xa.clear_halo(d)
+    xb.clear_halos()
+    torch.cuda.synchronize()
+    for ta, tb in zip(a, b):
+        assert torch.equal(ta.real_view(), tb.real_view())
+    # the reference's sequence against the shortened one
+    c, d_ = make(), make()
+    xc, xd = HaloExchangeVirtual(c, periodic=periodic), HaloExchangeVirtual(d_, periodic=periodic)
+    xc.clear_halos()
+    xc.exchange()
+    xd.clear_halos(only_unfilled=True)
+    xd.exchange()
+    torch.cuda.synchronize()
+    for tc, td in zip(c, d_):
+        assert torch.equal(tc.real_view(), td.real_view())
+    del rng
