@@ -273,29 +273,107 @@ __global__ __launch_bounds__(kBlockSize) void reduce_inner_kernel(const ReduceAr
     }
     block_sum<1>(acc, lds);
     if (threadIdx.x == 0)
-        a.partials[static_cast<size_t>(k) * a.groups + g] = acc[0];
+    {
+        if (a.groups == 1) // the only group of its output: no finishing launch
+        {
+            int64_t dst_off;
+            chain(k, a.num_kept, a.kept_div, a.kept_src, a.kept_dst, &dst_off);
+            T* p = reinterpret_cast<T*>(a.dst) + dst_off;
+            *p = *p + static_cast<T>(acc[0]);
+        }
+        else
+        {
+            a.partials[static_cast<size_t>(k) * a.groups + g] = acc[0];
+        }
+    }
 }
 
-// The innermost dimension is kept: a thread adds one group of its own output
-// element's addends; neighbouring threads own neighbouring outputs.
-template <typename T>
+// The innermost dimension is kept: a thread adds one group of the addends of its
+// own VEC neighbouring output elements (VEC > 1: the innermost kept dimension is
+// contiguous in source and destination and a multiple of VEC long); neighbouring
+// threads own neighbouring outputs.
+template <typename T, int VEC>
 __global__ __launch_bounds__(kBlockSize) void reduce_outer_kernel(const ReduceArgs a)
 {
-    const uint32_t k = blockIdx.x * kBlockSize + threadIdx.x, g = blockIdx.y;
+    typedef T Vec __attribute__((ext_vector_type(VEC), aligned(sizeof(T))));
+    const uint32_t k = (blockIdx.x * kBlockSize + threadIdx.x) * VEC, g = blockIdx.y;
     if (k >= a.kept_count)
         return;
+    int64_t dst_off;
     const T* src = reinterpret_cast<const T*>(a.src)
-                   + chain(k, a.num_kept, a.kept_div, a.kept_src, nullptr, nullptr);
+                   + chain(k, a.num_kept, a.kept_div, a.kept_src, a.kept_dst, &dst_off);
     const uint32_t begin = g * a.chunk;
     const uint32_t end = begin + a.chunk < a.red_count ? begin + a.chunk : a.red_count;
-    double acc = 0.0;
+    double acc[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j)
+        acc[j] = 0.0;
     for (uint32_t r = begin; r < end; ++r)
     {
-        const double x = static_cast<double>(
-            src[chain(r, a.num_reduced, a.red_div, a.red_src, nullptr, nullptr)]);
-        acc += a.square ? x * x : x;
+        const Vec v = *reinterpret_cast<const Vec*>(
+            src + chain(r, a.num_reduced, a.red_div, a.red_src, nullptr, nullptr));
+#pragma unroll
+        for (int j = 0; j < VEC; ++j)
+        {
+            const double x = static_cast<double>(v[j]);
+            acc[j] += a.square ? x * x : x;
+        }
     }
-    a.partials[static_cast<size_t>(g) * a.kept_count + k] = acc;
+    if (a.groups == 1) // the only group of its outputs: no finishing launch
+    {
+        Vec* p = reinterpret_cast<Vec*>(reinterpret_cast<T*>(a.dst) + dst_off);
+        Vec d = *p;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j)
+            d[j] = d[j] + static_cast<T>(acc[j]);
+        *p = d;
+    }
+    else
+    {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j)
+            a.partials[static_cast<size_t>(g) * a.kept_count + k + j] = acc[j];
+    }
+}
+
+// The innermost dimension is reduced and an output element has few addends (at
+// most 64 loads of VEC): `lanes` neighbouring lanes of a wave (a power of two)
+// share an output, each loads its vectors, and the lanes are combined by
+// exchanges at distance lanes/2, ..., 1 - a fixed order.  One group per output.
+template <typename T, int VEC>
+__global__ __launch_bounds__(kBlockSize) void reduce_inner_small_kernel(const ReduceArgs a, uint32_t lanes)
+{
+    typedef T Vec __attribute__((ext_vector_type(VEC), aligned(sizeof(T))));
+    const uint64_t t = static_cast<uint64_t>(blockIdx.x) * kBlockSize + threadIdx.x;
+    const uint64_t k64 = t / lanes;
+    const uint32_t lane = static_cast<uint32_t>(t - k64 * lanes);
+    const bool valid = k64 < a.kept_count;
+    const uint32_t k = valid ? static_cast<uint32_t>(k64) : 0;
+    double acc = 0.0;
+    int64_t dst_off = 0;
+    if (valid)
+    {
+        const T* src = reinterpret_cast<const T*>(a.src)
+                       + chain(k, a.num_kept, a.kept_div, a.kept_src, a.kept_dst, &dst_off);
+        for (uint32_t r = lane * VEC; r < a.red_count; r += lanes * VEC)
+        {
+            const Vec v = *reinterpret_cast<const Vec*>(
+                src + chain(r, a.num_reduced, a.red_div, a.red_src, nullptr, nullptr));
+#pragma unroll
+            for (int j = 0; j < VEC; ++j)
+            {
+                const double x = static_cast<double>(v[j]);
+                acc += a.square ? x * x : x;
+            }
+        }
+    }
+    for (uint32_t d = lanes / 2; d >= 1; d /= 2)
+        acc += __shfl_xor(acc, static_cast<int>(d), kWaveSize);
+    if (valid && lane == 0)
+    {
+        T* p = reinterpret_cast<T*>(a.dst) + dst_off;
+        *p = *p + static_cast<T>(acc);
+    }
 }
 
 // dst[k] += sum over the groups, in group order: a thread per output element.
@@ -392,6 +470,8 @@ struct ReducePlan
     ReduceArgs args;
     bool inner = false; // the innermost dimension with more than one element is reduced
     int vec = 1;        // elements per load of the inner reduction (a multiple divides every group)
+    int outer_vec = 1;  // neighbouring outputs per thread of the outer reduction
+    uint32_t small_lanes = 0; // > 0: inner reduction with few addends, this many lanes per output
     bool empty = false; // nothing to add
 };
 
@@ -487,6 +567,22 @@ int plan_reduce(const h2x_tensor_geometry* src, const h2x_tensor_geometry* dst, 
     a.groups = static_cast<uint32_t>((red + a.chunk - 1) / std::max<uint32_t>(a.chunk, 1));
     if (a.groups == 0)
         a.groups = 1;
+    // few addends per output: lanes of a wave share an output instead of a workgroup
+    plan->small_lanes = 0;
+    if (plan->inner && red <= 64ull * plan->vec)
+    {
+        uint32_t lanes = 1;
+        while (static_cast<uint64_t>(lanes) * plan->vec < red)
+            lanes *= 2;
+        plan->small_lanes = lanes;
+        a.chunk = static_cast<uint32_t>(red);
+        a.groups = 1;
+    }
+    // outer reduction: 16-byte vectors of neighbouring outputs
+    plan->outer_vec = 1;
+    if (!plan->inner && a.num_kept > 0 && a.kept_src[0] == 1 && a.kept_dst[0] == 1
+        && kept_extent[0] % max_vec == 0)
+        plan->outer_vec = max_vec;
     return H2X_SUCCESS;
 }
 
@@ -494,19 +590,40 @@ template <typename T>
 int reduce_typed(const ReducePlan& plan, hipStream_t stream)
 {
     const ReduceArgs& a = plan.args;
+    constexpr int kVec = 16 / sizeof(T);
     const unsigned int kept_blocks = (a.kept_count + kBlockSize - 1) / kBlockSize;
+    if (plan.small_lanes > 0)
+    {
+        const uint64_t threads = static_cast<uint64_t>(a.kept_count) * plan.small_lanes;
+        const uint64_t blocks = (threads + kBlockSize - 1) / kBlockSize;
+        if (blocks > 0x7fffffffull)
+            return H2X_ERR_TOO_LARGE;
+        if (plan.vec == kVec)
+            reduce_inner_small_kernel<T, kVec><<<static_cast<unsigned int>(blocks), kBlockSize, 0, stream>>>(
+                a, plan.small_lanes);
+        else
+            reduce_inner_small_kernel<T, 1><<<static_cast<unsigned int>(blocks), kBlockSize, 0, stream>>>(
+                a, plan.small_lanes);
+        return launch_status();
+    }
     if (plan.inner)
     {
-        constexpr int kVec = 16 / sizeof(T);
         if (plan.vec == kVec)
             reduce_inner_kernel<T, kVec><<<dim3(a.kept_count, a.groups), kBlockSize, 0, stream>>>(a);
         else
             reduce_inner_kernel<T, 1><<<dim3(a.kept_count, a.groups), kBlockSize, 0, stream>>>(a);
     }
+    else if (plan.outer_vec == kVec)
+    {
+        const unsigned int blocks = (a.kept_count / kVec + kBlockSize - 1) / kBlockSize;
+        reduce_outer_kernel<T, kVec><<<dim3(blocks, a.groups), kBlockSize, 0, stream>>>(a);
+    }
     else
     {
-        reduce_outer_kernel<T><<<dim3(kept_blocks, a.groups), kBlockSize, 0, stream>>>(a);
+        reduce_outer_kernel<T, 1><<<dim3(kept_blocks, a.groups), kBlockSize, 0, stream>>>(a);
     }
+    if (a.groups == 1)
+        return launch_status(); // the reduction kernel has accumulated into the destination itself
     if (a.groups >= 16 && a.kept_count <= 4096)
         reduce_finish_wide_kernel<T><<<a.kept_count, kBlockSize, 0, stream>>>(a, plan.inner ? 1 : 0);
     else

@@ -132,6 +132,13 @@ REDUCE_CASES = [
     ((6, 5, 2000), (0, 0, 3), (1, 2)),
     ((2, 3, 4, 6, 8), (0, 0, 1, 1, 1), (0, 2, 3, 4)),   # rows of whole 16-byte vectors that start on any element
     ((2, 3, 1100, 4), (0, 0, 1, 1), (0, 2, 3)),         # more than one group per output, groups of whole vectors
+    ((3, 5, 6, 64), (0, 0, 0, 0), (3,)),                # few addends per output: lanes of a wave share an output
+    ((3, 5, 6, 64), (0, 0, 1, 2), (3,)),
+    ((2, 3, 7, 9), (0, 0, 0, 1), (2, 3)),               # 63 addends in two reduced dimensions, no vectors
+    ((4, 3, 5, 1), (0, 0, 0, 0), (3,)),                 # a single addend
+    ((6, 4, 5, 64), (0, 0, 0, 0), (0,)),                # innermost kept: vectors of neighbouring outputs
+    ((6, 4, 5, 64), (0, 0, 1, 1), (0, 1)),
+    ((40, 3, 5, 8), (0, 0, 0, 2), (0, 2)),
 ]
 
 
