@@ -324,3 +324,25 @@ def test_haloed_tensors_match_oracle(case, oracle_mod):
         # halo cells are never written
         for t in (y, dx):
             assert int(torch.isnan(t.real_view()).sum()) == t.get_local_real_size() - t.get_local_size()
+
+
+def test_non_finite_inputs_propagate_as_in_the_oracle(oracle_mod):
+    """A NaN, an infinity, values near the float32 maximum (whose squares overflow
+    float32 but not the float64 accumulators) and denormals, each in a channel of
+    its own: NaNs and infinities come out in the same places as the oracle's, the
+    finite outputs within the tolerance; the untouched channels are unaffected."""
+    shape = (3, 6, 10, 12)
+    x, dy, scale, bias = bn_inputs(shape, seed=77)
+    x[1, 0, 3, 4] = np.nan
+    x[2, 1, 0, 0] = np.inf
+    x[:, 2] *= np.float32(1e38)          # sums of squares beyond the float32 range
+    x[:, 3] *= np.float32(1e-42)         # denormal inputs
+    x[0, 4, 5, 5] = -np.inf
+    bn, xin, yout, mean, var, rm, rv = _run_forward(x, scale, bias)
+    with np.errstate(all="ignore"):
+        y_o, mean_o, var_o = oracle_mod.bn_forward(x, scale, bias, np.zeros(6, np.float32), np.ones(6, np.float32),
+                                                   1e-5, 0.9)
+    assert_nan_parity(mean.cpu().numpy(), mean_o, "mean")
+    assert_nan_parity(var.cpu().numpy(), var_o, "var")
+    assert_nan_parity(yout.real_view().cpu().numpy(), y_o, "y")
+    assert np.isfinite(y_o[:, 5]).all() and np.isfinite(y_o[:, 3]).all()   # the test has teeth: finite channels exist
