@@ -237,3 +237,30 @@ def test_instance_forward_in_four_passes_equals_the_staged_calls(shape, dtype):
         outs.append([t.cpu().numpy() for t in (y, mx, ex)])
     for name, a, b in zip(("y", "sample_max", "sample_exp"), *outs):
         assert np.array_equal(a, b), name
+
+
+@pytest.mark.parametrize("shape", [(2, 21, 8, 8), (1, 200, 4, 4)])
+def test_non_finite_logits_propagate_as_in_the_oracle(shape, oracle_mod):
+    """A NaN, +inf and -inf logit, each at a pixel of its own, in the register kernel and
+    in the kernel that shares channels between waves: NaNs at the same positions as the
+    oracle's, the finite outputs within the tolerance, the other pixels unaffected."""
+    import torch
+    from dihydrogen_amd.layers import Softmax, SoftmaxMode
+    rng = np.random.default_rng(41)
+    x = (2.0 * rng.standard_normal(shape)).astype(np.float32)
+    x[0, 3, 1, 1] = np.nan
+    x[0, 5, 2, 2] = np.inf
+    x[0, 7, 3, 3] = -np.inf
+    mk = _tensors(shape)
+    xt, yt = mk(), mk()
+    xt.real_view().copy_(torch.from_numpy(x))
+    sm = Softmax()
+    sm.setup(xt, SoftmaxMode.CHANNEL)
+    assert sm.forward(xt, yt) == 0
+    torch.cuda.synchronize()
+    y = yt.real_view().cpu().numpy()
+    with np.errstate(all="ignore"):
+        y_o = oracle_mod.softmax_channel_forward(x)
+    assert np.array_equal(np.isnan(y), np.isnan(y_o))
+    ok = np.isfinite(y_o)
+    assert ok.sum() > y.size // 2 and max_rel(y[ok], y_o[ok]) <= TOL
