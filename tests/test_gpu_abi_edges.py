@@ -23,7 +23,10 @@ def _ptr(t, offset_elems=0):
 
 
 @pytest.mark.parametrize("offset", [0, 1, 2, 3])
-@pytest.mark.parametrize("spatial,real", [(37, 41), (64, 64), (64, 68), (5, 9)])
+@pytest.mark.parametrize("spatial,real", [(37, 41), (64, 64), (64, 68), (5, 9),
+                                          # long segments that are no multiple of 4 long or start off a 16-byte
+                                          # boundary: unaligned vectors, single elements at the end of a segment
+                                          (1027, 1031), (1028, 1028), (1030, 1040), (1025, 1025)])
 def test_bn_dense_unaligned_padded(offset, spatial, real, oracle_mod):
     import torch
     from dihydrogen_amd import capi

@@ -28,6 +28,10 @@ CASES = [
     (32, 8, 3, 3),          # short odd segments, folded, scalar
     (48, 40, 4, 4),         # short segments, folded, vector width 4
     (6, 5, 2, 7, 9),        # 5-D, 126 elements per segment
+    (3, 20, 37, 37),        # long odd segments (1369 = 4 * 342 + 1): unaligned vectors and single elements at the end
+    (1, 6, 19, 19),         # one sample, 361 elements
+    (2, 5, 11, 11, 11),     # 1331 = 4 * 332 + 3
+    (2, 4, 33, 34),         # 1122 = 4 * 280 + 2
 ]
 
 
