@@ -131,7 +131,7 @@ struct TensorMap
 };
 
 template <bool STRIDED>
-__device__ __forceinline__ size_t seg_offset(const TensorMap& m, size_t i)
+__device__ __forceinline__ size_t seg_offset(const TensorMap& m, size_t i, uint32_t* in_row = nullptr)
 {
     if constexpr (!STRIDED)
     {
@@ -143,6 +143,8 @@ __device__ __forceinline__ size_t seg_offset(const TensorMap& m, size_t i)
         const uint32_t x = static_cast<uint32_t>(i) - t * m.w.divisor;
         const uint32_t z = fastdiv(t, m.h);
         const uint32_t y = t - z * m.h.divisor;
+        if (in_row)
+            *in_row = m.w.divisor - x; // elements from i to the end of its row
         return x + y * static_cast<size_t>(m.sy) + z * static_cast<size_t>(m.sz);
     }
 }
@@ -187,6 +189,63 @@ __device__ __forceinline__ void store_vec(T* p, const T (&r)[VEC])
         for (int j = 0; j < VEC; ++j)
             t[j] = r[j];
         __builtin_nontemporal_store(t, reinterpret_cast<V*>(p));
+    }
+}
+
+// The VEC elements from interior index i on.  In the strided layout a vector may
+// run past the end of its row when rows are no multiple of VEC long (rows are at
+// least VEC long, so it touches two rows at most): its two parts are then moved
+// element by element, all other vectors whole (7 x 7 activations: 1 vector in 12).
+template <typename T, int VEC, bool STRIDED, bool STREAM = false>
+__device__ __forceinline__ void load_at(const T* p, const TensorMap& m, size_t i, T (&r)[VEC])
+{
+    if constexpr (!STRIDED || VEC == 1)
+    {
+        load_vec<T, VEC, !STRIDED, STREAM>(p + seg_offset<STRIDED>(m, i), r);
+    }
+    else
+    {
+        uint32_t in_row;
+        const size_t off = seg_offset<true>(m, i, &in_row);
+        if (in_row >= VEC)
+        {
+            load_vec<T, VEC, false, STREAM>(p + off, r);
+        }
+        else
+        {
+            const size_t next = seg_offset<true>(m, i + in_row); // the first element of the next row
+#pragma unroll
+            for (int j = 0; j < VEC; ++j)
+                r[j] = j < static_cast<int>(in_row) ? p[off + j] : p[next + j - in_row];
+        }
+    }
+}
+
+template <typename T, int VEC, bool STRIDED>
+__device__ __forceinline__ void store_at(T* p, const TensorMap& m, size_t i, const T (&r)[VEC])
+{
+    if constexpr (!STRIDED || VEC == 1)
+    {
+        store_vec<T, VEC, !STRIDED>(p + seg_offset<STRIDED>(m, i), r);
+    }
+    else
+    {
+        uint32_t in_row;
+        const size_t off = seg_offset<true>(m, i, &in_row);
+        if (in_row >= VEC)
+        {
+            store_vec<T, VEC, false>(p + off, r);
+        }
+        else
+        {
+            const size_t next = seg_offset<true>(m, i + in_row);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j)
+            {
+                const T one[1] = {r[j]};
+                store_vec<T, 1>(j < static_cast<int>(in_row) ? p + off + j : p + next + j - in_row, one);
+            }
+        }
     }
 }
 
@@ -329,8 +388,7 @@ __global__ __launch_bounds__(kBlockSize) void bn_sums_kernel(
             T v[kUnroll][VEC];
 #pragma unroll
             for (int u = 0; u < kUnroll; ++u)
-                load_vec<T, VEC, !STRIDED>(
-                    p + seg_offset<STRIDED>(mx, tile + u * kStride + threadIdx.x * VEC), v[u]);
+                load_at<T, VEC, STRIDED>(p, mx, tile + u * kStride + threadIdx.x * VEC, v[u]);
 #pragma unroll
             for (int u = 0; u < kUnroll; ++u)
 #pragma unroll
@@ -340,7 +398,7 @@ __global__ __launch_bounds__(kBlockSize) void bn_sums_kernel(
         for (size_t i = tile + threadIdx.x * VEC; i + VEC <= end; i += kStride)
         {
             T v[VEC];
-            load_vec<T, VEC, !STRIDED>(p + seg_offset<STRIDED>(mx, i), v);
+            load_at<T, VEC, STRIDED>(p, mx, i, v);
 #pragma unroll
             for (int j = 0; j < VEC; ++j)
                 accumulate(v[j]);
@@ -462,26 +520,24 @@ __global__ __launch_bounds__(kBlockSize) void bn_apply_kernel(
         T v[kUnroll][VEC];
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u)
-            load_vec<T, VEC, !STRIDED>(
-                xp + seg_offset<STRIDED>(mx, tile + u * kStride + threadIdx.x * VEC), v[u]);
+            load_at<T, VEC, STRIDED>(xp, mx, tile + u * kStride + threadIdx.x * VEC, v[u]);
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u)
         {
 #pragma unroll
             for (int j = 0; j < VEC; ++j)
                 v[u][j] = fma_t((v[u][j] - m) * inv_stdev, sc, bi);
-            store_vec<T, VEC, !STRIDED>(
-                yp + seg_offset<STRIDED>(my, tile + u * kStride + threadIdx.x * VEC), v[u]);
+            store_at<T, VEC, STRIDED>(yp, my, tile + u * kStride + threadIdx.x * VEC, v[u]);
         }
     }
     for (size_t i = tile + threadIdx.x * VEC; i + VEC <= end; i += kStride)
     {
         T v[VEC];
-        load_vec<T, VEC, !STRIDED>(xp + seg_offset<STRIDED>(mx, i), v);
+        load_at<T, VEC, STRIDED>(xp, mx, i, v);
 #pragma unroll
         for (int j = 0; j < VEC; ++j)
             v[j] = fma_t((v[j] - m) * inv_stdev, sc, bi);
-        store_vec<T, VEC, !STRIDED>(yp + seg_offset<STRIDED>(my, i), v);
+        store_at<T, VEC, STRIDED>(yp, my, i, v);
     }
     if constexpr (VEC > 1)
     {
@@ -548,8 +604,8 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop1_kernel(
             for (int u = 0; u < kUnroll2; ++u)
             {
                 const size_t i = tile + u * kStride + threadIdx.x * VEC;
-                load_vec<T, VEC, !STRIDED>(xp + seg_offset<STRIDED>(mx, i), xv[u]);
-                load_vec<T, VEC, !STRIDED, true>(dp + seg_offset<STRIDED>(md, i), dv[u]);
+                load_at<T, VEC, STRIDED>(xp, mx, i, xv[u]);
+                load_at<T, VEC, STRIDED, true>(dp, md, i, dv[u]);
             }
 #pragma unroll
             for (int u = 0; u < kUnroll2; ++u)
@@ -560,8 +616,8 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop1_kernel(
         for (size_t i = tile + threadIdx.x * VEC; i + VEC <= end; i += kStride)
         {
             T xv[VEC], dv[VEC];
-            load_vec<T, VEC, !STRIDED>(xp + seg_offset<STRIDED>(mx, i), xv);
-            load_vec<T, VEC, !STRIDED, true>(dp + seg_offset<STRIDED>(md, i), dv);
+            load_at<T, VEC, STRIDED>(xp, mx, i, xv);
+            load_at<T, VEC, STRIDED, true>(dp, md, i, dv);
 #pragma unroll
             for (int j = 0; j < VEC; ++j)
                 accumulate(xv[j], dv[j]);
@@ -647,8 +703,8 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop2_kernel(
         for (int u = 0; u < kUnroll2; ++u)
         {
             const size_t i = tile + u * kStride + threadIdx.x * VEC;
-            load_vec<T, VEC, !STRIDED>(xp + seg_offset<STRIDED>(mx, i), xv[u]);
-            load_vec<T, VEC, !STRIDED, true>(dp + seg_offset<STRIDED>(md, i), dv[u]);
+            load_at<T, VEC, STRIDED>(xp, mx, i, xv[u]);
+            load_at<T, VEC, STRIDED, true>(dp, md, i, dv[u]);
         }
 #pragma unroll
         for (int u = 0; u < kUnroll2; ++u)
@@ -659,22 +715,21 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop2_kernel(
                 T r = fma_t(dv[u][j] * sc, inv_stdev, dmean_term);
                 xv[u][j] = fma_t(xv[u][j] - m, dvar_term, r);
             }
-            store_vec<T, VEC, !STRIDED>(
-                op + seg_offset<STRIDED>(mo, tile + u * kStride + threadIdx.x * VEC), xv[u]);
+            store_at<T, VEC, STRIDED>(op, mo, tile + u * kStride + threadIdx.x * VEC, xv[u]);
         }
     }
     for (size_t i = tile + threadIdx.x * VEC; i + VEC <= end; i += kStride)
     {
         T xv[VEC], dv[VEC];
-        load_vec<T, VEC, !STRIDED>(xp + seg_offset<STRIDED>(mx, i), xv);
-        load_vec<T, VEC, !STRIDED, true>(dp + seg_offset<STRIDED>(md, i), dv);
+        load_at<T, VEC, STRIDED>(xp, mx, i, xv);
+        load_at<T, VEC, STRIDED, true>(dp, md, i, dv);
 #pragma unroll
         for (int j = 0; j < VEC; ++j)
         {
             T r = fma_t(dv[j] * sc, inv_stdev, dmean_term);
             xv[j] = fma_t(xv[j] - m, dvar_term, r);
         }
-        store_vec<T, VEC, !STRIDED>(op + seg_offset<STRIDED>(mo, i), xv);
+        store_at<T, VEC, STRIDED>(op, mo, i, xv);
     }
     if constexpr (VEC > 1)
     {
@@ -797,6 +852,7 @@ int strided_tensor(const h2x_tensor_geometry* g, const void* p, int num_samples,
 // tensor with the index itself, use vectors aligned to one element, and finish the
 // last few elements of a segment one by one (N 16, C 64, 57 x 57: forward 23 -> 15 us).
 constexpr size_t kMinUnalignedSegment = 256;
+constexpr size_t kMinRaggedRow = 64;
 
 template <typename T>
 int common_vector(std::initializer_list<const HostTensor*> ts, bool* strided)
@@ -822,10 +878,13 @@ int common_vector(std::initializer_list<const HostTensor*> ts, bool* strided)
         *strided = true;
         return full;
     }
-    // rows of a strided tensor must hold whole vectors; dense tensors in a strided
-    // launch are addressed with i itself, so rows do not matter for them
+    // Rows of a strided tensor hold whole vectors, or are long enough for the vectors that run
+    // past the end of a row (and are split in two, element by element) to be few: with rows
+    // of 49 elements every wave has some and the gain is gone (N 256, C 2048, 7 x 7: forward
+    // 102 -> 110 us), with 169 and 729 it is a third (N 32, C 256, 27 x 27: 30 -> 19 us).
+    // Dense tensors in a strided launch are addressed with i itself: rows do not matter.
     for (const HostTensor* t : ts)
-        if (t->strided && t->row % full != 0)
+        if (t->strided && t->row % full != 0 && t->row < kMinRaggedRow)
             return 1;
     return full;
 }

@@ -32,6 +32,9 @@ CASES = [
     (1, 6, 19, 19),         # one sample, 361 elements
     (2, 5, 11, 11, 11),     # 1331 = 4 * 332 + 3
     (2, 4, 33, 34),         # 1122 = 4 * 280 + 2
+    (5, 6, 27, 27),         # folded rows of 729: vectors that cross a row end are split
+    (6, 3, 13, 13),         # folded rows of 169
+    (3, 4, 5, 13),          # folded rows of 65, just above the limit for split vectors
 ]
 
 
@@ -278,6 +281,8 @@ HALO_CASES = [
     ((16, 8, 12, 4, 2), (2, 1, 2, 1, 1), (1, 0, 2, 0, 0)),
     ((8, 8, 8, 3, 2), (2, 2, 2, 1, 1), (1, 1, 1, 0, 0)),
     ((16, 8, 6, 2), (1, 2, 1, 1), (0, 3, 0, 0)),        # halo only on the outermost spatial dimension: dense path
+    ((134, 6, 3, 2), (2, 2, 1, 1), (1, 1, 0, 0)),       # haloed rows of 67 elements: vectors split at row ends
+    ((130, 4, 6, 2, 2), (2, 1, 2, 1, 1), (2, 0, 1, 0, 0)),  # 5-D, rows of 65
 ]
 
 
