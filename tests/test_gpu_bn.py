@@ -35,6 +35,16 @@ CASES = [
     (5, 6, 27, 27),         # folded rows of 729: vectors that cross a row end are split
     (6, 3, 13, 13),         # folded rows of 169
     (3, 4, 5, 13),          # folded rows of 65, just above the limit for split vectors
+    # short segments: a workgroup serves a window of whole channels
+    (5, 300, 7, 7),         # 19 channels a window, the last window partly filled, last slot of 1 element
+    (3, 70, 14, 14),        # 196 elements: whole vectors only
+    (7, 33, 16, 16),        # 256 elements, the longest short segment: 4 channels a window
+    (9, 260, 1, 1),         # one element per segment, two windows
+    (130, 12, 2, 1),        # two elements per segment
+    (2, 9, 3, 5, 17),       # 255 elements: last slot of 3
+    (512, 600, 1, 1),       # few windows, many samples: four rows of lanes share a workgroup's samples
+    (300, 500, 3, 3),       # the same with three slots a segment
+    (37, 2, 3, 3, 3),       # 27 elements, two channels, one workgroup a range of samples
 ]
 
 
@@ -131,7 +141,8 @@ def test_backward_matches_oracle(shape, oracle_mod):
 
 @pytest.mark.parametrize("dtype", ["float32", "float64"])
 @pytest.mark.parametrize("shape", [(8, 64, 56, 56), (2, 3, 4, 5), (3, 5, 7, 9, 11), (64, 32, 7, 7), (1, 1, 1, 1),
-                                   (2, 4, 40, 40, 40), (1, 300, 3, 3), (3, 20, 37, 37), (2, 16, 8, 16, 16), (1, 24, 2, 1024)])
+                                   (2, 4, 40, 40, 40), (1, 300, 3, 3), (3, 20, 37, 37), (2, 16, 8, 16, 16), (1, 24, 2, 1024),
+                                   (40, 300, 7, 7), (512, 600, 1, 1), (6, 9, 3, 5, 17), (33, 70, 14, 14)])
 def test_two_launch_forward_and_backward_equal_the_staged_calls(shape, dtype):
     """forward()/backward() of a single rank finish the channel sums inside the
     normalising / input-gradient kernel (h2x_bn_forward_local, _backward_local);
@@ -172,12 +183,12 @@ def test_two_launch_forward_and_backward_equal_the_staged_calls(shape, dtype):
         assert np.array_equal(a, b, equal_nan=True), name
 
 
-def test_backprop2_in_place(oracle_mod):
+@pytest.mark.parametrize("shape", [(2, 6, 8, 12), (9, 45, 7, 7)])
+def test_backprop2_in_place(shape, oracle_mod):
     """dx may alias x (legacy/src/dnn_backend/batchnorm.cu:1303-1314)."""
     import torch
     from dihydrogen_amd.tensor import Distribution, LocaleVirtual, Tensor
 
-    shape = (2, 6, 8, 12)
     x, dy, scale, bias = bn_inputs(shape, seed=7)
     bn, xin, yout, mean, var, rm, rv = _run_forward(x, scale, bias)
     dist = Distribution.make_localized_distribution(4)
@@ -221,11 +232,11 @@ def test_deterministic_and_workspace_reuse():
     assert max_rel(results[0][0], s64.astype(np.float32)) <= 1e-6
 
 
-def test_float64(oracle_mod):
-    shape = (2, 5, 6, 10)
+@pytest.mark.parametrize("shape", [(2, 5, 6, 10), (12, 50, 7, 7), (6, 7, 3, 5, 17)])
+def test_float64(shape, oracle_mod):
     x, dy, scale, bias = bn_inputs(shape, seed=5, dtype=np.float64)
     bn, xin, yout, mean, var, rm, rv = _run_forward(x, scale, bias, dtype="float64")
-    rm_o, rv_o = np.zeros(5), np.ones(5)
+    rm_o, rv_o = np.zeros(shape[1]), np.ones(shape[1])
     y_o, mean_o, var_o = oracle_mod.bn_forward(x, scale, bias, rm_o, rv_o, 1e-5, 0.9)
     assert max_rel(mean.cpu().numpy(), mean_o) <= 1e-10
     assert max_rel(var.cpu().numpy(), var_o) <= 1e-10
