@@ -381,21 +381,21 @@ def cpu_baseline(repeats: int = 5):
 # TCC_EA0_WRREQ_64B), request counts summed over the L2 channels, per dispatch.
 # label -> (bytes read, bytes written) per launch
 PMC_TRAFFIC = {
-    "bn_sums": (268460032, 131072),
-    "bn_apply": (268466688, 268487808),
-    "bn_backprop1": (536914816, 131072),
-    "bn_backprop2": (536907264, 268435456),
-    "halo_dim0_pack": (149642272, 8652800),    # 4 faces (2 ranks) a launch, four launches a step
-    "halo_dim0_unpack": (9220144, 43264000),
+    "bn_sums": (268452864, 131072),
+    "bn_apply": (268466688, 268480896),
+    "bn_backprop1": (536914688, 131072),
+    "bn_backprop2": (536904192, 268435456),
+    "halo_dim0_pack": (149674720, 8652800),    # 4 faces (2 ranks) a launch, four launches a step
+    "halo_dim0_unpack": (9219456, 43264000),
     "halo_dim1_pack": (42624768, 34611200),
-    "halo_dim1_unpack": (34637568, 36217216),
+    "halo_dim1_unpack": (34637568, 36217024),
     "halo_dim2_pack": (34694400, 34611200),
-    "halo_dim2_unpack": (34637568, 34619456),
+    "halo_dim2_unpack": (34637568, 34619392),
 }
 # sha256 (first 16 hex digits) of the kernel sources the table was measured with, see
 # kernel_sources_sha(); with other sources the traffic fields are omitted
-PMC_SOURCES_SHA = "a1591ced7145abb1"
-PMC_COMMIT = "167563f"
+PMC_SOURCES_SHA = "b8e0337f723a8f20"
+PMC_COMMIT = "e8f8648"
 
 KERNEL_OF = {
     "bn_sums": "bn_sums_kernel<float,4> (+bn_finish_kernel<float,2>)",
@@ -764,6 +764,12 @@ def main() -> int:
         breakdown["C3_bn3d_haloed_fwd_bwd"] = entry(8 * bn3h.elems * 4, bn3h.elems,
                                                     lambda: (bn3h.forward(), bn3h.backward()), inner=2)
         del bn3h
+        torch.cuda.empty_cache()
+        # short segments (the last stage of a ResNet): a workgroup serves a window of whole channels
+        bn7 = BatchNormWorkload((256, 2048, 7, 7), SEED + 7)
+        breakdown["bn2d_7x7_N256_C2048_fwd"] = entry(3 * bn7.elems * 4, bn7.elems, bn7.forward)
+        breakdown["bn2d_7x7_N256_C2048_bwd"] = entry(5 * bn7.elems * 4, bn7.elems, bn7.backward)
+        del bn7
         torch.cuda.empty_cache()
         # configs 1 and 4 fit in the memory-side cache: warm = back to back, cold = after a 512 MB read
         evict = torch.empty(1 << 27, device="cuda").fill_(1.0)
