@@ -7,8 +7,11 @@
 // so x (or y and dy) is read from HBM exactly once with fully coalesced
 // 4*VEC-byte accesses and no LDS staging; the reference stages a
 // C x 256 tile in LDS and walks it three times
-// (legacy/src/dnn_backend/softmax.cu:538-593,621-669).  Channel counts beyond
-// the largest register tile fall back to a kernel that re-reads its inputs.
+// (legacy/src/dnn_backend/softmax.cu:538-593,621-669).  Above 32 channels the
+// four waves of a workgroup share the channels of 64 * VEC pixels, still in
+// registers; channel counts beyond the largest such tile fall back to a kernel
+// that re-reads its inputs; tensors with one pixel per sample have a kernel
+// that puts the channels, which are contiguous then, on the lanes of a wave.
 #include "h2x_device.hpp"
 
 #include <cfloat>
@@ -294,6 +297,264 @@ __global__ __launch_bounds__(kBlockSize) void softmax_bwd_wide_kernel(
         }
 }
 
+// forward, up to 4 * CPW channels, register-resident.  A workgroup serves
+// 64 * VEC neighbouring pixels; its four waves share the channels (wave g takes
+// c = g, g + 4, ...: CPW of them at most) and keep their values in registers, so
+// x is read once; maxima and sums are combined through LDS in wave order.  The
+// arithmetic, partial sums included, is that of softmax_fwd_wide_kernel, which
+// re-reads its tile twice and whose tiles of 64 * C elements the L2 does not
+// hold once every CU runs eight of them (N 16, C 150, 128 x 128: 100 us there,
+// 60 us with the tile in registers).
+template <typename T, int VEC, int CPW>
+__global__ __launch_bounds__(kBlockSize) void softmax_fwd_split_kernel(
+    const T* __restrict__ x, T* __restrict__ y, int num_channels, size_t spatial)
+{
+    using P = Pack<T, VEC>;
+    __shared__ T lds[kWavesPerBlock][kWaveSize * VEC];
+    const int lane = threadIdx.x % kWaveSize;
+    const int g = threadIdx.x / kWaveSize;
+    const size_t s =
+        (static_cast<size_t>(xcd_contiguous(blockIdx.x, gridDim.x)) * kWaveSize + lane) * VEC;
+    const bool active = s < spatial;
+    const size_t base = static_cast<size_t>(blockIdx.y) * num_channels * spatial + (active ? s : 0);
+    const T* xp = x + base;
+    T* yp = y + base;
+    constexpr T kMin = Limits<T>::min_normal;
+
+    P v[CPW];
+    T mx[VEC], sum[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j)
+    {
+        mx[j] = kMin;
+        sum[j] = T(0);
+    }
+    if (active)
+    {
+#pragma unroll
+        for (int k = 0; k < CPW; ++k)
+            if (g + k * kWavesPerBlock < num_channels)
+                v[k] = P::load(xp + static_cast<size_t>(g + k * kWavesPerBlock) * spatial);
+#pragma unroll
+        for (int k = 0; k < CPW; ++k)
+            if (g + k * kWavesPerBlock < num_channels)
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+                    mx[j] = v[k][j] > mx[j] ? v[k][j] : mx[j];
+    }
+#pragma unroll
+    for (int j = 0; j < VEC; ++j)
+        lds[g][lane * VEC + j] = mx[j];
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < VEC; ++j)
+#pragma unroll
+        for (int w = 0; w < kWavesPerBlock; ++w)
+            mx[j] = lds[w][lane * VEC + j] > mx[j] ? lds[w][lane * VEC + j] : mx[j];
+    __syncthreads();
+
+    if (active)
+    {
+#pragma unroll
+        for (int k = 0; k < CPW; ++k)
+            if (g + k * kWavesPerBlock < num_channels)
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+                {
+                    const T e = exp_t(v[k][j] - mx[j]);
+                    v[k][j] = e;
+                    sum[j] += e;
+                }
+    }
+#pragma unroll
+    for (int j = 0; j < VEC; ++j)
+        lds[g][lane * VEC + j] = sum[j];
+    __syncthreads();
+    T inv[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j)
+    {
+        T t = lds[0][lane * VEC + j];
+#pragma unroll
+        for (int w = 1; w < kWavesPerBlock; ++w)
+            t += lds[w][lane * VEC + j];
+        inv[j] = T(1) / t;
+    }
+    if (active)
+    {
+#pragma unroll
+        for (int k = 0; k < CPW; ++k)
+            if (g + k * kWavesPerBlock < num_channels)
+            {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+                {
+                    const T r = v[k][j] * inv[j];
+                    v[k][j] = r > kMin ? r : kMin;
+                }
+                P::store(yp + static_cast<size_t>(g + k * kWavesPerBlock) * spatial, v[k]);
+            }
+    }
+}
+
+// backward likewise: y and dy of up to 4 * CPW channels in registers.
+template <typename T, int VEC, int CPW>
+__global__ __launch_bounds__(kBlockSize) void softmax_bwd_split_kernel(
+    const T* __restrict__ y, const T* __restrict__ dy, T* __restrict__ dx, int num_channels,
+    size_t spatial)
+{
+    using P = Pack<T, VEC>;
+    __shared__ T lds[kWavesPerBlock][kWaveSize * VEC];
+    const int lane = threadIdx.x % kWaveSize;
+    const int g = threadIdx.x / kWaveSize;
+    const size_t s =
+        (static_cast<size_t>(xcd_contiguous(blockIdx.x, gridDim.x)) * kWaveSize + lane) * VEC;
+    const bool active = s < spatial;
+    const size_t base = static_cast<size_t>(blockIdx.y) * num_channels * spatial + (active ? s : 0);
+    const T* yp = y + base;
+    const T* gp = dy + base;
+    T* op = dx + base;
+    constexpr T kMin = Limits<T>::min_normal;
+
+    P yv[CPW], gv[CPW];
+    T dp[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j)
+        dp[j] = T(0);
+    if (active)
+    {
+#pragma unroll
+        for (int k = 0; k < CPW; ++k)
+            if (g + k * kWavesPerBlock < num_channels)
+            {
+                yv[k] = P::load(yp + static_cast<size_t>(g + k * kWavesPerBlock) * spatial);
+                gv[k] = P::load(gp + static_cast<size_t>(g + k * kWavesPerBlock) * spatial);
+            }
+#pragma unroll
+        for (int k = 0; k < CPW; ++k)
+            if (g + k * kWavesPerBlock < num_channels)
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+                    dp[j] = fma_t(yv[k][j], gv[k][j], dp[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < VEC; ++j)
+        lds[g][lane * VEC + j] = dp[j];
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < VEC; ++j)
+    {
+        T t = lds[0][lane * VEC + j];
+#pragma unroll
+        for (int w = 1; w < kWavesPerBlock; ++w)
+            t += lds[w][lane * VEC + j];
+        dp[j] = t;
+    }
+    if (active)
+    {
+#pragma unroll
+        for (int k = 0; k < CPW; ++k)
+            if (g + k * kWavesPerBlock < num_channels)
+            {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+                    yv[k][j] = yv[k][j] > kMin ? yv[k][j] * (gv[k][j] - dp[j]) : T(0);
+                P::store(op + static_cast<size_t>(g + k * kWavesPerBlock) * spatial, yv[k]);
+            }
+    }
+}
+
+// One pixel per sample (the output of a fully connected layer): the channels of
+// a sample are contiguous, so a wave takes a sample, lane l the channels l,
+// l + 64, ... (CPL of them at most), and maxima, sums and dot products are
+// combined across the lanes with a butterfly of shuffles.  The kernels above
+// would put one sample on each lane and read with a stride of C elements
+// (N 256, C 1000: 176 us).
+template <typename T>
+__device__ __forceinline__ T wave_butterfly_sum(T v)
+{
+#pragma unroll
+    for (int m = kWaveSize / 2; m >= 1; m >>= 1)
+        v += __shfl_xor(v, m, kWaveSize);
+    return v;
+}
+
+template <typename T, int CPL>
+__global__ __launch_bounds__(kBlockSize) void softmax_fwd_row_kernel(
+    const T* __restrict__ x, T* __restrict__ y, int num_channels, int num_samples)
+{
+    const int lane = threadIdx.x % kWaveSize;
+    const int n = blockIdx.x * kWavesPerBlock + threadIdx.x / kWaveSize;
+    if (n >= num_samples)
+        return;
+    const T* xp = x + static_cast<size_t>(n) * num_channels;
+    T* yp = y + static_cast<size_t>(n) * num_channels;
+    constexpr T kMin = Limits<T>::min_normal;
+    T v[CPL];
+    T mx = kMin;
+#pragma unroll
+    for (int k = 0; k < CPL; ++k)
+        if (lane + k * kWaveSize < num_channels)
+            v[k] = xp[lane + k * kWaveSize];
+#pragma unroll
+    for (int k = 0; k < CPL; ++k)
+        if (lane + k * kWaveSize < num_channels)
+            mx = v[k] > mx ? v[k] : mx;
+#pragma unroll
+    for (int m = kWaveSize / 2; m >= 1; m >>= 1)
+    {
+        const T o = __shfl_xor(mx, m, kWaveSize);
+        mx = o > mx ? o : mx;
+    }
+    T sum = T(0);
+#pragma unroll
+    for (int k = 0; k < CPL; ++k)
+        if (lane + k * kWaveSize < num_channels)
+        {
+            v[k] = exp_t(v[k] - mx);
+            sum += v[k];
+        }
+    const T inv = T(1) / wave_butterfly_sum(sum);
+#pragma unroll
+    for (int k = 0; k < CPL; ++k)
+        if (lane + k * kWaveSize < num_channels)
+        {
+            const T r = v[k] * inv;
+            yp[lane + k * kWaveSize] = r > kMin ? r : kMin;
+        }
+}
+
+template <typename T, int CPL>
+__global__ __launch_bounds__(kBlockSize) void softmax_bwd_row_kernel(
+    const T* __restrict__ y, const T* __restrict__ dy, T* __restrict__ dx, int num_channels,
+    int num_samples)
+{
+    const int lane = threadIdx.x % kWaveSize;
+    const int n = blockIdx.x * kWavesPerBlock + threadIdx.x / kWaveSize;
+    if (n >= num_samples)
+        return;
+    const size_t base = static_cast<size_t>(n) * num_channels;
+    constexpr T kMin = Limits<T>::min_normal;
+    T yv[CPL], gv[CPL];
+    T dp = T(0);
+#pragma unroll
+    for (int k = 0; k < CPL; ++k)
+        if (lane + k * kWaveSize < num_channels)
+        {
+            yv[k] = y[base + lane + k * kWaveSize];
+            gv[k] = dy[base + lane + k * kWaveSize];
+        }
+#pragma unroll
+    for (int k = 0; k < CPL; ++k)
+        if (lane + k * kWaveSize < num_channels)
+            dp = fma_t(yv[k], gv[k], dp);
+    dp = wave_butterfly_sum(dp);
+#pragma unroll
+    for (int k = 0; k < CPL; ++k)
+        if (lane + k * kWaveSize < num_channels)
+            dx[base + lane + k * kWaveSize] = yv[k] > kMin ? yv[k] * (gv[k] - dp) : T(0);
+}
+
 // Largest vector (elements) usable for all of the given pointers.
 template <typename T>
 int vector_width(size_t spatial, int want, std::initializer_list<const void*> ptrs)
@@ -326,10 +587,11 @@ dim3 pixel_grid_xcd(size_t spatial, int vec, int num_samples)
     return dim3(static_cast<unsigned int>((blocks + kNumXcd - 1) / kNumXcd * kNumXcd), num_samples);
 }
 
-// 64 pixels per workgroup, padded for xcd_contiguous.
-dim3 wide_grid(size_t spatial, int num_samples)
+// 64 * vec pixels per workgroup, padded for xcd_contiguous.
+dim3 wide_grid(size_t spatial, int vec, int num_samples)
 {
-    const size_t blocks = (spatial + kWaveSize - 1) / kWaveSize;
+    const size_t per_block = static_cast<size_t>(kWaveSize) * vec;
+    const size_t blocks = (spatial + per_block - 1) / per_block;
     return dim3(static_cast<unsigned int>((blocks + kNumXcd - 1) / kNumXcd * kNumXcd), num_samples);
 }
 
@@ -345,14 +607,56 @@ void launch_bwd(const T* y, const T* dy, T* dx, int n, int c, size_t s, hipStrea
     softmax_bwd_reg_kernel<T, VEC, CMAX><<<pixel_grid_xcd(s, VEC, n), kBlockSize, 0, st>>>(y, dy, dx, c, s);
 }
 
-// Register budget: CMAX * VEC * sizeof(T)/4 VGPRs for the forward tile, twice
-// that backward; tiles are kept at or below 128 VGPRs.
+// Which kernel serves which channel count (float; measured on MI355X).  Up to
+// 32 channels a thread keeps all channels of its pixels (softmax_*_reg_kernel:
+// config 4, 21 channels, 28 / 40 us).  Beyond, the four waves of a workgroup
+// share the channels (softmax_*_split_kernel) with the smallest register tile
+// that holds them and two pixels a lane where the geometry allows: against one
+// thread per pixel with 64 or 128 channels in registers, N 4, C 100, 256 x 256
+// takes 34 instead of 68 us forward and 53 instead of 63 us backward; against
+// the re-reading kernel N 16, C 150, 128 x 128 takes 60 instead of 100 us and 89
+// instead of 150 us, N 8, C 256, 64 x 64 18 instead of 59 us and 19 instead of
+// 55 us.  Tiles wider than needed cost time (every lane walks the whole tile
+// under a predicate), hence the steps of 16.  More channels than the largest
+// tile holds (512; double: 256) take the re-reading kernel.
+template <typename T, int VEC, int CPW>
+int launch_fwd_split(const T* x, T* y, int n, int c, size_t s, hipStream_t st)
+{
+    softmax_fwd_split_kernel<T, VEC, CPW><<<wide_grid(s, VEC, n), kBlockSize, 0, st>>>(x, y, c, s);
+    return launch_status();
+}
+
+template <typename T, int VEC, int CPW>
+int launch_bwd_split(const T* y, const T* dy, T* dx, int n, int c, size_t s, hipStream_t st)
+{
+    softmax_bwd_split_kernel<T, VEC, CPW>
+        <<<wide_grid(s, VEC, n), kBlockSize, 0, st>>>(y, dy, dx, c, s);
+    return launch_status();
+}
+
 template <typename T>
 int forward_impl(int n, int c, size_t s, const void* xv, void* yv, hipStream_t st)
 {
     const T* x = static_cast<const T*>(xv);
     T* y = static_cast<T*>(yv);
     constexpr int kWords = sizeof(T) / 4;
+    if (s == 1)
+    {
+        const unsigned int blocks = (static_cast<unsigned int>(n) + kWavesPerBlock - 1) / kWavesPerBlock;
+#define H2X_FWD_ROW(CP)                                                                            \
+    do                                                                                             \
+    {                                                                                              \
+        softmax_fwd_row_kernel<T, CP><<<blocks, kBlockSize, 0, st>>>(x, y, c, n);                   \
+        return launch_status();                                                                    \
+    } while (0)
+        if (c <= 1 * kWaveSize) H2X_FWD_ROW(1);
+        if (c <= 2 * kWaveSize) H2X_FWD_ROW(2);
+        if (c <= 4 * kWaveSize) H2X_FWD_ROW(4);
+        if (c <= 8 * kWaveSize) H2X_FWD_ROW(8);
+        if (c <= 16 * kWaveSize) H2X_FWD_ROW(16);
+        if (c <= 32 * kWaveSize) H2X_FWD_ROW(32);
+#undef H2X_FWD_ROW
+    }
     const int v4 = vector_width<T>(s, 4 / kWords, {xv, yv});
 #define H2X_FWD(V, CM)                                                                             \
     do                                                                                             \
@@ -375,13 +679,20 @@ int forward_impl(int n, int c, size_t s, const void* xv, void* yv, hipStream_t s
             if (c <= 8) H2X_FWD(2, 8);
             if (c <= 16) H2X_FWD(2, 16);
             if (c <= 32) H2X_FWD(2, 32);
-            if (c <= 64) H2X_FWD(2, 64);
+            if (c <= 64) return launch_fwd_split<T, 2, 16>(x, y, n, c, s, st);
+            if (c <= 128) return launch_fwd_split<T, 2, 32>(x, y, n, c, s, st);
+            if (c <= 192) return launch_fwd_split<T, 2, 48>(x, y, n, c, s, st);
+            if (c <= 256) return launch_fwd_split<T, 2, 64>(x, y, n, c, s, st);
         }
         if (c <= 8) H2X_FWD(1, 8);
         if (c <= 16) H2X_FWD(1, 16);
         if (c <= 32) H2X_FWD(1, 32);
-        if (c <= 64) H2X_FWD(1, 64);
-        if (c <= 128) H2X_FWD(1, 128);
+        if (c <= 64) return launch_fwd_split<T, 1, 16>(x, y, n, c, s, st);
+        if (c <= 128) return launch_fwd_split<T, 1, 32>(x, y, n, c, s, st);
+        if (c <= 192) return launch_fwd_split<T, 1, 48>(x, y, n, c, s, st);
+        if (c <= 256) return launch_fwd_split<T, 1, 64>(x, y, n, c, s, st);
+        if (c <= 384) return launch_fwd_split<T, 1, 96>(x, y, n, c, s, st);
+        if (c <= 512) return launch_fwd_split<T, 1, 128>(x, y, n, c, s, st);
     }
     else
     {
@@ -394,10 +705,13 @@ int forward_impl(int n, int c, size_t s, const void* xv, void* yv, hipStream_t s
         if (c <= 8) H2X_FWD(1, 8);
         if (c <= 16) H2X_FWD(1, 16);
         if (c <= 32) H2X_FWD(1, 32);
-        if (c <= 64) H2X_FWD(1, 64);
+        if (c <= 64) return launch_fwd_split<T, 1, 16>(x, y, n, c, s, st);
+        if (c <= 128) return launch_fwd_split<T, 1, 32>(x, y, n, c, s, st);
+        if (c <= 192) return launch_fwd_split<T, 1, 48>(x, y, n, c, s, st);
+        if (c <= 256) return launch_fwd_split<T, 1, 64>(x, y, n, c, s, st);
     }
 #undef H2X_FWD
-    softmax_fwd_wide_kernel<T><<<wide_grid(s, n), kBlockSize, 0, st>>>(x, y, c, s);
+    softmax_fwd_wide_kernel<T><<<wide_grid(s, 1, n), kBlockSize, 0, st>>>(x, y, c, s);
     return launch_status();
 }
 
@@ -409,6 +723,23 @@ int backward_impl(int n, int c, size_t s, const void* yv, const void* dyv, void*
     const T* dy = static_cast<const T*>(dyv);
     T* dx = static_cast<T*>(dxv);
     constexpr int kWords = sizeof(T) / 4;
+    if (s == 1)
+    {
+        const unsigned int blocks = (static_cast<unsigned int>(n) + kWavesPerBlock - 1) / kWavesPerBlock;
+#define H2X_BWD_ROW(CP)                                                                            \
+    do                                                                                             \
+    {                                                                                              \
+        softmax_bwd_row_kernel<T, CP><<<blocks, kBlockSize, 0, st>>>(y, dy, dx, c, n);              \
+        return launch_status();                                                                    \
+    } while (0)
+        if (c <= 1 * kWaveSize) H2X_BWD_ROW(1);
+        if (c <= 2 * kWaveSize) H2X_BWD_ROW(2);
+        if (c <= 4 * kWaveSize) H2X_BWD_ROW(4);
+        if (c <= 8 * kWaveSize) H2X_BWD_ROW(8);
+        if (c <= 16 * kWaveSize) H2X_BWD_ROW(16);
+        if (c <= 32 * kWaveSize) H2X_BWD_ROW(32);
+#undef H2X_BWD_ROW
+    }
     const int v4 = vector_width<T>(s, 4 / kWords, {yv, dyv, dxv});
 #define H2X_BWD(V, CM)                                                                             \
     do                                                                                             \
@@ -428,11 +759,20 @@ int backward_impl(int n, int c, size_t s, const void* yv, const void* dyv, void*
             if (c <= 8) H2X_BWD(2, 8);
             if (c <= 16) H2X_BWD(2, 16);
             if (c <= 32) H2X_BWD(2, 32);
+            if (c <= 64) return launch_bwd_split<T, 2, 16>(y, dy, dx, n, c, s, st);
+            if (c <= 128) return launch_bwd_split<T, 2, 32>(y, dy, dx, n, c, s, st);
+            if (c <= 192) return launch_bwd_split<T, 2, 48>(y, dy, dx, n, c, s, st);
+            if (c <= 256) return launch_bwd_split<T, 2, 64>(y, dy, dx, n, c, s, st);
         }
         if (c <= 8) H2X_BWD(1, 8);
         if (c <= 16) H2X_BWD(1, 16);
         if (c <= 32) H2X_BWD(1, 32);
-        if (c <= 64) H2X_BWD(1, 64);
+        if (c <= 64) return launch_bwd_split<T, 1, 16>(y, dy, dx, n, c, s, st);
+        if (c <= 128) return launch_bwd_split<T, 1, 32>(y, dy, dx, n, c, s, st);
+        if (c <= 192) return launch_bwd_split<T, 1, 48>(y, dy, dx, n, c, s, st);
+        if (c <= 256) return launch_bwd_split<T, 1, 64>(y, dy, dx, n, c, s, st);
+        if (c <= 384) return launch_bwd_split<T, 1, 96>(y, dy, dx, n, c, s, st);
+        if (c <= 512) return launch_bwd_split<T, 1, 128>(y, dy, dx, n, c, s, st);
     }
     else
     {
@@ -444,9 +784,13 @@ int backward_impl(int n, int c, size_t s, const void* yv, const void* dyv, void*
         if (c <= 8) H2X_BWD(1, 8);
         if (c <= 16) H2X_BWD(1, 16);
         if (c <= 32) H2X_BWD(1, 32);
+        if (c <= 64) return launch_bwd_split<T, 1, 16>(y, dy, dx, n, c, s, st);
+        if (c <= 128) return launch_bwd_split<T, 1, 32>(y, dy, dx, n, c, s, st);
+        if (c <= 192) return launch_bwd_split<T, 1, 48>(y, dy, dx, n, c, s, st);
+        if (c <= 256) return launch_bwd_split<T, 1, 64>(y, dy, dx, n, c, s, st);
     }
 #undef H2X_BWD
-    softmax_bwd_wide_kernel<T><<<wide_grid(s, n), kBlockSize, 0, st>>>(y, dy, dx, c, s);
+    softmax_bwd_wide_kernel<T><<<wide_grid(s, 1, n), kBlockSize, 0, st>>>(y, dy, dx, c, s);
     return launch_status();
 }
 
@@ -654,6 +998,121 @@ __global__ __launch_bounds__(kBlockSize) void softmax_inst_map_kernel(
     P::store(out + off, v);
 }
 
+// Samples of at most 64 * CPL elements (the softmax behind a classifier: 10 to
+// a few thousand classes): a wave takes a sample, holds it in registers and
+// combines its lanes with shuffles, so a reduction is one launch without
+// partials, and the whole forward pass of samples that are whole on this rank is
+// one launch too (N 4096, 10 elements a sample: 18 us in five launches before).
+// Sums are accumulated in fp64, lane by lane and then across the lanes as a
+// butterfly; the staged and the fused path add in the same order.
+enum InstSmall : int
+{
+    kSmallMax = 0,     // result[n] = max x
+    kSmallExpSum = 1,  // out = exp(x - param[n]); result[n] = sum
+    kSmallSumExp = 2,  // result[n] = sum exp(x - param[n])
+    kSmallDot = 3,     // result[n] = sum a * b
+    kSmallForward = 4  // result[n] = max, result2[n] = sum, out = max(exp(x - max) / sum, min_output)
+};
+
+template <typename T, int CPL, int MODE>
+__global__ __launch_bounds__(kBlockSize) void softmax_inst_small_kernel(
+    const T* __restrict__ a, const T* __restrict__ b, T* __restrict__ out,
+    const T* __restrict__ sample_param, T* __restrict__ result, T* __restrict__ result2,
+    int sample_size, int num_samples, T min_output)
+{
+    const int lane = threadIdx.x % kWaveSize;
+    const int n = blockIdx.x * kWavesPerBlock + threadIdx.x / kWaveSize;
+    if (n >= num_samples)
+        return;
+    const size_t base = static_cast<size_t>(n) * sample_size;
+    T va[CPL], vb[CPL];
+#pragma unroll
+    for (int k = 0; k < CPL; ++k)
+        if (lane + k * kWaveSize < sample_size)
+        {
+            va[k] = a[base + lane + k * kWaveSize];
+            if constexpr (MODE == kSmallDot)
+                vb[k] = b[base + lane + k * kWaveSize];
+        }
+    T shift = T(0);
+    if constexpr (MODE == kSmallMax || MODE == kSmallForward)
+    {
+        T mx = Limits<T>::min_normal; // softmax.cu:88-99: the maximum starts at min_normal
+#pragma unroll
+        for (int k = 0; k < CPL; ++k)
+            if (lane + k * kWaveSize < sample_size)
+                mx = va[k] >= mx ? va[k] : mx;
+        mx = wave_max(mx);
+        if (lane == 0)
+            result[n] = mx;
+        if constexpr (MODE == kSmallMax)
+            return;
+        shift = mx;
+    }
+    else if constexpr (MODE != kSmallDot)
+    {
+        shift = sample_param[n];
+    }
+    double acc = 0.0;
+#pragma unroll
+    for (int k = 0; k < CPL; ++k)
+        if (lane + k * kWaveSize < sample_size)
+        {
+            if constexpr (MODE == kSmallDot)
+            {
+                acc = __builtin_fma(static_cast<double>(va[k]), static_cast<double>(vb[k]), acc);
+            }
+            else
+            {
+                va[k] = exp_t(va[k] - shift);
+                acc += static_cast<double>(va[k]);
+            }
+        }
+    acc = wave_butterfly_sum(acc);
+    const T total = static_cast<T>(acc);
+    if (lane == 0)
+        (MODE == kSmallForward ? result2 : result)[n] = total;
+    if constexpr (MODE == kSmallExpSum || MODE == kSmallForward)
+    {
+#pragma unroll
+        for (int k = 0; k < CPL; ++k)
+            if (lane + k * kWaveSize < sample_size)
+            {
+                if constexpr (MODE == kSmallForward)
+                {
+                    const T r = va[k] / total;
+                    va[k] = r > min_output ? r : min_output;
+                }
+                out[base + lane + k * kWaveSize] = va[k];
+            }
+    }
+}
+
+constexpr size_t kInstSmallSample = 32 * kWaveSize;
+
+template <typename T, int MODE>
+int inst_small(int n, size_t sample_size, const void* a, const void* b, void* out,
+               const void* param, void* result, void* result2, T min_output, hipStream_t st)
+{
+    const unsigned int blocks = (static_cast<unsigned int>(n) + kWavesPerBlock - 1) / kWavesPerBlock;
+#define H2X_INST_SMALL(CP)                                                                         \
+    do                                                                                             \
+    {                                                                                              \
+        softmax_inst_small_kernel<T, CP, MODE><<<blocks, kBlockSize, 0, st>>>(                     \
+            static_cast<const T*>(a), static_cast<const T*>(b), static_cast<T*>(out),              \
+            static_cast<const T*>(param), static_cast<T*>(result), static_cast<T*>(result2),       \
+            static_cast<int>(sample_size), n, min_output);                                         \
+        return launch_status();                                                                    \
+    } while (0)
+    if (sample_size <= 1 * kWaveSize) H2X_INST_SMALL(1);
+    if (sample_size <= 2 * kWaveSize) H2X_INST_SMALL(2);
+    if (sample_size <= 4 * kWaveSize) H2X_INST_SMALL(4);
+    if (sample_size <= 8 * kWaveSize) H2X_INST_SMALL(8);
+    if (sample_size <= 16 * kWaveSize) H2X_INST_SMALL(16);
+    H2X_INST_SMALL(32);
+#undef H2X_INST_SMALL
+}
+
 template <typename T>
 T inst_min_output()
 {
@@ -682,6 +1141,14 @@ template <typename T, int MODE>
 int inst_reduce(int n, size_t sample_size, const void* a, const void* b, void* out,
                 const void* param, void* result, void* workspace, hipStream_t st)
 {
+    if (sample_size <= kInstSmallSample && n > 0)
+    {
+        constexpr int kSmallMode = MODE == kInstMax      ? kSmallMax
+                                   : MODE == kInstExpSum ? kSmallExpSum
+                                   : MODE == kInstSumExp ? kSmallSumExp
+                                                         : kSmallDot;
+        return inst_small<T, kSmallMode>(n, sample_size, a, b, out, param, result, nullptr, T(0), st);
+    }
     constexpr int kFull = 16 / sizeof(T);
     const int v = vector_width<T>(sample_size, kFull, {a, b ? b : a, out ? out : a});
     const InstChunking ch = inst_chunking(sample_size, n, v);
@@ -725,6 +1192,9 @@ template <typename T>
 int inst_forward_local(int n, size_t sample_size, const void* x, void* y, void* sample_max,
                        void* sample_exp, void* workspace, hipStream_t st)
 {
+    if (sample_size <= kInstSmallSample && n > 0)
+        return inst_small<T, kSmallForward>(n, sample_size, x, nullptr, y, nullptr, sample_max,
+                                            sample_exp, inst_min_output<T>(), st);
     int err = inst_reduce<T, kInstMax>(n, sample_size, x, nullptr, nullptr, nullptr, sample_max,
                                        workspace, st);
     // `y` takes part in the choice of the vector width only, as in the staged call,

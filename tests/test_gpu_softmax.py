@@ -17,13 +17,23 @@ CASES = [
     (2, 21, 7, 9),        # scalar path
     (3, 4, 8, 8),
     (2, 1, 4, 4),         # one channel
-    (1, 33, 6, 10),       # float2 tile
-    (2, 70, 3, 5),        # CMAX 128, scalar
-    (1, 200, 4, 4),       # more than 128 channels: the waves of a workgroup share the channels
+    (1, 33, 6, 10),       # more than 32 channels: the waves of a workgroup share the channels, two pixels a lane
+    (2, 70, 3, 5),        # the same, one pixel a lane
+    (2, 64, 8, 16),       # 16 channels a wave exactly
+    (1, 200, 4, 4),       # 50 of 64 channels a wave
+    (1, 384, 3, 3),       # 96 channels a wave
     (2, 150, 9, 7),
     (3, 300, 16, 16),
-    (4, 1000, 1, 1),      # one pixel per sample
+    (4, 1000, 1, 1),      # one pixel per sample: a wave per sample, lanes over the channels
+    (70, 10, 1, 1),       # the same with fewer channels than lanes
+    (3, 2048, 1, 1),      # 32 channels a lane, the most
+    (2, 2100, 1, 1),      # beyond that: the re-reading kernel
     (2, 19, 4, 6, 10),    # 5-D
+    (2, 256, 6, 10),      # 64 channels a wave in registers, two pixels a lane
+    (2, 257, 3, 5),       # 65 of 128 channels a wave, one pixel a lane
+    (1, 512, 4, 4),       # the most the register tiles hold
+    (1, 513, 2, 2),       # beyond that: the re-reading kernel
+    (3, 150, 40, 40),     # several workgroups a sample, the last one partly filled
 ]
 
 
@@ -59,11 +69,12 @@ def test_forward_backward(shape, oracle_mod):
     torch.cuda.synchronize()
     dx = dxt.real_view().cpu().numpy()
     dx_o = oracle_mod.softmax_channel_backward(y, dy)
-    if shape[1] <= 64:
+    if shape[1] <= 32 and int(np.prod(shape[2:])) > 1:
         assert np.array_equal(dx, dx_o) or max_rel(dx, dx_o) <= TOL
     else:
-        # above 64 channels dp = sum_c y * dy is formed from four partial sums, the oracle's
-        # from one running sum: dx = y * (dy - dp) then agrees to the tolerance in units of
+        # above 32 channels dp = sum_c y * dy is formed from four partial sums (one pixel per
+        # sample: from the lanes' partial sums), the oracle's from one running sum:
+        # dx = y * (dy - dp) then agrees to the tolerance in units of
         # the terms that are added up (|dy| and sum_c |y * dy|), not of their difference
         terms = np.abs(dy) + (y.astype(np.float64) * np.abs(dy)).sum(axis=1, keepdims=True)
         bound = TOL * y * terms
@@ -118,10 +129,10 @@ def test_all_negative_logits_keep_reference_maximum(oracle_mod):
     assert max_rel(yt.real_view().cpu().numpy(), oracle_mod.softmax_channel_forward(x)) <= TOL
 
 
-def test_float64(oracle_mod):
+@pytest.mark.parametrize("shape", [(2, 9, 4, 6), (2, 100, 4, 6), (1, 200, 3, 3), (1, 300, 2, 2), (3, 130, 1, 1)])
+def test_float64(shape, oracle_mod):
     import torch
     from dihydrogen_amd.layers import Softmax, SoftmaxMode
-    shape = (2, 9, 4, 6)
     rng = np.random.default_rng(17)
     x = 2.0 * rng.standard_normal(shape)
     dy = rng.standard_normal(shape)
@@ -139,7 +150,9 @@ def test_float64(oracle_mod):
     assert max_rel(dxt.real_view().cpu().numpy(), oracle_mod.softmax_channel_backward(y, dy)) <= 1e-12
 
 
-INSTANCE_CASES = [(16, 21, 64, 64), (3, 4, 5, 6), (2, 7, 9), (1, 2, 3, 4, 5), (5, 1, 1, 1), (2, 64, 128, 128)]
+INSTANCE_CASES = [(16, 21, 64, 64), (3, 4, 5, 6), (2, 7, 9), (1, 2, 3, 4, 5), (5, 1, 1, 1), (2, 64, 128, 128),
+                  # samples of at most 2048 elements: a wave per sample
+                  (300, 10, 1, 1), (7, 1000, 1, 1), (3, 2048, 1, 1), (2, 2049, 1, 1), (130, 5, 13, 1)]
 
 
 @pytest.mark.parametrize("shape", INSTANCE_CASES)
