@@ -755,14 +755,20 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop2_kernel(
 // cache line with the neighbouring channels.  A workgroup per channel that walks
 // from sample to sample then fetches 2-3 lines for 196 bytes and leaves its
 // output as partial lines (N 256, C 2048, 7 x 7: 169 MB read and 637 k partial
-// writes for a 103 MB tensor; 106 MB read here, forward 102 us -> 56 us,
-// backward 170 us -> 100 us; N 512, C 4096, 1 x 1: 100 -> 12 us, 138 -> 25 us).  These kernels give a workgroup a window of
+// writes for a 103 MB tensor; 106 MB read here, forward 102 us -> 52 us,
+// backward 170 us -> 91 us; N 512, C 4096, 1 x 1: 100 -> 12 us, 138 -> 25 us).
+// These kernels give a workgroup a window of
 // neighbouring whole channels instead -- one contiguous piece of memory per
 // sample -- and walk through a range of samples.  A segment is padded to
 // `slots` vectors; lane t serves slot t mod slots of channel t div slots for
 // every sample, so its channel and that channel's parameters are fixed for the
 // whole kernel.  The last slot of a segment whose length is no multiple of the
-// vector holds fewer elements and moves them one by one (RAGGED).  Where few
+// vector owns fewer elements: its vector starts that much earlier, so that it
+// is still loaded whole, overlaps the slot before it, and only the elements it
+// owns are added up or stored (kTailOverlap; in place of x, dx may be written
+// by the neighbouring lane before this lane reads the overlap, which it does
+// not use).  Segments shorter than a vector move element by element
+// (kTailScalar).  Where few
 // channels and many samples would leave a reduction with too few workgroups,
 // the lanes of a workgroup form `rows` rows that take every rows-th sample of
 // a narrower window.
@@ -775,19 +781,27 @@ struct ShortGeometry
     int samples_per_group;  // samples one workgroup walks through (blockIdx.y counts these ranges)
 };
 
+enum ShortTail : int
+{
+    kTailNone = 0,    // segments are whole vectors
+    kTailOverlap = 1, // the last vector of a segment overlaps the one before it
+    kTailScalar = 2   // segments shorter than a vector
+};
+
 struct ShortLane
 {
     int row;    // row of lanes: its samples are row, row + rows, ... of the workgroup's range
     int q;      // channel within the workgroup's window
     int slot;   // slot of the channel's segment
     int c;      // channel
-    int first;  // first element of the slot within its segment
-    int valid;  // elements of the slot that lie inside the segment; 0: an idle lane
+    int first;  // first element of the slot's vector within its segment
+    int valid;  // elements the slot owns; 0: an idle lane
+    int skip;   // leading elements of its vector that the slot before it owns (kTailOverlap)
     bool heads; // first lane of its channel in its row
     bool leads; // first lane of its channel in row 0
 };
 
-template <int VEC>
+template <int VEC, int TAIL>
 __device__ __forceinline__ ShortLane short_lane(const ShortGeometry& g)
 {
     ShortLane l;
@@ -798,19 +812,32 @@ __device__ __forceinline__ ShortLane short_lane(const ShortGeometry& g)
     const int v = t - l.q * g.slots;
     l.slot = v;
     l.c = static_cast<int>(blockIdx.x) * g.channels_per_group + l.q;
-    l.first = v * VEC;
-    const int left = g.spatial - l.first;
+    const int left = g.spatial - v * VEC;
     const bool active = l.q < g.channels_per_group && l.c < g.num_channels;
     l.valid = active ? (left < VEC ? left : VEC) : 0;
+    l.skip = TAIL == kTailOverlap && active ? VEC - l.valid : 0;
+    l.first = v * VEC - l.skip;
     l.heads = active && v == 0;
     l.leads = l.heads && l.row == 0;
     return l;
 }
 
-template <typename T, int VEC, bool RAGGED, bool STREAM = false>
-__device__ __forceinline__ void load_slot(const T* p, int valid, T (&r)[VEC])
+// Whether element j of the lane's vector is one the lane owns.
+template <int VEC, int TAIL>
+__device__ __forceinline__ bool slot_owns(const ShortLane& l, int j)
 {
-    if (!RAGGED || valid == VEC)
+    if constexpr (TAIL == kTailNone)
+        return true;
+    else if constexpr (TAIL == kTailOverlap)
+        return j >= l.skip;
+    else
+        return j < l.valid;
+}
+
+template <typename T, int VEC, int TAIL, bool STREAM = false>
+__device__ __forceinline__ void load_slot(const T* p, const ShortLane& l, T (&r)[VEC])
+{
+    if constexpr (TAIL != kTailScalar)
     {
         load_vec<T, VEC, false, STREAM>(p, r);
     }
@@ -821,23 +848,27 @@ __device__ __forceinline__ void load_slot(const T* p, int valid, T (&r)[VEC])
             r[j] = T(0);
 #pragma unroll
         for (int j = 0; j < VEC - 1; ++j)
-            if (j < valid)
+            if (j < l.valid)
                 r[j] = STREAM ? __builtin_nontemporal_load(p + j) : p[j];
     }
 }
 
-template <typename T, int VEC, bool RAGGED>
-__device__ __forceinline__ void store_slot(T* p, int valid, const T (&r)[VEC])
+// rewrite: the output does not alias an input, so the elements in which the
+// last vector overlaps its neighbour may be stored by both lanes (each made
+// the same values from the same inputs) and every lane stores a whole vector.
+template <typename T, int VEC, int TAIL>
+__device__ __forceinline__ void store_slot(T* p, const ShortLane& l, const T (&r)[VEC],
+                                           bool rewrite)
 {
-    if (!RAGGED || valid == VEC)
+    if (TAIL == kTailNone || (TAIL == kTailOverlap && (rewrite || l.skip == 0)))
     {
         store_vec<T, VEC, false>(p, r);
     }
     else
     {
 #pragma unroll
-        for (int j = 0; j < VEC - 1; ++j)
-            if (j < valid)
+        for (int j = 0; j < VEC; ++j)
+            if (slot_owns<VEC, TAIL>(l, j))
                 __builtin_nontemporal_store(r[j], p + j);
     }
 }
@@ -956,12 +987,12 @@ __global__ void bn_finish_short_kernel(const double* __restrict__ partials, int 
         outs[k][c] = static_cast<T>(t[k]);
 }
 
-template <typename T, int VEC, bool RAGGED>
+template <typename T, int VEC, int TAIL>
 __global__ __launch_bounds__(kBlockSize) void bn_sums_short_kernel(
     const T* __restrict__ x, T* __restrict__ sums, T* __restrict__ sqsums, double* partials,
     int64_t stride_n, int64_t stride_c, const ShortGeometry g, bool always_partials)
 {
-    const ShortLane l = short_lane<VEC>(g);
+    const ShortLane l = short_lane<VEC, TAIL>(g);
     double acc[2] = {0.0, 0.0};
     if (l.valid > 0)
     {
@@ -969,7 +1000,7 @@ __global__ __launch_bounds__(kBlockSize) void bn_sums_short_kernel(
 #pragma unroll
             for (int j = 0; j < VEC; ++j)
             {
-                if (RAGGED && j >= l.valid)
+                if (!slot_owns<VEC, TAIL>(l, j))
                     continue;
                 const double d = static_cast<double>(v[j]);
                 acc[0] += d;
@@ -990,7 +1021,7 @@ __global__ __launch_bounds__(kBlockSize) void bn_sums_short_kernel(
             T v[kUnroll][VEC];
 #pragma unroll
             for (int u = 0; u < kUnroll; ++u)
-                load_slot<T, VEC, RAGGED>(p + (n + u * step) * stride_n, l.valid, v[u]);
+                load_slot<T, VEC, TAIL>(p + (n + u * step) * stride_n, l, v[u]);
 #pragma unroll
             for (int u = 0; u < kUnroll; ++u)
                 accumulate(v[u]);
@@ -998,7 +1029,7 @@ __global__ __launch_bounds__(kBlockSize) void bn_sums_short_kernel(
         for (; n < end; n += step)
         {
             T v[VEC];
-            load_slot<T, VEC, RAGGED>(p + n * stride_n, l.valid, v);
+            load_slot<T, VEC, TAIL>(p + n * stride_n, l, v);
             accumulate(v);
         }
     }
@@ -1006,14 +1037,14 @@ __global__ __launch_bounds__(kBlockSize) void bn_sums_short_kernel(
     finish_short<T, 2>(g, l, acc, partials, always_partials, out);
 }
 
-template <typename T, int VEC, bool RAGGED, bool FUSED>
+template <typename T, int VEC, int TAIL, bool FUSED>
 __global__ __launch_bounds__(kBlockSize) void bn_apply_short_kernel(
     const T* __restrict__ x, const T* __restrict__ mean, const T* __restrict__ var,
     const T* __restrict__ scale, const T* __restrict__ bias, T* __restrict__ y, T epsilon,
     int64_t x_stride_n, int64_t x_stride_c, int64_t y_stride_n, int64_t y_stride_c,
     const ShortGeometry g, const FusedStats<T> fused)
 {
-    const ShortLane l = short_lane<VEC>(g);
+    const ShortLane l = short_lane<VEC, TAIL>(g);
     T m = T(0), variance = T(0);
     if constexpr (FUSED)
     {
@@ -1062,28 +1093,28 @@ __global__ __launch_bounds__(kBlockSize) void bn_apply_short_kernel(
         T v[kUnroll][VEC];
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u)
-            load_slot<T, VEC, RAGGED>(xp + (n + u) * x_stride_n, l.valid, v[u]);
+            load_slot<T, VEC, TAIL>(xp + (n + u) * x_stride_n, l, v[u]);
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u)
         {
 #pragma unroll
             for (int j = 0; j < VEC; ++j)
                 v[u][j] = fma_t((v[u][j] - m) * inv_stdev, sc, bi);
-            store_slot<T, VEC, RAGGED>(yp + (n + u) * y_stride_n, l.valid, v[u]);
+            store_slot<T, VEC, TAIL>(yp + (n + u) * y_stride_n, l, v[u], true);
         }
     }
     for (; n < end; ++n)
     {
         T v[VEC];
-        load_slot<T, VEC, RAGGED>(xp + n * x_stride_n, l.valid, v);
+        load_slot<T, VEC, TAIL>(xp + n * x_stride_n, l, v);
 #pragma unroll
         for (int j = 0; j < VEC; ++j)
             v[j] = fma_t((v[j] - m) * inv_stdev, sc, bi);
-        store_slot<T, VEC, RAGGED>(yp + n * y_stride_n, l.valid, v);
+        store_slot<T, VEC, TAIL>(yp + n * y_stride_n, l, v, true);
     }
 }
 
-template <typename T, int VEC, bool RAGGED>
+template <typename T, int VEC, int TAIL>
 __global__ __launch_bounds__(kBlockSize) void bn_backprop1_short_kernel(
     const T* __restrict__ x, const T* __restrict__ dy, const T* __restrict__ mean,
     const T* __restrict__ var, const T* __restrict__ scale, T* __restrict__ dscale,
@@ -1091,7 +1122,7 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop1_short_kernel(
     double* partials, int64_t x_stride_n, int64_t x_stride_c, int64_t d_stride_n,
     int64_t d_stride_c, const ShortGeometry g, bool always_partials)
 {
-    const ShortLane l = short_lane<VEC>(g);
+    const ShortLane l = short_lane<VEC, TAIL>(g);
     double acc[4] = {0.0, 0.0, 0.0, 0.0};
     if (l.valid > 0)
     {
@@ -1105,7 +1136,7 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop1_short_kernel(
 #pragma unroll
             for (int j = 0; j < VEC; ++j)
             {
-                if (RAGGED && j >= l.valid)
+                if (!slot_owns<VEC, TAIL>(l, j))
                     continue;
                 const T xm = xv[j] - m;
                 const T xhat = xm * inv_stdev;
@@ -1132,8 +1163,8 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop1_short_kernel(
 #pragma unroll
             for (int u = 0; u < kUnroll2; ++u)
             {
-                load_slot<T, VEC, RAGGED>(xp + (n + u * step) * x_stride_n, l.valid, xv[u]);
-                load_slot<T, VEC, RAGGED, true>(dp + (n + u * step) * d_stride_n, l.valid, dv[u]);
+                load_slot<T, VEC, TAIL>(xp + (n + u * step) * x_stride_n, l, xv[u]);
+                load_slot<T, VEC, TAIL, true>(dp + (n + u * step) * d_stride_n, l, dv[u]);
             }
 #pragma unroll
             for (int u = 0; u < kUnroll2; ++u)
@@ -1142,8 +1173,8 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop1_short_kernel(
         for (; n < end; n += step)
         {
             T xv[VEC], dv[VEC];
-            load_slot<T, VEC, RAGGED>(xp + n * x_stride_n, l.valid, xv);
-            load_slot<T, VEC, RAGGED, true>(dp + n * d_stride_n, l.valid, dv);
+            load_slot<T, VEC, TAIL>(xp + n * x_stride_n, l, xv);
+            load_slot<T, VEC, TAIL, true>(dp + n * d_stride_n, l, dv);
             accumulate(xv, dv);
         }
     }
@@ -1151,16 +1182,17 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop1_short_kernel(
     finish_short<T, 4>(g, l, acc, partials, always_partials, out);
 }
 
-// x and dx may alias: each lane reads its elements before it writes them.
-template <typename T, int VEC, bool RAGGED, bool FUSED>
+// x and dx may alias: each lane reads its elements before it writes them
+// (`disjoint`: they share no memory).
+template <typename T, int VEC, int TAIL, bool FUSED>
 __global__ __launch_bounds__(kBlockSize) void bn_backprop2_short_kernel(
     const T* x, const T* __restrict__ dy, const T* __restrict__ mean, const T* __restrict__ var,
     const T* __restrict__ scale, const T* __restrict__ dmean, const T* __restrict__ dvar, T* dx,
     T epsilon, size_t num_per_sum, int64_t x_stride_n, int64_t x_stride_c, int64_t d_stride_n,
     int64_t d_stride_c, int64_t o_stride_n, int64_t o_stride_c, const ShortGeometry g,
-    const FusedStats<T> fused)
+    bool disjoint, const FusedStats<T> fused)
 {
-    const ShortLane l = short_lane<VEC>(g);
+    const ShortLane l = short_lane<VEC, TAIL>(g);
     T dmean_c = T(0), dvar_c = T(0);
     if constexpr (FUSED)
     {
@@ -1210,8 +1242,8 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop2_short_kernel(
 #pragma unroll
         for (int u = 0; u < kUnroll2; ++u)
         {
-            load_slot<T, VEC, RAGGED>(xp + (n + u) * x_stride_n, l.valid, xv[u]);
-            load_slot<T, VEC, RAGGED, true>(dp + (n + u) * d_stride_n, l.valid, dv[u]);
+            load_slot<T, VEC, TAIL>(xp + (n + u) * x_stride_n, l, xv[u]);
+            load_slot<T, VEC, TAIL, true>(dp + (n + u) * d_stride_n, l, dv[u]);
         }
 #pragma unroll
         for (int u = 0; u < kUnroll2; ++u)
@@ -1222,21 +1254,21 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop2_short_kernel(
                 const T r = fma_t(dv[u][j] * sc, inv_stdev, dmean_term);
                 xv[u][j] = fma_t(xv[u][j] - m, dvar_term, r);
             }
-            store_slot<T, VEC, RAGGED>(op + (n + u) * o_stride_n, l.valid, xv[u]);
+            store_slot<T, VEC, TAIL>(op + (n + u) * o_stride_n, l, xv[u], disjoint);
         }
     }
     for (; n < end; ++n)
     {
         T xv[VEC], dv[VEC];
-        load_slot<T, VEC, RAGGED>(xp + n * x_stride_n, l.valid, xv);
-        load_slot<T, VEC, RAGGED, true>(dp + n * d_stride_n, l.valid, dv);
+        load_slot<T, VEC, TAIL>(xp + n * x_stride_n, l, xv);
+        load_slot<T, VEC, TAIL, true>(dp + n * d_stride_n, l, dv);
 #pragma unroll
         for (int j = 0; j < VEC; ++j)
         {
             const T r = fma_t(dv[j] * sc, inv_stdev, dmean_term);
             xv[j] = fma_t(xv[j] - m, dvar_term, r);
         }
-        store_slot<T, VEC, RAGGED>(op + n * o_stride_n, l.valid, xv);
+        store_slot<T, VEC, TAIL>(op + n * o_stride_n, l, xv, disjoint);
     }
 }
 
@@ -1515,23 +1547,30 @@ int short_elementwise_groups(ShortGeometry* g, int unroll, size_t prologue_bytes
     return (g->num_samples + g->samples_per_group - 1) / g->samples_per_group;
 }
 
-// Launches kernel<T, V, RAGGED> of the short-segment family.
+// Launches kernel<T, V, TAIL> of the short-segment family.
 #define H2X_DISPATCH_SHORT(KERNEL, GRID, ...)                                                      \
     do                                                                                             \
     {                                                                                              \
-        if (sg.spatial % full_vec<T>() != 0)                                                       \
-            KERNEL<T, full_vec<T>(), true><<<GRID, kBlockSize, 0, stream>>>(__VA_ARGS__);          \
+        if (sg.spatial % full_vec<T>() == 0)                                                       \
+            KERNEL<T, full_vec<T>(), kTailNone><<<GRID, kBlockSize, 0, stream>>>(__VA_ARGS__);     \
+        else if (sg.spatial > full_vec<T>())                                                       \
+            KERNEL<T, full_vec<T>(), kTailOverlap><<<GRID, kBlockSize, 0, stream>>>(__VA_ARGS__);  \
         else                                                                                       \
-            KERNEL<T, full_vec<T>(), false><<<GRID, kBlockSize, 0, stream>>>(__VA_ARGS__);         \
+            KERNEL<T, full_vec<T>(), kTailScalar><<<GRID, kBlockSize, 0, stream>>>(__VA_ARGS__);   \
     } while (0)
 
 #define H2X_DISPATCH_SHORT_FUSED(KERNEL, FUSED, GRID, ...)                                         \
     do                                                                                             \
     {                                                                                              \
-        if (sg.spatial % full_vec<T>() != 0)                                                       \
-            KERNEL<T, full_vec<T>(), true, FUSED><<<GRID, kBlockSize, 0, stream>>>(__VA_ARGS__);   \
+        if (sg.spatial % full_vec<T>() == 0)                                                       \
+            KERNEL<T, full_vec<T>(), kTailNone, FUSED>                                             \
+                <<<GRID, kBlockSize, 0, stream>>>(__VA_ARGS__);                                    \
+        else if (sg.spatial > full_vec<T>())                                                       \
+            KERNEL<T, full_vec<T>(), kTailOverlap, FUSED>                                          \
+                <<<GRID, kBlockSize, 0, stream>>>(__VA_ARGS__);                                    \
         else                                                                                       \
-            KERNEL<T, full_vec<T>(), false, FUSED><<<GRID, kBlockSize, 0, stream>>>(__VA_ARGS__);  \
+            KERNEL<T, full_vec<T>(), kTailScalar, FUSED>                                           \
+                <<<GRID, kBlockSize, 0, stream>>>(__VA_ARGS__);                                    \
     } while (0)
 
 // Launches kernel<T, V, STRIDED> for the width and layout chosen at run time.
@@ -1820,6 +1859,15 @@ int backprop2_impl(int num_samples, int num_channels, size_t spatial, size_t num
         return H2X_ERR_UNSUPPORTED; // the partials are laid out for the other family of kernels
     if (is_short)
     {
+        // whether x and dx share memory (the reference allows dx to be x itself)
+        const auto span = [&](const HostTensor& t) {
+            return (static_cast<size_t>(num_samples - 1) * t.map.stride_n
+                    + static_cast<size_t>(num_channels - 1) * t.map.stride_c + spatial)
+                   * sizeof(T);
+        };
+        const char* xb = static_cast<const char*>(x);
+        const char* ob = static_cast<const char*>(dx);
+        const bool disjoint = xb + span(tx_in) <= ob || ob + span(to_in) <= xb;
         const dim3 grid(short_windows(sg),
                         short_elementwise_groups(&sg, kUnroll / 2,
                                                  fused ? fused->groups * 4 * sizeof(double) : 0,
@@ -1832,7 +1880,7 @@ int backprop2_impl(int num_samples, int num_channels, size_t spatial, size_t num
                                      static_cast<T*>(dx), static_cast<T>(epsilon), num_per_sum,
                                      tx_in.map.stride_n, tx_in.map.stride_c, td_in.map.stride_n,
                                      td_in.map.stride_c, to_in.map.stride_n, to_in.map.stride_c, sg,
-                                     *fused);
+                                     disjoint, *fused);
         else
             H2X_DISPATCH_SHORT_FUSED(bn_backprop2_short_kernel, false, grid,
                                      static_cast<const T*>(x), static_cast<const T*>(dy),
@@ -1841,7 +1889,8 @@ int backprop2_impl(int num_samples, int num_channels, size_t spatial, size_t num
                                      static_cast<const T*>(dvar), static_cast<T*>(dx),
                                      static_cast<T>(epsilon), num_per_sum, tx_in.map.stride_n,
                                      tx_in.map.stride_c, td_in.map.stride_n, td_in.map.stride_c,
-                                     to_in.map.stride_n, to_in.map.stride_c, sg, FusedStats<T>());
+                                     to_in.map.stride_n, to_in.map.stride_c, sg, disjoint,
+                                     FusedStats<T>());
         return launch_status();
     }
     HostTensor tx = tx_in, td = td_in, to = to_in;
