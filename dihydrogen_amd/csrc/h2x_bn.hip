@@ -775,10 +775,23 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop2_kernel(
 struct ShortGeometry
 {
     int num_samples, num_channels, spatial;
-    int slots;              // vectors a segment is padded to
+    int row;                // elements that are contiguous in every tensor of the launch: the
+                            // whole segment, or a row of it when some tensor has halos inside
+    int slots_per_row;      // vectors a row is padded to
+    int slots;              // vectors a segment is padded to: its rows * slots_per_row
+    int rows_per_plane;     // rows in a plane of the segment (launches that go row by row)
     int rows;               // rows of lanes, each on samples of its own
     int channels_per_group; // whole channels one workgroup serves: kBlockSize / rows / slots
     int samples_per_group;  // samples one workgroup walks through (blockIdx.y counts these ranges)
+};
+
+// One tensor of a short-segment launch: where sample n, channel c starts and
+// where the rows of its segment lie.
+struct ShortTensor
+{
+    int64_t stride_n, stride_c;
+    int h;          // rows per plane (interior extent of spatial dimension 1)
+    int64_t sy, sz; // strides of spatial dimensions 1 and 2
 };
 
 enum ShortTail : int
@@ -794,7 +807,8 @@ struct ShortLane
     int q;      // channel within the workgroup's window
     int slot;   // slot of the channel's segment
     int c;      // channel
-    int first;  // first element of the slot's vector within its segment
+    int line;   // row of the segment the slot lies in
+    int first;  // first element of the slot's vector within its row
     int valid;  // elements the slot owns; 0: an idle lane
     int skip;   // leading elements of its vector that the slot before it owns (kTailOverlap)
     bool heads; // first lane of its channel in its row
@@ -812,11 +826,13 @@ __device__ __forceinline__ ShortLane short_lane(const ShortGeometry& g)
     const int v = t - l.q * g.slots;
     l.slot = v;
     l.c = static_cast<int>(blockIdx.x) * g.channels_per_group + l.q;
-    const int left = g.spatial - v * VEC;
+    l.line = v / g.slots_per_row;
+    const int k = v - l.line * g.slots_per_row;
+    const int left = g.row - k * VEC;
     const bool active = l.q < g.channels_per_group && l.c < g.num_channels;
     l.valid = active ? (left < VEC ? left : VEC) : 0;
     l.skip = TAIL == kTailOverlap && active ? VEC - l.valid : 0;
-    l.first = v * VEC - l.skip;
+    l.first = k * VEC - l.skip;
     l.heads = active && v == 0;
     l.leads = l.heads && l.row == 0;
     return l;
@@ -832,6 +848,16 @@ __device__ __forceinline__ bool slot_owns(const ShortLane& l, int j)
         return j >= l.skip;
     else
         return j < l.valid;
+}
+
+// Where a lane's slot starts in one tensor, relative to the start of the
+// (sample, channel) segment.  The lane's place in the segment never changes, so
+// this is worked out once.
+__device__ __forceinline__ int slot_offset(const ShortLane& l, const ShortTensor& t)
+{
+    const int z = l.line / t.h;
+    const int y = l.line - z * t.h;
+    return static_cast<int>(l.first + y * t.sy + z * t.sz);
 }
 
 template <typename T, int VEC, int TAIL, bool STREAM = false>
@@ -854,8 +880,8 @@ __device__ __forceinline__ void load_slot(const T* p, const ShortLane& l, T (&r)
 }
 
 // rewrite: the output does not alias an input, so the elements in which the
-// last vector overlaps its neighbour may be stored by both lanes (each made
-// the same values from the same inputs) and every lane stores a whole vector.
+// last vector of a row overlaps its neighbour may be stored by both lanes (each
+// made the same values from the same inputs) and every lane stores a whole vector.
 template <typename T, int VEC, int TAIL>
 __device__ __forceinline__ void store_slot(T* p, const ShortLane& l, const T (&r)[VEC],
                                            bool rewrite)
@@ -990,7 +1016,7 @@ __global__ void bn_finish_short_kernel(const double* __restrict__ partials, int 
 template <typename T, int VEC, int TAIL>
 __global__ __launch_bounds__(kBlockSize) void bn_sums_short_kernel(
     const T* __restrict__ x, T* __restrict__ sums, T* __restrict__ sqsums, double* partials,
-    int64_t stride_n, int64_t stride_c, const ShortGeometry g, bool always_partials)
+    const ShortTensor tx, const ShortGeometry g, bool always_partials)
 {
     const ShortLane l = short_lane<VEC, TAIL>(g);
     double acc[2] = {0.0, 0.0};
@@ -1010,7 +1036,8 @@ __global__ __launch_bounds__(kBlockSize) void bn_sums_short_kernel(
                     acc[1] += d * d;
             }
         };
-        const T* p = x + l.c * stride_c + l.first;
+        const T* p = x + l.c * tx.stride_c + slot_offset(l, tx);
+        const int64_t stride_n = tx.stride_n;
         int n = blockIdx.y * g.samples_per_group;
         const int end = n + g.samples_per_group < g.num_samples ? n + g.samples_per_group
                                                                 : g.num_samples;
@@ -1041,8 +1068,7 @@ template <typename T, int VEC, int TAIL, bool FUSED>
 __global__ __launch_bounds__(kBlockSize) void bn_apply_short_kernel(
     const T* __restrict__ x, const T* __restrict__ mean, const T* __restrict__ var,
     const T* __restrict__ scale, const T* __restrict__ bias, T* __restrict__ y, T epsilon,
-    int64_t x_stride_n, int64_t x_stride_c, int64_t y_stride_n, int64_t y_stride_c,
-    const ShortGeometry g, const FusedStats<T> fused)
+    const ShortTensor tx, const ShortTensor ty, const ShortGeometry g, const FusedStats<T> fused)
 {
     const ShortLane l = short_lane<VEC, TAIL>(g);
     T m = T(0), variance = T(0);
@@ -1083,8 +1109,9 @@ __global__ __launch_bounds__(kBlockSize) void bn_apply_short_kernel(
     const T inv_stdev = inv_sqrt_t(variance + epsilon);
     const T sc = scale[l.c];
     const T bi = bias[l.c];
-    const T* xp = x + l.c * x_stride_c + l.first;
-    T* yp = y + l.c * y_stride_c + l.first;
+    const T* xp = x + l.c * tx.stride_c + slot_offset(l, tx);
+    T* yp = y + l.c * ty.stride_c + slot_offset(l, ty);
+    const int64_t x_stride_n = tx.stride_n, y_stride_n = ty.stride_n;
     int n = blockIdx.y * g.samples_per_group;
     const int end =
         n + g.samples_per_group < g.num_samples ? n + g.samples_per_group : g.num_samples;
@@ -1119,8 +1146,8 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop1_short_kernel(
     const T* __restrict__ x, const T* __restrict__ dy, const T* __restrict__ mean,
     const T* __restrict__ var, const T* __restrict__ scale, T* __restrict__ dscale,
     T* __restrict__ dbias, T* __restrict__ dmean, T* __restrict__ dvar, T epsilon,
-    double* partials, int64_t x_stride_n, int64_t x_stride_c, int64_t d_stride_n,
-    int64_t d_stride_c, const ShortGeometry g, bool always_partials)
+    double* partials, const ShortTensor tx, const ShortTensor td, const ShortGeometry g,
+    bool always_partials)
 {
     const ShortLane l = short_lane<VEC, TAIL>(g);
     double acc[4] = {0.0, 0.0, 0.0, 0.0};
@@ -1150,8 +1177,9 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop1_short_kernel(
             }
         };
         constexpr int kUnroll2 = kUnroll / 2; // two streams: same bytes in flight
-        const T* xp = x + l.c * x_stride_c + l.first;
-        const T* dp = dy + l.c * d_stride_c + l.first;
+        const T* xp = x + l.c * tx.stride_c + slot_offset(l, tx);
+        const T* dp = dy + l.c * td.stride_c + slot_offset(l, td);
+        const int64_t x_stride_n = tx.stride_n, d_stride_n = td.stride_n;
         int n = blockIdx.y * g.samples_per_group;
         const int end = n + g.samples_per_group < g.num_samples ? n + g.samples_per_group
                                                                 : g.num_samples;
@@ -1188,9 +1216,8 @@ template <typename T, int VEC, int TAIL, bool FUSED>
 __global__ __launch_bounds__(kBlockSize) void bn_backprop2_short_kernel(
     const T* x, const T* __restrict__ dy, const T* __restrict__ mean, const T* __restrict__ var,
     const T* __restrict__ scale, const T* __restrict__ dmean, const T* __restrict__ dvar, T* dx,
-    T epsilon, size_t num_per_sum, int64_t x_stride_n, int64_t x_stride_c, int64_t d_stride_n,
-    int64_t d_stride_c, int64_t o_stride_n, int64_t o_stride_c, const ShortGeometry g,
-    bool disjoint, const FusedStats<T> fused)
+    T epsilon, size_t num_per_sum, const ShortTensor tx, const ShortTensor td,
+    const ShortTensor to, const ShortGeometry g, bool disjoint, const FusedStats<T> fused)
 {
     const ShortLane l = short_lane<VEC, TAIL>(g);
     T dmean_c = T(0), dvar_c = T(0);
@@ -1230,9 +1257,10 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop2_short_kernel(
     const T dmean_term = dmean_c / static_cast<T>(num_per_sum);
     const T dvar_term = dvar_c * T(2) / static_cast<T>(num_per_sum - 1);
     constexpr int kUnroll2 = kUnroll / 2;
-    const T* xp = x + l.c * x_stride_c + l.first;
-    const T* dp = dy + l.c * d_stride_c + l.first;
-    T* op = dx + l.c * o_stride_c + l.first;
+    const T* xp = x + l.c * tx.stride_c + slot_offset(l, tx);
+    const T* dp = dy + l.c * td.stride_c + slot_offset(l, td);
+    T* op = dx + l.c * to.stride_c + slot_offset(l, to);
+    const int64_t x_stride_n = tx.stride_n, d_stride_n = td.stride_n, o_stride_n = to.stride_n;
     int n = blockIdx.y * g.samples_per_group;
     const int end =
         n + g.samples_per_group < g.num_samples ? n + g.samples_per_group : g.num_samples;
@@ -1456,6 +1484,31 @@ constexpr size_t kShortSegment = 256;
 // Workgroups an elementwise short-segment pass aims at.
 constexpr int kShortElementwiseBlocks = 8192;
 
+// Elements from the first to the last interior element of a segment.
+size_t short_span(const HostTensor& t, size_t spatial)
+{
+    if (!t.strided)
+        return spatial;
+    const size_t w = t.map.w.divisor, h = t.map.h.divisor;
+    const size_t d = spatial / (w * h);
+    return (w - 1) + (h - 1) * static_cast<size_t>(t.map.sy) + (d - 1) * static_cast<size_t>(t.map.sz)
+           + 1;
+}
+
+// A tensor as a short-segment launch addresses it.  When the launch goes row by
+// row (some tensor has halos inside its segments), a dense tensor's rows follow
+// one another: strides row and row * h.
+ShortTensor short_tensor(const HostTensor& t, const ShortGeometry& g)
+{
+    ShortTensor r;
+    r.stride_n = t.map.stride_n;
+    r.stride_c = t.map.stride_c;
+    r.h = g.rows_per_plane;
+    r.sy = t.strided ? t.map.sy : g.row;
+    r.sz = t.strided ? t.map.sz : static_cast<int64_t>(g.row) * g.rows_per_plane;
+    return r;
+}
+
 // Whether a launch over these tensors takes the short-segment kernels, and the
 // window of channels a workgroup serves then.
 template <typename T>
@@ -1465,13 +1518,25 @@ bool short_segments(int num_samples, int num_channels, size_t spatial,
     if (spatial == 0 || spatial > kShortSegment || num_samples < 1 || num_channels < 1)
         return false;
     for (const HostTensor* t : ts)
-        if (t->strided)
-            return false;
+        if (t->strided && short_span(*t, spatial) > 0x7fffffffull)
+            return false; // offsets within a segment are kept as 32-bit integers
     const int vec = full_vec<T>();
     g->num_samples = num_samples;
     g->num_channels = num_channels;
     g->spatial = static_cast<int>(spatial);
-    g->slots = (g->spatial + vec - 1) / vec;
+    // dense tensors only: the segment is one row; else every tensor goes row by row
+    g->row = g->spatial;
+    g->rows_per_plane = 1;
+    for (const HostTensor* t : ts)
+        if (t->strided)
+        {
+            g->row = static_cast<int>(t->map.w.divisor);
+            g->rows_per_plane = static_cast<int>(t->map.h.divisor);
+        }
+    g->slots_per_row = (g->row + vec - 1) / vec;
+    g->slots = g->spatial / g->row * g->slots_per_row;
+    if (g->slots > kBlockSize)
+        return false;
     g->rows = 1;
     g->channels_per_group = kBlockSize / g->slots;
     g->samples_per_group = num_samples;
@@ -1547,13 +1612,13 @@ int short_elementwise_groups(ShortGeometry* g, int unroll, size_t prologue_bytes
     return (g->num_samples + g->samples_per_group - 1) / g->samples_per_group;
 }
 
-// Launches kernel<T, V, TAIL> of the short-segment family.
+// Launches kernel<T, V, TAIL> of the short-segment family (`sg`: the geometry).
 #define H2X_DISPATCH_SHORT(KERNEL, GRID, ...)                                                      \
     do                                                                                             \
     {                                                                                              \
-        if (sg.spatial % full_vec<T>() == 0)                                                       \
+        if (sg.row % full_vec<T>() == 0)                                                           \
             KERNEL<T, full_vec<T>(), kTailNone><<<GRID, kBlockSize, 0, stream>>>(__VA_ARGS__);     \
-        else if (sg.spatial > full_vec<T>())                                                       \
+        else if (sg.row > full_vec<T>())                                                           \
             KERNEL<T, full_vec<T>(), kTailOverlap><<<GRID, kBlockSize, 0, stream>>>(__VA_ARGS__);  \
         else                                                                                       \
             KERNEL<T, full_vec<T>(), kTailScalar><<<GRID, kBlockSize, 0, stream>>>(__VA_ARGS__);   \
@@ -1562,10 +1627,10 @@ int short_elementwise_groups(ShortGeometry* g, int unroll, size_t prologue_bytes
 #define H2X_DISPATCH_SHORT_FUSED(KERNEL, FUSED, GRID, ...)                                         \
     do                                                                                             \
     {                                                                                              \
-        if (sg.spatial % full_vec<T>() == 0)                                                       \
+        if (sg.row % full_vec<T>() == 0)                                                           \
             KERNEL<T, full_vec<T>(), kTailNone, FUSED>                                             \
                 <<<GRID, kBlockSize, 0, stream>>>(__VA_ARGS__);                                    \
-        else if (sg.spatial > full_vec<T>())                                                       \
+        else if (sg.row > full_vec<T>())                                                           \
             KERNEL<T, full_vec<T>(), kTailOverlap, FUSED>                                          \
                 <<<GRID, kBlockSize, 0, stream>>>(__VA_ARGS__);                                    \
         else                                                                                       \
@@ -1644,7 +1709,7 @@ int sums_impl(int num_samples, int num_channels, size_t spatial, const HostTenso
         const dim3 grid(short_windows(sg), groups);
         H2X_DISPATCH_SHORT(bn_sums_short_kernel, grid, static_cast<const T*>(x),
                            static_cast<T*>(sums), static_cast<T*>(sqsums), partials,
-                           tx_in.map.stride_n, tx_in.map.stride_c, sg, fused_out != nullptr);
+                           short_tensor(tx_in, sg), sg, fused_out != nullptr);
         if (fused_out)
         {
             fused_out->groups = groups;
@@ -1733,16 +1798,14 @@ int apply_impl(int num_samples, int num_channels, size_t spatial, const HostTens
             H2X_DISPATCH_SHORT_FUSED(bn_apply_short_kernel, true, grid, static_cast<const T*>(x),
                                      nullptr, nullptr, static_cast<const T*>(scale),
                                      static_cast<const T*>(bias), static_cast<T*>(y),
-                                     static_cast<T>(epsilon), tx_in.map.stride_n,
-                                     tx_in.map.stride_c, ty_in.map.stride_n, ty_in.map.stride_c, sg,
-                                     *fused);
+                                     static_cast<T>(epsilon), short_tensor(tx_in, sg),
+                                     short_tensor(ty_in, sg), sg, *fused);
         else
             H2X_DISPATCH_SHORT_FUSED(bn_apply_short_kernel, false, grid, static_cast<const T*>(x),
                                      static_cast<const T*>(mean), static_cast<const T*>(var),
                                      static_cast<const T*>(scale), static_cast<const T*>(bias),
                                      static_cast<T*>(y), static_cast<T>(epsilon),
-                                     tx_in.map.stride_n, tx_in.map.stride_c, ty_in.map.stride_n,
-                                     ty_in.map.stride_c, sg, FusedStats<T>());
+                                     short_tensor(tx_in, sg), short_tensor(ty_in, sg), sg, FusedStats<T>());
         return launch_status();
     }
     HostTensor tx = tx_in, ty = ty_in;
@@ -1795,8 +1858,7 @@ int backprop1_impl(int num_samples, int num_channels, size_t spatial, const Host
                            static_cast<const T*>(var), static_cast<const T*>(scale),
                            static_cast<T*>(dscale), static_cast<T*>(dbias), static_cast<T*>(dmean),
                            static_cast<T*>(dvar), static_cast<T>(epsilon), partials,
-                           tx_in.map.stride_n, tx_in.map.stride_c, td_in.map.stride_n,
-                           td_in.map.stride_c, sg, fused_out != nullptr);
+                           short_tensor(tx_in, sg), short_tensor(td_in, sg), sg, fused_out != nullptr);
         if (fused_out)
         {
             fused_out->groups = groups;
@@ -1862,7 +1924,8 @@ int backprop2_impl(int num_samples, int num_channels, size_t spatial, size_t num
         // whether x and dx share memory (the reference allows dx to be x itself)
         const auto span = [&](const HostTensor& t) {
             return (static_cast<size_t>(num_samples - 1) * t.map.stride_n
-                    + static_cast<size_t>(num_channels - 1) * t.map.stride_c + spatial)
+                    + static_cast<size_t>(num_channels - 1) * t.map.stride_c
+                    + short_span(t, spatial))
                    * sizeof(T);
         };
         const char* xb = static_cast<const char*>(x);
@@ -1878,18 +1941,16 @@ int backprop2_impl(int num_samples, int num_channels, size_t spatial, size_t num
                                      static_cast<const T*>(mean), static_cast<const T*>(var),
                                      static_cast<const T*>(scale), nullptr, nullptr,
                                      static_cast<T*>(dx), static_cast<T>(epsilon), num_per_sum,
-                                     tx_in.map.stride_n, tx_in.map.stride_c, td_in.map.stride_n,
-                                     td_in.map.stride_c, to_in.map.stride_n, to_in.map.stride_c, sg,
-                                     disjoint, *fused);
+                                     short_tensor(tx_in, sg), short_tensor(td_in, sg), short_tensor(to_in, sg),
+                                     sg, disjoint, *fused);
         else
             H2X_DISPATCH_SHORT_FUSED(bn_backprop2_short_kernel, false, grid,
                                      static_cast<const T*>(x), static_cast<const T*>(dy),
                                      static_cast<const T*>(mean), static_cast<const T*>(var),
                                      static_cast<const T*>(scale), static_cast<const T*>(dmean),
                                      static_cast<const T*>(dvar), static_cast<T*>(dx),
-                                     static_cast<T>(epsilon), num_per_sum, tx_in.map.stride_n,
-                                     tx_in.map.stride_c, td_in.map.stride_n, td_in.map.stride_c,
-                                     to_in.map.stride_n, to_in.map.stride_c, sg, disjoint,
+                                     static_cast<T>(epsilon), num_per_sum, short_tensor(tx_in, sg),
+                                     short_tensor(td_in, sg), short_tensor(to_in, sg), sg, disjoint,
                                      FusedStats<T>());
         return launch_status();
     }

@@ -294,6 +294,12 @@ HALO_CASES = [
     ((16, 8, 6, 2), (1, 2, 1, 1), (0, 3, 0, 0)),        # halo only on the outermost spatial dimension: dense path
     ((134, 6, 3, 2), (2, 2, 1, 1), (1, 1, 0, 0)),       # haloed rows of 67 elements: vectors split at row ends
     ((130, 4, 6, 2, 2), (2, 1, 2, 1, 1), (2, 0, 1, 0, 0)),  # 5-D, rows of 65
+    # small haloed tiles: the short-segment kernels with each lane's place in the tile worked out once
+    ((28, 28, 40, 3), (2, 2, 1, 1), (1, 1, 0, 0)),      # 14 x 14 in 16 x 16: one vector in seven crosses a row end
+    ((14, 14, 70, 5), (2, 2, 1, 1), (1, 1, 0, 0)),      # 7 x 7 in 9 x 9, odd segment length
+    ((12, 12, 12, 9, 2), (2, 2, 2, 1, 1), (1, 1, 1, 0, 0)),  # 6 x 6 x 6 in 8 x 8 x 8
+    ((16, 16, 30, 4), (2, 2, 1, 1), (2, 2, 0, 0)),      # 8 x 8 with a halo of 2
+    ((6, 6, 300, 33), (2, 3, 1, 1), (1, 1, 0, 0)),      # 3 x 2: shorter than a vector times two, many channels and samples
 ]
 
 
