@@ -1,16 +1,17 @@
 // Channel-wise batch-normalisation kernels for gfx950 and their C entry points.
 //
-// Two layouts (and, for dense tensors whose (sample, channel) segments have at
-// most 256 elements, a third family of kernels that gives a workgroup a window
-// of neighbouring whole channels: see "short segments" below).  Dense: element
+// Two layouts (and, for tensors whose (sample, channel) segments have at most
+// 256 elements, a third family of kernels that gives a workgroup a window of
+// neighbouring whole channels: see "short segments" below).  Dense: element
 // (n, c, i) of a tensor lives at
 // base[(n*C + c)*real + i], i < spatial -- the geometry of the reference's
 // optimised kernels (legacy/src/dnn_backend/batchnorm.cu:134-190).  Strided:
 // the interior of a tensor with halos on any spatial dimension, addressed
 // through the tensor's strides like the reference's generic kernels
-// (batchnorm.cu:39-90,369-418,899-980,1303-1369); the flat interior index of
-// an element is split into (x, y, z) with multiply-high divisions and rows are
-// read with unaligned vectors.  Every kernel is a pure HBM stream: 16-byte
+// (batchnorm.cu:39-90,369-418,899-980,1303-1369); rows are padded to whole
+// vectors, an index is split into (row, vector of the row) with multiply-high
+// divisions, and every vector is one unaligned 16-byte access (see TensorMap).
+// Every kernel is a pure HBM stream: 16-byte
 // accesses when the geometry allows, several loads in flight per lane,
 // per-channel parameters fetched once per workgroup.
 //
@@ -123,18 +124,30 @@ Chunking make_chunking(size_t spatial, size_t segments, size_t budget, size_t ti
     return c;
 }
 
-// Where the elements of one tensor live.  Element i (flat index over the
-// interior spatial extents, innermost first) of segment (n, c) is at
+// Where the elements of one tensor live.  Element i of segment (n, c) is at
 // base[n*stride_n + c*stride_c + offset(i)]; offset(i) = i for the dense layout.
+// Strided layout (tensors with halos inside their segments, samples folded into
+// rows, dense tensors that vectors cannot address aligned): element by element,
+// i is the flat index over the interior extents, innermost first.  With vectors,
+// every row (the `width` contiguous interior elements) is padded to `spr`
+// vectors and i counts the elements of the padded rows: vector k of a row
+// starts at element min(k * VEC, width - VEC), so the last vector of a row that
+// is no multiple of VEC long overlaps the one before it instead of running into
+// the next row, and every vector is contiguous in every tensor of the launch.
+// The `skip` leading elements of such a vector belong to its neighbour:
+// reductions leave them out; elementwise kernels store them twice (the same
+// values) where the output shares no memory with an input, else one by one.
 struct TensorMap
 {
     int64_t stride_n, stride_c;
     FastDiv w, h;     // interior extents of spatial dimensions 0 and 1 (strided layout)
     int64_t sy, sz;   // strides of spatial dimensions 1 and 2 (strided layout)
+    FastDiv spr;      // vectors a row is padded to (strided layout with vectors)
+    uint32_t width;   // elements of a row (strided layout with vectors)
 };
 
 template <bool STRIDED>
-__device__ __forceinline__ size_t seg_offset(const TensorMap& m, size_t i, uint32_t* in_row = nullptr)
+__device__ __forceinline__ size_t seg_offset(const TensorMap& m, size_t i)
 {
     if constexpr (!STRIDED)
     {
@@ -146,10 +159,23 @@ __device__ __forceinline__ size_t seg_offset(const TensorMap& m, size_t i, uint3
         const uint32_t x = static_cast<uint32_t>(i) - t * m.w.divisor;
         const uint32_t z = fastdiv(t, m.h);
         const uint32_t y = t - z * m.h.divisor;
-        if (in_row)
-            *in_row = m.w.divisor - x; // elements from i to the end of its row
         return x + y * static_cast<size_t>(m.sy) + z * static_cast<size_t>(m.sz);
     }
+}
+
+// Offset of the vector at padded index i (a multiple of VEC) and the number of
+// its leading elements that the vector before it owns.
+template <int VEC>
+__device__ __forceinline__ size_t row_vector_offset(const TensorMap& m, size_t i, uint32_t* skip)
+{
+    const uint32_t slot = static_cast<uint32_t>(i) / VEC;
+    const uint32_t r = fastdiv(slot, m.spr);
+    const uint32_t x = (slot - r * m.spr.divisor) * VEC;
+    const uint32_t last = m.width - VEC;
+    *skip = x > last ? x - last : 0;
+    const uint32_t z = fastdiv(r, m.h);
+    const uint32_t y = r - z * m.h.divisor;
+    return (x > last ? last : x) + y * static_cast<size_t>(m.sy) + z * static_cast<size_t>(m.sz);
 }
 
 // ALIGNED: the address is a multiple of the vector size (dense layout); rows
@@ -195,37 +221,30 @@ __device__ __forceinline__ void store_vec(T* p, const T (&r)[VEC])
     }
 }
 
-// The VEC elements from interior index i on.  In the strided layout a vector may
-// run past the end of its row when rows are no multiple of VEC long (rows are at
-// least VEC long, so it touches two rows at most): its two parts are then moved
-// element by element, all other vectors whole (rows of 49 elements: 1 vector in 12).
+// The VEC elements at index i; returns how many of the leading ones belong to
+// the vector before (strided layout with vectors, else 0).
 template <typename T, int VEC, bool STRIDED, bool STREAM = false>
-__device__ __forceinline__ void load_at(const T* p, const TensorMap& m, size_t i, T (&r)[VEC])
+__device__ __forceinline__ uint32_t load_at(const T* p, const TensorMap& m, size_t i, T (&r)[VEC])
 {
     if constexpr (!STRIDED || VEC == 1)
     {
         load_vec<T, VEC, !STRIDED, STREAM>(p + seg_offset<STRIDED>(m, i), r);
+        return 0;
     }
     else
     {
-        uint32_t in_row;
-        const size_t off = seg_offset<true>(m, i, &in_row);
-        if (in_row >= VEC)
-        {
-            load_vec<T, VEC, false, STREAM>(p + off, r);
-        }
-        else
-        {
-            const size_t next = seg_offset<true>(m, i + in_row); // the first element of the next row
-#pragma unroll
-            for (int j = 0; j < VEC; ++j)
-                r[j] = j < static_cast<int>(in_row) ? p[off + j] : p[next + j - in_row];
-        }
+        uint32_t skip;
+        const size_t off = row_vector_offset<VEC>(m, i, &skip);
+        load_vec<T, VEC, false, STREAM>(p + off, r);
+        return skip;
     }
 }
 
+// rewrite: the elements a vector shares with the one before it may be stored
+// by both (the output shares no memory with the inputs they were made from).
 template <typename T, int VEC, bool STRIDED>
-__device__ __forceinline__ void store_at(T* p, const TensorMap& m, size_t i, const T (&r)[VEC])
+__device__ __forceinline__ void store_at(T* p, const TensorMap& m, size_t i, const T (&r)[VEC],
+                                         bool rewrite)
 {
     if constexpr (!STRIDED || VEC == 1)
     {
@@ -233,21 +252,18 @@ __device__ __forceinline__ void store_at(T* p, const TensorMap& m, size_t i, con
     }
     else
     {
-        uint32_t in_row;
-        const size_t off = seg_offset<true>(m, i, &in_row);
-        if (in_row >= VEC)
+        uint32_t skip;
+        const size_t off = row_vector_offset<VEC>(m, i, &skip);
+        if (skip == 0 || rewrite)
         {
             store_vec<T, VEC, false>(p + off, r);
         }
         else
         {
-            const size_t next = seg_offset<true>(m, i + in_row);
 #pragma unroll
-            for (int j = 0; j < VEC; ++j)
-            {
-                const T one[1] = {r[j]};
-                store_vec<T, 1>(j < static_cast<int>(in_row) ? p + off + j : p + next + j - in_row, one);
-            }
+            for (int j = 1; j < VEC; ++j)
+                if (j >= static_cast<int>(skip))
+                    __builtin_nontemporal_store(r[j], p + off + j);
         }
     }
 }
@@ -389,22 +405,25 @@ __global__ __launch_bounds__(kBlockSize) void bn_sums_kernel(
         for (; tile + kTile <= end; tile += kTile)
         {
             T v[kUnroll][VEC];
+            uint32_t skip[kUnroll];
 #pragma unroll
             for (int u = 0; u < kUnroll; ++u)
-                load_at<T, VEC, STRIDED>(p, mx, tile + u * kStride + threadIdx.x * VEC, v[u]);
+                skip[u] = load_at<T, VEC, STRIDED>(p, mx, tile + u * kStride + threadIdx.x * VEC, v[u]);
 #pragma unroll
             for (int u = 0; u < kUnroll; ++u)
 #pragma unroll
                 for (int j = 0; j < VEC; ++j)
-                    accumulate(v[u][j]);
+                    if (j >= static_cast<int>(skip[u]))
+                        accumulate(v[u][j]);
         }
         for (size_t i = tile + threadIdx.x * VEC; i + VEC <= end; i += kStride)
         {
             T v[VEC];
-            load_at<T, VEC, STRIDED>(p, mx, i, v);
+            const uint32_t skip = load_at<T, VEC, STRIDED>(p, mx, i, v);
 #pragma unroll
             for (int j = 0; j < VEC; ++j)
-                accumulate(v[j]);
+                if (j >= static_cast<int>(skip))
+                    accumulate(v[j]);
         }
         if constexpr (VEC > 1)
         {
@@ -531,7 +550,7 @@ __global__ __launch_bounds__(kBlockSize) void bn_apply_kernel(
 #pragma unroll
             for (int j = 0; j < VEC; ++j)
                 v[u][j] = fma_t((v[u][j] - m) * inv_stdev, sc, bi);
-            store_at<T, VEC, STRIDED>(yp, my, tile + u * kStride + threadIdx.x * VEC, v[u]);
+            store_at<T, VEC, STRIDED>(yp, my, tile + u * kStride + threadIdx.x * VEC, v[u], true);
         }
     }
     for (size_t i = tile + threadIdx.x * VEC; i + VEC <= end; i += kStride)
@@ -541,7 +560,7 @@ __global__ __launch_bounds__(kBlockSize) void bn_apply_kernel(
 #pragma unroll
         for (int j = 0; j < VEC; ++j)
             v[j] = fma_t((v[j] - m) * inv_stdev, sc, bi);
-        store_at<T, VEC, STRIDED>(yp, my, i, v);
+        store_at<T, VEC, STRIDED>(yp, my, i, v, true);
     }
     if constexpr (VEC > 1)
     {
@@ -604,27 +623,30 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop1_kernel(
         for (; tile + kTile <= end; tile += kTile)
         {
             T xv[kUnroll2][VEC], dv[kUnroll2][VEC];
+            uint32_t skip[kUnroll2];
 #pragma unroll
             for (int u = 0; u < kUnroll2; ++u)
             {
                 const size_t i = tile + u * kStride + threadIdx.x * VEC;
-                load_at<T, VEC, STRIDED>(xp, mx, i, xv[u]);
+                skip[u] = load_at<T, VEC, STRIDED>(xp, mx, i, xv[u]);
                 load_at<T, VEC, STRIDED, true>(dp, md, i, dv[u]);
             }
 #pragma unroll
             for (int u = 0; u < kUnroll2; ++u)
 #pragma unroll
                 for (int j = 0; j < VEC; ++j)
-                    accumulate(xv[u][j], dv[u][j]);
+                    if (j >= static_cast<int>(skip[u]))
+                        accumulate(xv[u][j], dv[u][j]);
         }
         for (size_t i = tile + threadIdx.x * VEC; i + VEC <= end; i += kStride)
         {
             T xv[VEC], dv[VEC];
-            load_at<T, VEC, STRIDED>(xp, mx, i, xv);
+            const uint32_t skip = load_at<T, VEC, STRIDED>(xp, mx, i, xv);
             load_at<T, VEC, STRIDED, true>(dp, md, i, dv);
 #pragma unroll
             for (int j = 0; j < VEC; ++j)
-                accumulate(xv[j], dv[j]);
+                if (j >= static_cast<int>(skip))
+                    accumulate(xv[j], dv[j]);
         }
         if constexpr (VEC > 1)
         {
@@ -650,14 +672,14 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop1_kernel(
 // ---- backward: input gradient ------------------------------------------------
 // Replaces backprop2_opt_kernel, batchnorm.cu:1371-1418.  x and dx may alias:
 // each thread reads its elements before it writes them, so neither is
-// restrict-qualified.
+// restrict-qualified (`disjoint`: they share no memory).
 template <typename T, int VEC, bool STRIDED, bool FUSED = false>
 __global__ __launch_bounds__(kBlockSize) void bn_backprop2_kernel(
     const T* x, const T* __restrict__ dy, const T* __restrict__ mean,
     const T* __restrict__ var, const T* __restrict__ scale, const T* __restrict__ dmean,
     const T* __restrict__ dvar, T* dx, T epsilon, size_t num_per_sum, int num_channels,
     size_t spatial, const TensorMap mx, const TensorMap md, const TensorMap mo, size_t chunk,
-    int chunks_per_seg, const FusedStats<T> fused = FusedStats<T>())
+    int chunks_per_seg, bool disjoint, const FusedStats<T> fused = FusedStats<T>())
 {
     const size_t seg = blockIdx.x / chunks_per_seg;
     const int k = blockIdx.x - seg * chunks_per_seg;
@@ -719,7 +741,7 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop2_kernel(
                 T r = fma_t(dv[u][j] * sc, inv_stdev, dmean_term);
                 xv[u][j] = fma_t(xv[u][j] - m, dvar_term, r);
             }
-            store_at<T, VEC, STRIDED>(op, mo, tile + u * kStride + threadIdx.x * VEC, xv[u]);
+            store_at<T, VEC, STRIDED>(op, mo, tile + u * kStride + threadIdx.x * VEC, xv[u], disjoint);
         }
     }
     for (size_t i = tile + threadIdx.x * VEC; i + VEC <= end; i += kStride)
@@ -733,7 +755,7 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop2_kernel(
             T r = fma_t(dv[j] * sc, inv_stdev, dmean_term);
             xv[j] = fma_t(xv[j] - m, dvar_term, r);
         }
-        store_at<T, VEC, STRIDED>(op, mo, i, xv);
+        store_at<T, VEC, STRIDED>(op, mo, i, xv, disjoint);
     }
     if constexpr (VEC > 1)
     {
@@ -768,7 +790,14 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop2_kernel(
 // owns are added up or stored (kTailOverlap; in place of x, dx may be written
 // by the neighbouring lane before this lane reads the overlap, which it does
 // not use).  Segments shorter than a vector move element by element
-// (kTailScalar).  Where few
+// (kTailScalar).  When a tensor of the launch has halos inside its segments
+// the slots follow the rows of the segment instead (each row padded to whole
+// vectors, the last vector of a row overlapping the one before it), so that a
+// slot is contiguous in every tensor; where it starts in each tensor is worked
+// out once, as the lane's place in the segment never changes (N 32, C 512,
+// 14 x 14 with a halo of 1: forward 34 -> 14 us, backward 46 -> 20 us against
+// the strided kernels, which give such a segment a workgroup of its own).
+// Where few
 // channels and many samples would leave a reduction with too few workgroups,
 // the lanes of a workgroup form `rows` rows that take every rows-th sample of
 // a narrower window.
@@ -1330,6 +1359,8 @@ void set_dense_map(TensorMap* m)
     m->w = make_fastdiv(0x7fffffffu);
     m->h = make_fastdiv(1);
     m->sy = m->sz = 0;
+    m->spr = make_fastdiv(1);
+    m->width = 0;
 }
 
 template <typename T>
@@ -1395,6 +1426,8 @@ int strided_tensor(const h2x_tensor_geometry* g, const void* p, int num_samples,
         t.map.h = make_fastdiv(ns > 1 ? static_cast<uint32_t>(g->local_shape[1]) : 1u);
         t.map.sy = ns > 1 ? g->strides[1] : 0;
         t.map.sz = ns > 2 ? g->strides[2] : 0;
+        t.map.spr = make_fastdiv(1);
+        t.map.width = 0;
         t.aligned = false;
     }
     *out = t;
@@ -1403,11 +1436,10 @@ int strided_tensor(const h2x_tensor_geometry* g, const void* p, int num_samples,
 
 // Vector width all tensors of a launch allow, and whether the strided kernels are needed.
 // Dense tensors whose segments are no multiple of the vector long, or start off a
-// 16-byte boundary, are handed to the strided kernels too: those address a dense
-// tensor with the index itself, use vectors aligned to one element, and finish the
-// last few elements of a segment one by one (N 16, C 64, 57 x 57: forward 23 -> 15 us).
+// 16-byte boundary, are handed to the strided kernels too, as tensors with one row
+// per segment: vectors aligned to one element, the last one of a segment overlapping
+// the one before it (N 16, C 64, 57 x 57: forward 23 -> 15 us against element by element).
 constexpr size_t kMinUnalignedSegment = 256;
-constexpr size_t kMinRaggedRow = 64;
 
 template <typename T>
 int common_vector(std::initializer_list<const HostTensor*> ts, bool* strided)
@@ -1433,15 +1465,43 @@ int common_vector(std::initializer_list<const HostTensor*> ts, bool* strided)
         *strided = true;
         return full;
     }
-    // Rows of a strided tensor hold whole vectors, or are long enough for the vectors that run
-    // past the end of a row (and are split in two, element by element) to be few: with rows
-    // of 49 elements every wave has some and the gain is gone (N 256, C 2048, folded rows of 49:
-    // forward 102 -> 110 us), with 169 and 729 it is a third (N 32, C 256, 27 x 27: 30 -> 19 us).
-    // Dense tensors in a strided launch are addressed with i itself: rows do not matter.
+    // a row of a strided tensor must hold a vector
     for (const HostTensor* t : ts)
-        if (t->strided && t->row % full != 0 && t->row < kMinRaggedRow)
+        if (t->strided && t->row < static_cast<size_t>(full))
             return 1;
     return full;
+}
+
+// Sets the tensors of a strided launch with vectors up for padded rows (see
+// TensorMap) and returns the padded length of a segment.  The rows are those of
+// the tensors with halos or folded samples; a launch of dense tensors only has
+// one row per segment.  Dense tensors in a launch with rows are addressed row by
+// row like the others.
+template <typename T>
+size_t pad_rows(std::initializer_list<HostTensor*> ts, size_t spatial)
+{
+    const uint32_t vec = full_vec<T>();
+    size_t width = spatial;
+    uint32_t rows_per_plane = 1;
+    for (const HostTensor* t : ts)
+        if (t->strided)
+        {
+            width = t->row;
+            rows_per_plane = t->map.h.divisor;
+        }
+    const size_t spr = (width + vec - 1) / vec;
+    for (HostTensor* t : ts)
+    {
+        if (!t->strided)
+        {
+            t->map.h = make_fastdiv(rows_per_plane);
+            t->map.sy = static_cast<int64_t>(width);
+            t->map.sz = static_cast<int64_t>(width) * rows_per_plane;
+        }
+        t->map.spr = make_fastdiv(static_cast<uint32_t>(spr));
+        t->map.width = static_cast<uint32_t>(width);
+    }
+    return spatial / width * spr * vec;
 }
 
 // Segments of 257 to 1023 elements (19 x 19, 27 x 27, 28 x 28 activations; shorter
@@ -1729,6 +1789,10 @@ int sums_impl(int num_samples, int num_channels, size_t spatial, const HostTenso
         return H2X_ERR_TOO_LARGE;
     bool strided;
     const int vw = common_vector<T>({&tx}, &strided);
+    if (strided && vw > 1)
+        spatial = pad_rows<T>({&tx}, spatial);
+    if (spatial >= (1ull << 31) && strided)
+        return H2X_ERR_TOO_LARGE;
     const int gmax = max_groups_per_channel(num_channels);
     const size_t tile = static_cast<size_t>(kBlockSize) * vw * kUnroll;
     const Chunking ch = make_chunking(spatial, num_samples, gmax, tile, tile);
@@ -1815,6 +1879,10 @@ int apply_impl(int num_samples, int num_channels, size_t spatial, const HostTens
     const size_t segments = static_cast<size_t>(num_samples) * num_channels;
     bool strided;
     const int vw = common_vector<T>({&tx, &ty}, &strided);
+    if (strided && vw > 1)
+        spatial = pad_rows<T>({&tx, &ty}, spatial);
+    if (spatial >= (1ull << 31) && strided)
+        return H2X_ERR_TOO_LARGE;
     const Chunking ch = elementwise_chunking(spatial, segments, vw, kUnroll);
     const size_t blocks = segments * ch.chunks_per_seg;
     if (!grid_ok(blocks))
@@ -1878,6 +1946,10 @@ int backprop1_impl(int num_samples, int num_channels, size_t spatial, const Host
         return H2X_ERR_TOO_LARGE;
     bool strided;
     const int vw = common_vector<T>({&tx, &td}, &strided);
+    if (strided && vw > 1)
+        spatial = pad_rows<T>({&tx, &td}, spatial);
+    if (spatial >= (1ull << 31) && strided)
+        return H2X_ERR_TOO_LARGE;
     const int gmax = max_groups_per_channel(num_channels);
     const size_t tile = static_cast<size_t>(kBlockSize) * vw * (kUnroll / 2);
     const Chunking ch = make_chunking(spatial, num_samples, gmax, tile, tile);
@@ -1919,18 +1991,17 @@ int backprop2_impl(int num_samples, int num_channels, size_t spatial, size_t num
         short_segments<T>(num_samples, num_channels, spatial, {&tx_in, &td_in, &to_in}, &sg);
     if (fused && fused->sequential != is_short)
         return H2X_ERR_UNSUPPORTED; // the partials are laid out for the other family of kernels
+    // whether x and dx share memory (the reference allows dx to be x itself)
+    const auto span = [&](const HostTensor& t) {
+        return (static_cast<size_t>(num_samples - 1) * t.map.stride_n
+                + static_cast<size_t>(num_channels - 1) * t.map.stride_c + short_span(t, spatial))
+               * sizeof(T);
+    };
+    const char* xb = static_cast<const char*>(x);
+    const char* ob = static_cast<const char*>(dx);
+    const bool disjoint = xb + span(tx_in) <= ob || ob + span(to_in) <= xb;
     if (is_short)
     {
-        // whether x and dx share memory (the reference allows dx to be x itself)
-        const auto span = [&](const HostTensor& t) {
-            return (static_cast<size_t>(num_samples - 1) * t.map.stride_n
-                    + static_cast<size_t>(num_channels - 1) * t.map.stride_c
-                    + short_span(t, spatial))
-                   * sizeof(T);
-        };
-        const char* xb = static_cast<const char*>(x);
-        const char* ob = static_cast<const char*>(dx);
-        const bool disjoint = xb + span(tx_in) <= ob || ob + span(to_in) <= xb;
         const dim3 grid(short_windows(sg),
                         short_elementwise_groups(&sg, kUnroll / 2,
                                                  fused ? fused->groups * 4 * sizeof(double) : 0,
@@ -1961,6 +2032,10 @@ int backprop2_impl(int num_samples, int num_channels, size_t spatial, size_t num
     const size_t segments = static_cast<size_t>(num_samples) * num_channels;
     bool strided;
     const int vw = common_vector<T>({&tx, &td, &to}, &strided);
+    if (strided && vw > 1)
+        spatial = pad_rows<T>({&tx, &td, &to}, spatial);
+    if (spatial >= (1ull << 31) && strided)
+        return H2X_ERR_TOO_LARGE;
     const Chunking ch = elementwise_chunking(spatial, segments, vw, kUnroll / 2);
     const size_t blocks = segments * ch.chunks_per_seg;
     if (!grid_ok(blocks))
@@ -1972,14 +2047,14 @@ int backprop2_impl(int num_samples, int num_channels, size_t spatial, size_t num
                            static_cast<const T*>(var), static_cast<const T*>(scale), nullptr,
                            nullptr, static_cast<T*>(dx), static_cast<T>(epsilon), num_per_sum,
                            num_channels, spatial, tx.map, td.map, to.map, ch.chunk,
-                           ch.chunks_per_seg, *fused);
+                           ch.chunks_per_seg, disjoint, *fused);
     else
         H2X_DISPATCH(bn_backprop2_kernel, grid, static_cast<const T*>(x), static_cast<const T*>(dy),
                      static_cast<const T*>(mean), static_cast<const T*>(var),
                      static_cast<const T*>(scale), static_cast<const T*>(dmean),
                      static_cast<const T*>(dvar), static_cast<T*>(dx), static_cast<T>(epsilon),
                      num_per_sum, num_channels, spatial, tx.map, td.map, to.map, ch.chunk,
-                     ch.chunks_per_seg);
+                     ch.chunks_per_seg, disjoint);
     return launch_status();
 }
 
