@@ -381,21 +381,21 @@ def cpu_baseline(repeats: int = 5):
 # TCC_EA0_WRREQ_64B), request counts summed over the L2 channels, per dispatch.
 # label -> (bytes read, bytes written) per launch
 PMC_TRAFFIC = {
-    "bn_sums": (268460032, 131072),
-    "bn_apply": (268466688, 268500864),
-    "bn_backprop1": (536914496, 131072),
-    "bn_backprop2": (536907264, 268435840),
-    "halo_dim0_pack": (149690480, 8652800),    # 4 faces (2 ranks) a launch, four launches a step
-    "halo_dim0_unpack": (9217280, 43264000),
+    "bn_sums": (268460544, 131072),
+    "bn_apply": (268466176, 268483200),
+    "bn_backprop1": (536915328, 131072),
+    "bn_backprop2": (536907776, 268435456),
+    "halo_dim0_pack": (149477968, 8652800),    # 4 faces (2 ranks) a launch, four launches a step
+    "halo_dim0_unpack": (9218224, 43264000),
     "halo_dim1_pack": (42624768, 34611200),
-    "halo_dim1_unpack": (34637568, 36216896),
+    "halo_dim1_unpack": (34637504, 36216128),
     "halo_dim2_pack": (34694400, 34611200),
-    "halo_dim2_unpack": (34637568, 34619392),
+    "halo_dim2_unpack": (34637568, 34619488),
 }
 # sha256 (first 16 hex digits) of the kernel sources the table was measured with, see
 # kernel_sources_sha(); with other sources the traffic fields are omitted
-PMC_SOURCES_SHA = "cd50224aa3e20ce5"
-PMC_COMMIT = "22857ea"
+PMC_SOURCES_SHA = "e8f4000d51cee6f5"
+PMC_COMMIT = "cccf888"
 
 KERNEL_OF = {
     "bn_sums": "bn_sums_kernel<float,4> (+bn_finish_kernel<float,2>)",
