@@ -34,8 +34,9 @@ def test_static_scratch_entry_point_matches_workspace_entry_point():
     lib = capi.load()
     g = torch.Generator(device="cuda").manual_seed(99)
     # first a large input (many workgroups per channel), then a smaller one with
-    # fewer channels and fewer partial sums per channel
-    for shape in ((4, 64, 32, 32, 32), (2, 5, 7, 9, 11)):
+    # fewer channels and fewer partial sums per channel, then short segments (another
+    # family of kernels, which lays its partial sums out range by range)
+    for shape in ((4, 64, 32, 32, 32), (2, 5, 7, 9, 11), (300, 40, 7, 7), (3, 70, 14, 14)):
         x = torch.empty(shape, device="cuda").normal_(0, 1, generator=g)
         want = _sums(lib, capi, torch, x, static=False)
         got = _sums(lib, capi, torch, x, static=True)
