@@ -10,8 +10,9 @@
 // (legacy/src/dnn_backend/softmax.cu:538-593,621-669).  Above 32 channels the
 // four waves of a workgroup share the channels of 64 * VEC pixels, still in
 // registers; channel counts beyond the largest such tile fall back to a kernel
-// that re-reads its inputs; tensors with one pixel per sample have a kernel
-// that puts the channels, which are contiguous then, on the lanes of a wave.
+// that re-reads its inputs; tensors with one pixel per sample have kernels
+// that put the channels, which are contiguous then, on the lanes of a wave or,
+// beyond 2048 channels, on the threads of a workgroup.
 #include "h2x_device.hpp"
 
 #include <cfloat>
@@ -555,6 +556,72 @@ __global__ __launch_bounds__(kBlockSize) void softmax_bwd_row_kernel(
             dx[base + lane + k * kWaveSize] = yv[k] > kMin ? yv[k] * (gv[k] - dp) : T(0);
 }
 
+// One pixel per sample and more channels than a wave holds in registers: a
+// workgroup takes a sample and walks its channels (contiguous) three times
+// forward, twice backward; the re-reads come from the L2.  Thread t adds up the
+// channels t, t + 256, ...; the lanes of a wave are combined as a butterfly and
+// the waves through LDS in wave order.
+template <typename T>
+__device__ __forceinline__ T block_combine(T v, bool is_max, T* lds)
+{
+#pragma unroll
+    for (int m = kWaveSize / 2; m >= 1; m >>= 1)
+    {
+        const T o = __shfl_xor(v, m, kWaveSize);
+        v = is_max ? (o > v ? o : v) : v + o;
+    }
+    __syncthreads(); // lds may still be read from the previous call
+    if ((threadIdx.x & (kWaveSize - 1)) == 0)
+        lds[threadIdx.x / kWaveSize] = v;
+    __syncthreads();
+    T r = lds[0];
+#pragma unroll
+    for (int w = 1; w < kWavesPerBlock; ++w)
+        r = is_max ? (lds[w] > r ? lds[w] : r) : r + lds[w];
+    return r;
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlockSize) void softmax_fwd_long_row_kernel(
+    const T* __restrict__ x, T* __restrict__ y, int num_channels)
+{
+    __shared__ T lds[kWavesPerBlock];
+    const T* xp = x + static_cast<size_t>(blockIdx.x) * num_channels;
+    T* yp = y + static_cast<size_t>(blockIdx.x) * num_channels;
+    constexpr T kMin = Limits<T>::min_normal;
+    T mx = kMin;
+    for (int c = threadIdx.x; c < num_channels; c += kBlockSize)
+        mx = xp[c] > mx ? xp[c] : mx;
+    mx = block_combine(mx, true, lds);
+    T sum = T(0);
+    for (int c = threadIdx.x; c < num_channels; c += kBlockSize)
+        sum += exp_t(xp[c] - mx);
+    const T inv = T(1) / block_combine(sum, false, lds);
+    for (int c = threadIdx.x; c < num_channels; c += kBlockSize)
+    {
+        const T r = exp_t(xp[c] - mx) * inv;
+        yp[c] = r > kMin ? r : kMin;
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlockSize) void softmax_bwd_long_row_kernel(
+    const T* __restrict__ y, const T* __restrict__ dy, T* __restrict__ dx, int num_channels)
+{
+    __shared__ T lds[kWavesPerBlock];
+    const size_t base = static_cast<size_t>(blockIdx.x) * num_channels;
+    constexpr T kMin = Limits<T>::min_normal;
+    T dp = T(0);
+    for (int c = threadIdx.x; c < num_channels; c += kBlockSize)
+        dp = fma_t(y[base + c], dy[base + c], dp);
+    dp = block_combine(dp, false, lds);
+    for (int c = threadIdx.x; c < num_channels; c += kBlockSize)
+    {
+        const T yi = y[base + c];
+        dx[base + c] = yi > kMin ? yi * (dy[base + c] - dp) : T(0);
+    }
+}
+
 // Largest vector (elements) usable for all of the given pointers.
 template <typename T>
 int vector_width(size_t spatial, int want, std::initializer_list<const void*> ptrs)
@@ -656,6 +723,8 @@ int forward_impl(int n, int c, size_t s, const void* xv, void* yv, hipStream_t s
         if (c <= 16 * kWaveSize) H2X_FWD_ROW(16);
         if (c <= 32 * kWaveSize) H2X_FWD_ROW(32);
 #undef H2X_FWD_ROW
+        softmax_fwd_long_row_kernel<T><<<n, kBlockSize, 0, st>>>(x, y, c);
+        return launch_status();
     }
     const int v4 = vector_width<T>(s, 4 / kWords, {xv, yv});
 #define H2X_FWD(V, CM)                                                                             \
@@ -739,6 +808,8 @@ int backward_impl(int n, int c, size_t s, const void* yv, const void* dyv, void*
         if (c <= 16 * kWaveSize) H2X_BWD_ROW(16);
         if (c <= 32 * kWaveSize) H2X_BWD_ROW(32);
 #undef H2X_BWD_ROW
+        softmax_bwd_long_row_kernel<T><<<n, kBlockSize, 0, st>>>(y, dy, dx, c);
+        return launch_status();
     }
     const int v4 = vector_width<T>(s, 4 / kWords, {yv, dyv, dxv});
 #define H2X_BWD(V, CM)                                                                             \

@@ -27,7 +27,8 @@ CASES = [
     (4, 1000, 1, 1),      # one pixel per sample: a wave per sample, lanes over the channels
     (70, 10, 1, 1),       # the same with fewer channels than lanes
     (3, 2048, 1, 1),      # 32 channels a lane, the most
-    (2, 2100, 1, 1),      # beyond that: the re-reading kernel
+    (2, 2100, 1, 1),      # beyond that: a workgroup per sample
+    (3, 40000, 1, 1),     # a large vocabulary
     (2, 19, 4, 6, 10),    # 5-D
     (2, 256, 6, 10),      # 64 channels a wave in registers, two pixels a lane
     (2, 257, 3, 5),       # 65 of 128 channels a wave, one pixel a lane
