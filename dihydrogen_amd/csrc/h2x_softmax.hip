@@ -159,6 +159,8 @@ __global__ __launch_bounds__(kBlockSize) void softmax_fwd_reg_kernel(
         }
 }
 
+constexpr int kWideBatch = 8;
+
 // forward, any channel count.  A workgroup serves 64 neighbouring pixels; its
 // four waves share the channels (wave g takes c = g, g + 4, ...), combine their
 // maxima and sums through LDS in wave order, and walk their channels again for
@@ -179,12 +181,23 @@ __global__ __launch_bounds__(kBlockSize) void softmax_fwd_wide_kernel(
     T* yp = y + base;
     constexpr T kMin = Limits<T>::min_normal;
 
+    // kWideBatch loads are issued together in every pass: the channel loop of a
+    // wave is a chain of dependent operations on values that are a memory
+    // latency away each (N 8, C 1000, 64 x 64 backward: 334 us one by one)
+    constexpr int kStep = kWavesPerBlock * kWideBatch;
     T mx = kMin;
     if (active)
-        for (int c = g; c < num_channels; c += kWavesPerBlock)
+        for (int c0 = g; c0 < num_channels; c0 += kStep)
         {
-            const T v = xp[static_cast<size_t>(c) * spatial];
-            mx = v > mx ? v : mx;
+            T v[kWideBatch];
+#pragma unroll
+            for (int u = 0; u < kWideBatch; ++u)
+                if (c0 + u * kWavesPerBlock < num_channels)
+                    v[u] = xp[static_cast<size_t>(c0 + u * kWavesPerBlock) * spatial];
+#pragma unroll
+            for (int u = 0; u < kWideBatch; ++u)
+                if (c0 + u * kWavesPerBlock < num_channels)
+                    mx = v[u] > mx ? v[u] : mx;
         }
     lds[g][lane] = mx;
     __syncthreads();
@@ -195,8 +208,18 @@ __global__ __launch_bounds__(kBlockSize) void softmax_fwd_wide_kernel(
 
     T sum = T(0);
     if (active)
-        for (int c = g; c < num_channels; c += kWavesPerBlock)
-            sum += exp_t(xp[static_cast<size_t>(c) * spatial] - mx);
+        for (int c0 = g; c0 < num_channels; c0 += kStep)
+        {
+            T v[kWideBatch];
+#pragma unroll
+            for (int u = 0; u < kWideBatch; ++u)
+                if (c0 + u * kWavesPerBlock < num_channels)
+                    v[u] = xp[static_cast<size_t>(c0 + u * kWavesPerBlock) * spatial];
+#pragma unroll
+            for (int u = 0; u < kWideBatch; ++u)
+                if (c0 + u * kWavesPerBlock < num_channels)
+                    sum += exp_t(v[u] - mx);
+        }
     lds[g][lane] = sum;
     __syncthreads();
     sum = lds[0][lane];
@@ -206,10 +229,20 @@ __global__ __launch_bounds__(kBlockSize) void softmax_fwd_wide_kernel(
     const T inv = T(1) / sum;
 
     if (active)
-        for (int c = g; c < num_channels; c += kWavesPerBlock)
+        for (int c0 = g; c0 < num_channels; c0 += kStep)
         {
-            const T r = exp_t(xp[static_cast<size_t>(c) * spatial] - mx) * inv;
-            yp[static_cast<size_t>(c) * spatial] = r > kMin ? r : kMin;
+            T v[kWideBatch];
+#pragma unroll
+            for (int u = 0; u < kWideBatch; ++u)
+                if (c0 + u * kWavesPerBlock < num_channels)
+                    v[u] = xp[static_cast<size_t>(c0 + u * kWavesPerBlock) * spatial];
+#pragma unroll
+            for (int u = 0; u < kWideBatch; ++u)
+                if (c0 + u * kWavesPerBlock < num_channels)
+                {
+                    const T r = exp_t(v[u] - mx) * inv;
+                    yp[static_cast<size_t>(c0 + u * kWavesPerBlock) * spatial] = r > kMin ? r : kMin;
+                }
         }
 }
 
@@ -278,10 +311,24 @@ __global__ __launch_bounds__(kBlockSize) void softmax_bwd_wide_kernel(
     T* op = dx + base;
     constexpr T kMin = Limits<T>::min_normal;
 
+    constexpr int kStep = kWavesPerBlock * kWideBatch;
     T dp = T(0);
     if (active)
-        for (int c = g; c < num_channels; c += kWavesPerBlock)
-            dp = fma_t(yp[static_cast<size_t>(c) * spatial], gp[static_cast<size_t>(c) * spatial], dp);
+        for (int c0 = g; c0 < num_channels; c0 += kStep)
+        {
+            T yv[kWideBatch], gv[kWideBatch];
+#pragma unroll
+            for (int u = 0; u < kWideBatch; ++u)
+                if (c0 + u * kWavesPerBlock < num_channels)
+                {
+                    yv[u] = yp[static_cast<size_t>(c0 + u * kWavesPerBlock) * spatial];
+                    gv[u] = gp[static_cast<size_t>(c0 + u * kWavesPerBlock) * spatial];
+                }
+#pragma unroll
+            for (int u = 0; u < kWideBatch; ++u)
+                if (c0 + u * kWavesPerBlock < num_channels)
+                    dp = fma_t(yv[u], gv[u], dp);
+        }
     lds[g][lane] = dp;
     __syncthreads();
     dp = lds[0][lane];
@@ -290,28 +337,39 @@ __global__ __launch_bounds__(kBlockSize) void softmax_bwd_wide_kernel(
         dp += lds[w][lane];
 
     if (active)
-        for (int c = g; c < num_channels; c += kWavesPerBlock)
+        for (int c0 = g; c0 < num_channels; c0 += kStep)
         {
-            const T yi = yp[static_cast<size_t>(c) * spatial];
-            op[static_cast<size_t>(c) * spatial] =
-                yi > kMin ? yi * (gp[static_cast<size_t>(c) * spatial] - dp) : T(0);
+            T yv[kWideBatch], gv[kWideBatch];
+#pragma unroll
+            for (int u = 0; u < kWideBatch; ++u)
+                if (c0 + u * kWavesPerBlock < num_channels)
+                {
+                    yv[u] = yp[static_cast<size_t>(c0 + u * kWavesPerBlock) * spatial];
+                    gv[u] = gp[static_cast<size_t>(c0 + u * kWavesPerBlock) * spatial];
+                }
+#pragma unroll
+            for (int u = 0; u < kWideBatch; ++u)
+                if (c0 + u * kWavesPerBlock < num_channels)
+                    op[static_cast<size_t>(c0 + u * kWavesPerBlock) * spatial] =
+                        yv[u] > kMin ? yv[u] * (gv[u] - dp) : T(0);
         }
 }
 
-// forward, up to 4 * CPW channels, register-resident.  A workgroup serves
-// 64 * VEC neighbouring pixels; its four waves share the channels (wave g takes
-// c = g, g + 4, ...: CPW of them at most) and keep their values in registers, so
+// forward, up to WAVES * CPW channels, register-resident.  A workgroup serves
+// 64 * VEC neighbouring pixels; its WAVES (four, or eight above 512 channels)
+// waves share the channels (wave g takes c = g, g + WAVES, ...: CPW of them at
+// most) and keep their values in registers, so
 // x is read once; maxima and sums are combined through LDS in wave order.  The
 // arithmetic, partial sums included, is that of softmax_fwd_wide_kernel, which
 // re-reads its tile twice and whose tiles of 64 * C elements the L2 does not
 // hold once every CU runs eight of them (N 16, C 150, 128 x 128: 100 us there,
 // 60 us with the tile in registers).
-template <typename T, int VEC, int CPW>
-__global__ __launch_bounds__(kBlockSize) void softmax_fwd_split_kernel(
+template <typename T, int VEC, int CPW, int WAVES>
+__global__ __launch_bounds__(WAVES * kWaveSize) void softmax_fwd_split_kernel(
     const T* __restrict__ x, T* __restrict__ y, int num_channels, size_t spatial)
 {
     using P = Pack<T, VEC>;
-    __shared__ T lds[kWavesPerBlock][kWaveSize * VEC];
+    __shared__ T lds[WAVES][kWaveSize * VEC];
     const int lane = threadIdx.x % kWaveSize;
     const int g = threadIdx.x / kWaveSize;
     const size_t s =
@@ -334,11 +392,11 @@ __global__ __launch_bounds__(kBlockSize) void softmax_fwd_split_kernel(
     {
 #pragma unroll
         for (int k = 0; k < CPW; ++k)
-            if (g + k * kWavesPerBlock < num_channels)
-                v[k] = P::load(xp + static_cast<size_t>(g + k * kWavesPerBlock) * spatial);
+            if (g + k * WAVES < num_channels)
+                v[k] = P::load(xp + static_cast<size_t>(g + k * WAVES) * spatial);
 #pragma unroll
         for (int k = 0; k < CPW; ++k)
-            if (g + k * kWavesPerBlock < num_channels)
+            if (g + k * WAVES < num_channels)
 #pragma unroll
                 for (int j = 0; j < VEC; ++j)
                     mx[j] = v[k][j] > mx[j] ? v[k][j] : mx[j];
@@ -350,7 +408,7 @@ __global__ __launch_bounds__(kBlockSize) void softmax_fwd_split_kernel(
 #pragma unroll
     for (int j = 0; j < VEC; ++j)
 #pragma unroll
-        for (int w = 0; w < kWavesPerBlock; ++w)
+        for (int w = 0; w < WAVES; ++w)
             mx[j] = lds[w][lane * VEC + j] > mx[j] ? lds[w][lane * VEC + j] : mx[j];
     __syncthreads();
 
@@ -358,7 +416,7 @@ __global__ __launch_bounds__(kBlockSize) void softmax_fwd_split_kernel(
     {
 #pragma unroll
         for (int k = 0; k < CPW; ++k)
-            if (g + k * kWavesPerBlock < num_channels)
+            if (g + k * WAVES < num_channels)
 #pragma unroll
                 for (int j = 0; j < VEC; ++j)
                 {
@@ -377,7 +435,7 @@ __global__ __launch_bounds__(kBlockSize) void softmax_fwd_split_kernel(
     {
         T t = lds[0][lane * VEC + j];
 #pragma unroll
-        for (int w = 1; w < kWavesPerBlock; ++w)
+        for (int w = 1; w < WAVES; ++w)
             t += lds[w][lane * VEC + j];
         inv[j] = T(1) / t;
     }
@@ -385,7 +443,7 @@ __global__ __launch_bounds__(kBlockSize) void softmax_fwd_split_kernel(
     {
 #pragma unroll
         for (int k = 0; k < CPW; ++k)
-            if (g + k * kWavesPerBlock < num_channels)
+            if (g + k * WAVES < num_channels)
             {
 #pragma unroll
                 for (int j = 0; j < VEC; ++j)
@@ -393,19 +451,19 @@ __global__ __launch_bounds__(kBlockSize) void softmax_fwd_split_kernel(
                     const T r = v[k][j] * inv[j];
                     v[k][j] = r > kMin ? r : kMin;
                 }
-                P::store(yp + static_cast<size_t>(g + k * kWavesPerBlock) * spatial, v[k]);
+                P::store(yp + static_cast<size_t>(g + k * WAVES) * spatial, v[k]);
             }
     }
 }
 
-// backward likewise: y and dy of up to 4 * CPW channels in registers.
-template <typename T, int VEC, int CPW>
-__global__ __launch_bounds__(kBlockSize) void softmax_bwd_split_kernel(
+// backward likewise: y and dy of up to WAVES * CPW channels in registers.
+template <typename T, int VEC, int CPW, int WAVES>
+__global__ __launch_bounds__(WAVES * kWaveSize) void softmax_bwd_split_kernel(
     const T* __restrict__ y, const T* __restrict__ dy, T* __restrict__ dx, int num_channels,
     size_t spatial)
 {
     using P = Pack<T, VEC>;
-    __shared__ T lds[kWavesPerBlock][kWaveSize * VEC];
+    __shared__ T lds[WAVES][kWaveSize * VEC];
     const int lane = threadIdx.x % kWaveSize;
     const int g = threadIdx.x / kWaveSize;
     const size_t s =
@@ -426,14 +484,14 @@ __global__ __launch_bounds__(kBlockSize) void softmax_bwd_split_kernel(
     {
 #pragma unroll
         for (int k = 0; k < CPW; ++k)
-            if (g + k * kWavesPerBlock < num_channels)
+            if (g + k * WAVES < num_channels)
             {
-                yv[k] = P::load(yp + static_cast<size_t>(g + k * kWavesPerBlock) * spatial);
-                gv[k] = P::load(gp + static_cast<size_t>(g + k * kWavesPerBlock) * spatial);
+                yv[k] = P::load(yp + static_cast<size_t>(g + k * WAVES) * spatial);
+                gv[k] = P::load(gp + static_cast<size_t>(g + k * WAVES) * spatial);
             }
 #pragma unroll
         for (int k = 0; k < CPW; ++k)
-            if (g + k * kWavesPerBlock < num_channels)
+            if (g + k * WAVES < num_channels)
 #pragma unroll
                 for (int j = 0; j < VEC; ++j)
                     dp[j] = fma_t(yv[k][j], gv[k][j], dp[j]);
@@ -447,7 +505,7 @@ __global__ __launch_bounds__(kBlockSize) void softmax_bwd_split_kernel(
     {
         T t = lds[0][lane * VEC + j];
 #pragma unroll
-        for (int w = 1; w < kWavesPerBlock; ++w)
+        for (int w = 1; w < WAVES; ++w)
             t += lds[w][lane * VEC + j];
         dp[j] = t;
     }
@@ -455,12 +513,12 @@ __global__ __launch_bounds__(kBlockSize) void softmax_bwd_split_kernel(
     {
 #pragma unroll
         for (int k = 0; k < CPW; ++k)
-            if (g + k * kWavesPerBlock < num_channels)
+            if (g + k * WAVES < num_channels)
             {
 #pragma unroll
                 for (int j = 0; j < VEC; ++j)
                     yv[k][j] = yv[k][j] > kMin ? yv[k][j] * (gv[k][j] - dp[j]) : T(0);
-                P::store(op + static_cast<size_t>(g + k * kWavesPerBlock) * spatial, yv[k]);
+                P::store(op + static_cast<size_t>(g + k * WAVES) * spatial, yv[k]);
             }
     }
 }
@@ -685,19 +743,21 @@ void launch_bwd(const T* y, const T* dy, T* dx, int n, int c, size_t s, hipStrea
 // instead of 150 us, N 8, C 256, 64 x 64 18 instead of 59 us and 19 instead of
 // 55 us.  Tiles wider than needed cost time (every lane walks the whole tile
 // under a predicate), hence the steps of 16.  More channels than the largest
-// tile holds (512; double: 256) take the re-reading kernel.
-template <typename T, int VEC, int CPW>
+// tile holds (eight waves: 1024 forward, 768 backward; double: 256) take the
+// re-reading kernel.
+template <typename T, int VEC, int CPW, int WAVES = kWavesPerBlock>
 int launch_fwd_split(const T* x, T* y, int n, int c, size_t s, hipStream_t st)
 {
-    softmax_fwd_split_kernel<T, VEC, CPW><<<wide_grid(s, VEC, n), kBlockSize, 0, st>>>(x, y, c, s);
+    softmax_fwd_split_kernel<T, VEC, CPW, WAVES>
+        <<<wide_grid(s, VEC, n), WAVES * kWaveSize, 0, st>>>(x, y, c, s);
     return launch_status();
 }
 
-template <typename T, int VEC, int CPW>
+template <typename T, int VEC, int CPW, int WAVES = kWavesPerBlock>
 int launch_bwd_split(const T* y, const T* dy, T* dx, int n, int c, size_t s, hipStream_t st)
 {
-    softmax_bwd_split_kernel<T, VEC, CPW>
-        <<<wide_grid(s, VEC, n), kBlockSize, 0, st>>>(y, dy, dx, c, s);
+    softmax_bwd_split_kernel<T, VEC, CPW, WAVES>
+        <<<wide_grid(s, VEC, n), WAVES * kWaveSize, 0, st>>>(y, dy, dx, c, s);
     return launch_status();
 }
 
@@ -762,6 +822,8 @@ int forward_impl(int n, int c, size_t s, const void* xv, void* yv, hipStream_t s
         if (c <= 256) return launch_fwd_split<T, 1, 64>(x, y, n, c, s, st);
         if (c <= 384) return launch_fwd_split<T, 1, 96>(x, y, n, c, s, st);
         if (c <= 512) return launch_fwd_split<T, 1, 128>(x, y, n, c, s, st);
+        if (c <= 768) return launch_fwd_split<T, 1, 96, 8>(x, y, n, c, s, st);
+        if (c <= 1024) return launch_fwd_split<T, 1, 128, 8>(x, y, n, c, s, st);
     }
     else
     {
@@ -844,6 +906,7 @@ int backward_impl(int n, int c, size_t s, const void* yv, const void* dyv, void*
         if (c <= 256) return launch_bwd_split<T, 1, 64>(y, dy, dx, n, c, s, st);
         if (c <= 384) return launch_bwd_split<T, 1, 96>(y, dy, dx, n, c, s, st);
         if (c <= 512) return launch_bwd_split<T, 1, 128>(y, dy, dx, n, c, s, st);
+        if (c <= 768) return launch_bwd_split<T, 1, 96, 8>(y, dy, dx, n, c, s, st);
     }
     else
     {

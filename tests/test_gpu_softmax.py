@@ -32,8 +32,12 @@ CASES = [
     (2, 19, 4, 6, 10),    # 5-D
     (2, 256, 6, 10),      # 64 channels a wave in registers, two pixels a lane
     (2, 257, 3, 5),       # 65 of 128 channels a wave, one pixel a lane
-    (1, 512, 4, 4),       # the most the register tiles hold
-    (1, 513, 2, 2),       # beyond that: the re-reading kernel
+    (1, 512, 4, 4),       # the most four waves hold
+    (1, 513, 2, 2),       # eight waves share the channels
+    (2, 768, 2, 3),       # the most eight waves hold backward
+    (1, 800, 3, 2),       # forward in registers, backward the re-reading kernel
+    (2, 1024, 3, 3),      # the most eight waves hold forward
+    (1, 1025, 2, 2),      # beyond that: the re-reading kernel
     (3, 150, 40, 40),     # several workgroups a sample, the last one partly filled
 ]
 
