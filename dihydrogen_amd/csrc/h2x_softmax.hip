@@ -96,19 +96,41 @@ struct Pack
     }
 };
 
+// Where the VEC pixels of a lane start (offset of their first channel) and
+// whether they exist; `index` counts the lanes of the grid's x dimension in tile
+// order.  Tensors with few pixels per sample (flat_samples > 0; one pixel a lane)
+// count their pixels through all samples, so that a tile of 64 or 256 pixels is
+// full whatever the size of a sample; otherwise blockIdx.y is the sample.
+template <int VEC>
+__device__ __forceinline__ bool lane_pixels(size_t index, int num_channels, size_t spatial,
+                                            int flat_samples, size_t* base)
+{
+    const size_t p = index * VEC;
+    if (flat_samples > 0)
+    {
+        const unsigned int n = static_cast<unsigned int>(p) / static_cast<unsigned int>(spatial);
+        const bool exists = n < static_cast<unsigned int>(flat_samples);
+        *base = exists ? static_cast<size_t>(n) * num_channels * spatial + (p - n * spatial) : 0;
+        return exists;
+    }
+    const bool exists = p < spatial;
+    *base = static_cast<size_t>(blockIdx.y) * num_channels * spatial + (exists ? p : 0);
+    return exists;
+}
+
 // forward, register-resident.  Replaces fp_channel_kernel, softmax.cu:538-593:
 // running maximum starts at min_normal (positive), the sum is taken in channel
 // order, y = max(e * (1 / sum), min_normal).
 template <typename T, int VEC, int CMAX>
 __global__ __launch_bounds__(kBlockSize) void softmax_fwd_reg_kernel(
-    const T* __restrict__ x, T* __restrict__ y, int num_channels, size_t spatial)
+    const T* __restrict__ x, T* __restrict__ y, int num_channels, size_t spatial, int flat_samples)
 {
     using P = Pack<T, VEC>;
-    const size_t s =
-        (static_cast<size_t>(xcd_contiguous(blockIdx.x, gridDim.x)) * kBlockSize + threadIdx.x) * VEC;
-    if (s >= spatial)
+    size_t base;
+    if (!lane_pixels<VEC>(static_cast<size_t>(xcd_contiguous(blockIdx.x, gridDim.x)) * kBlockSize
+                              + threadIdx.x,
+                          num_channels, spatial, flat_samples, &base))
         return;
-    const size_t base = static_cast<size_t>(blockIdx.y) * num_channels * spatial + s;
     const T* xp = x + base;
     T* yp = y + base;
     constexpr T kMin = Limits<T>::min_normal;
@@ -169,14 +191,15 @@ constexpr int kWideBatch = 8;
 // running sum over all channels (softmax.cu:565-580).
 template <typename T>
 __global__ __launch_bounds__(kBlockSize) void softmax_fwd_wide_kernel(
-    const T* __restrict__ x, T* __restrict__ y, int num_channels, size_t spatial)
+    const T* __restrict__ x, T* __restrict__ y, int num_channels, size_t spatial, int flat_samples)
 {
     __shared__ T lds[kWavesPerBlock][kWaveSize];
     const int lane = threadIdx.x % kWaveSize;
     const int g = threadIdx.x / kWaveSize;
-    const size_t s = static_cast<size_t>(xcd_contiguous(blockIdx.x, gridDim.x)) * kWaveSize + lane;
-    const bool active = s < spatial;
-    const size_t base = static_cast<size_t>(blockIdx.y) * num_channels * spatial + (active ? s : 0);
+    size_t base;
+    const bool active =
+        lane_pixels<1>(static_cast<size_t>(xcd_contiguous(blockIdx.x, gridDim.x)) * kWaveSize + lane,
+                       num_channels, spatial, flat_samples, &base);
     const T* xp = x + base;
     T* yp = y + base;
     constexpr T kMin = Limits<T>::min_normal;
@@ -251,14 +274,14 @@ __global__ __launch_bounds__(kBlockSize) void softmax_fwd_wide_kernel(
 template <typename T, int VEC, int CMAX>
 __global__ __launch_bounds__(kBlockSize) void softmax_bwd_reg_kernel(
     const T* __restrict__ y, const T* __restrict__ dy, T* __restrict__ dx, int num_channels,
-    size_t spatial)
+    size_t spatial, int flat_samples)
 {
     using P = Pack<T, VEC>;
-    const size_t s =
-        (static_cast<size_t>(xcd_contiguous(blockIdx.x, gridDim.x)) * kBlockSize + threadIdx.x) * VEC;
-    if (s >= spatial)
+    size_t base;
+    if (!lane_pixels<VEC>(static_cast<size_t>(xcd_contiguous(blockIdx.x, gridDim.x)) * kBlockSize
+                              + threadIdx.x,
+                          num_channels, spatial, flat_samples, &base))
         return;
-    const size_t base = static_cast<size_t>(blockIdx.y) * num_channels * spatial + s;
     const T* yp = y + base;
     const T* gp = dy + base;
     T* op = dx + base;
@@ -298,14 +321,15 @@ __global__ __launch_bounds__(kBlockSize) void softmax_bwd_reg_kernel(
 template <typename T>
 __global__ __launch_bounds__(kBlockSize) void softmax_bwd_wide_kernel(
     const T* __restrict__ y, const T* __restrict__ dy, T* __restrict__ dx, int num_channels,
-    size_t spatial)
+    size_t spatial, int flat_samples)
 {
     __shared__ T lds[kWavesPerBlock][kWaveSize];
     const int lane = threadIdx.x % kWaveSize;
     const int g = threadIdx.x / kWaveSize;
-    const size_t s = static_cast<size_t>(xcd_contiguous(blockIdx.x, gridDim.x)) * kWaveSize + lane;
-    const bool active = s < spatial;
-    const size_t base = static_cast<size_t>(blockIdx.y) * num_channels * spatial + (active ? s : 0);
+    size_t base;
+    const bool active =
+        lane_pixels<1>(static_cast<size_t>(xcd_contiguous(blockIdx.x, gridDim.x)) * kWaveSize + lane,
+                       num_channels, spatial, flat_samples, &base);
     const T* yp = y + base;
     const T* gp = dy + base;
     T* op = dx + base;
@@ -366,16 +390,16 @@ __global__ __launch_bounds__(kBlockSize) void softmax_bwd_wide_kernel(
 // 60 us with the tile in registers).
 template <typename T, int VEC, int CPW, int WAVES>
 __global__ __launch_bounds__(WAVES * kWaveSize) void softmax_fwd_split_kernel(
-    const T* __restrict__ x, T* __restrict__ y, int num_channels, size_t spatial)
+    const T* __restrict__ x, T* __restrict__ y, int num_channels, size_t spatial, int flat_samples)
 {
     using P = Pack<T, VEC>;
     __shared__ T lds[WAVES][kWaveSize * VEC];
     const int lane = threadIdx.x % kWaveSize;
     const int g = threadIdx.x / kWaveSize;
-    const size_t s =
-        (static_cast<size_t>(xcd_contiguous(blockIdx.x, gridDim.x)) * kWaveSize + lane) * VEC;
-    const bool active = s < spatial;
-    const size_t base = static_cast<size_t>(blockIdx.y) * num_channels * spatial + (active ? s : 0);
+    size_t base;
+    const bool active = lane_pixels<VEC>(
+        static_cast<size_t>(xcd_contiguous(blockIdx.x, gridDim.x)) * kWaveSize + lane, num_channels,
+        spatial, flat_samples, &base);
     const T* xp = x + base;
     T* yp = y + base;
     constexpr T kMin = Limits<T>::min_normal;
@@ -460,16 +484,16 @@ __global__ __launch_bounds__(WAVES * kWaveSize) void softmax_fwd_split_kernel(
 template <typename T, int VEC, int CPW, int WAVES>
 __global__ __launch_bounds__(WAVES * kWaveSize) void softmax_bwd_split_kernel(
     const T* __restrict__ y, const T* __restrict__ dy, T* __restrict__ dx, int num_channels,
-    size_t spatial)
+    size_t spatial, int flat_samples)
 {
     using P = Pack<T, VEC>;
     __shared__ T lds[WAVES][kWaveSize * VEC];
     const int lane = threadIdx.x % kWaveSize;
     const int g = threadIdx.x / kWaveSize;
-    const size_t s =
-        (static_cast<size_t>(xcd_contiguous(blockIdx.x, gridDim.x)) * kWaveSize + lane) * VEC;
-    const bool active = s < spatial;
-    const size_t base = static_cast<size_t>(blockIdx.y) * num_channels * spatial + (active ? s : 0);
+    size_t base;
+    const bool active = lane_pixels<VEC>(
+        static_cast<size_t>(xcd_contiguous(blockIdx.x, gridDim.x)) * kWaveSize + lane, num_channels,
+        spatial, flat_samples, &base);
     const T* yp = y + base;
     const T* gp = dy + base;
     T* op = dx + base;
@@ -703,33 +727,54 @@ dim3 pixel_grid(size_t spatial, int vec, int num_samples)
     return dim3(static_cast<unsigned int>((spatial + per_block - 1) / per_block), num_samples);
 }
 
-// The same, padded to a multiple of the XCD count for kernels that reorder
-// their tiles with xcd_contiguous (tiles past the end do nothing).
-dim3 pixel_grid_xcd(size_t spatial, int vec, int num_samples)
+// Samples of fewer pixels than this have their pixels counted through all
+// samples (one pixel a lane): a tile is full whatever the size of a sample
+// (N 256, C 100, 7 x 7: one workgroup a sample with 49 of its 64 pixels, 17 us).
+constexpr size_t kFlatBelow = 128;
+
+int flat_samples(int num_samples, size_t spatial)
 {
-    const size_t per_block = static_cast<size_t>(kBlockSize) * vec;
-    const size_t blocks = (spatial + per_block - 1) / per_block;
-    return dim3(static_cast<unsigned int>((blocks + kNumXcd - 1) / kNumXcd * kNumXcd), num_samples);
+    return spatial < kFlatBelow && spatial * static_cast<size_t>(num_samples) < (1ull << 31)
+               ? num_samples
+               : 0;
 }
 
-// 64 * vec pixels per workgroup, padded for xcd_contiguous.
-dim3 wide_grid(size_t spatial, int vec, int num_samples)
+// Tiles of lanes * vec pixels, padded to a multiple of the XCD count for kernels
+// that reorder their tiles with xcd_contiguous (tiles past the end do nothing).
+dim3 tile_grid(size_t spatial, int lanes, int vec, int num_samples, int flat)
 {
-    const size_t per_block = static_cast<size_t>(kWaveSize) * vec;
-    const size_t blocks = (spatial + per_block - 1) / per_block;
-    return dim3(static_cast<unsigned int>((blocks + kNumXcd - 1) / kNumXcd * kNumXcd), num_samples);
+    const size_t per_block = static_cast<size_t>(lanes) * vec;
+    const size_t pixels = flat > 0 ? spatial * static_cast<size_t>(flat) : spatial;
+    const size_t blocks = (pixels + per_block - 1) / per_block;
+    return dim3(static_cast<unsigned int>((blocks + kNumXcd - 1) / kNumXcd * kNumXcd),
+                flat > 0 ? 1 : num_samples);
+}
+
+dim3 pixel_grid_xcd(size_t spatial, int vec, int num_samples, int flat)
+{
+    return tile_grid(spatial, kBlockSize, vec, num_samples, flat);
+}
+
+// 64 * vec pixels per workgroup.
+dim3 wide_grid(size_t spatial, int vec, int num_samples, int flat)
+{
+    return tile_grid(spatial, kWaveSize, vec, num_samples, flat);
 }
 
 template <typename T, int VEC, int CMAX>
 void launch_fwd(const T* x, T* y, int n, int c, size_t s, hipStream_t st)
 {
-    softmax_fwd_reg_kernel<T, VEC, CMAX><<<pixel_grid_xcd(s, VEC, n), kBlockSize, 0, st>>>(x, y, c, s);
+    const int flat = VEC == 1 ? flat_samples(n, s) : 0;
+    softmax_fwd_reg_kernel<T, VEC, CMAX>
+        <<<pixel_grid_xcd(s, VEC, n, flat), kBlockSize, 0, st>>>(x, y, c, s, flat);
 }
 
 template <typename T, int VEC, int CMAX>
 void launch_bwd(const T* y, const T* dy, T* dx, int n, int c, size_t s, hipStream_t st)
 {
-    softmax_bwd_reg_kernel<T, VEC, CMAX><<<pixel_grid_xcd(s, VEC, n), kBlockSize, 0, st>>>(y, dy, dx, c, s);
+    const int flat = VEC == 1 ? flat_samples(n, s) : 0;
+    softmax_bwd_reg_kernel<T, VEC, CMAX>
+        <<<pixel_grid_xcd(s, VEC, n, flat), kBlockSize, 0, st>>>(y, dy, dx, c, s, flat);
 }
 
 // Which kernel serves which channel count (float; measured on MI355X).  Up to
@@ -748,16 +793,18 @@ void launch_bwd(const T* y, const T* dy, T* dx, int n, int c, size_t s, hipStrea
 template <typename T, int VEC, int CPW, int WAVES = kWavesPerBlock>
 int launch_fwd_split(const T* x, T* y, int n, int c, size_t s, hipStream_t st)
 {
+    const int flat = VEC == 1 ? flat_samples(n, s) : 0;
     softmax_fwd_split_kernel<T, VEC, CPW, WAVES>
-        <<<wide_grid(s, VEC, n), WAVES * kWaveSize, 0, st>>>(x, y, c, s);
+        <<<wide_grid(s, VEC, n, flat), WAVES * kWaveSize, 0, st>>>(x, y, c, s, flat);
     return launch_status();
 }
 
 template <typename T, int VEC, int CPW, int WAVES = kWavesPerBlock>
 int launch_bwd_split(const T* y, const T* dy, T* dx, int n, int c, size_t s, hipStream_t st)
 {
+    const int flat = VEC == 1 ? flat_samples(n, s) : 0;
     softmax_bwd_split_kernel<T, VEC, CPW, WAVES>
-        <<<wide_grid(s, VEC, n), WAVES * kWaveSize, 0, st>>>(y, dy, dx, c, s);
+        <<<wide_grid(s, VEC, n, flat), WAVES * kWaveSize, 0, st>>>(y, dy, dx, c, s, flat);
     return launch_status();
 }
 
@@ -786,7 +833,7 @@ int forward_impl(int n, int c, size_t s, const void* xv, void* yv, hipStream_t s
         softmax_fwd_long_row_kernel<T><<<n, kBlockSize, 0, st>>>(x, y, c);
         return launch_status();
     }
-    const int v4 = vector_width<T>(s, 4 / kWords, {xv, yv});
+    const int v4 = s < kFlatBelow ? 1 : vector_width<T>(s, 4 / kWords, {xv, yv});
 #define H2X_FWD(V, CM)                                                                             \
     do                                                                                             \
     {                                                                                              \
@@ -842,7 +889,8 @@ int forward_impl(int n, int c, size_t s, const void* xv, void* yv, hipStream_t s
         if (c <= 256) return launch_fwd_split<T, 1, 64>(x, y, n, c, s, st);
     }
 #undef H2X_FWD
-    softmax_fwd_wide_kernel<T><<<wide_grid(s, 1, n), kBlockSize, 0, st>>>(x, y, c, s);
+    const int flat = flat_samples(n, s);
+    softmax_fwd_wide_kernel<T><<<wide_grid(s, 1, n, flat), kBlockSize, 0, st>>>(x, y, c, s, flat);
     return launch_status();
 }
 
@@ -873,7 +921,7 @@ int backward_impl(int n, int c, size_t s, const void* yv, const void* dyv, void*
         softmax_bwd_long_row_kernel<T><<<n, kBlockSize, 0, st>>>(y, dy, dx, c);
         return launch_status();
     }
-    const int v4 = vector_width<T>(s, 4 / kWords, {yv, dyv, dxv});
+    const int v4 = s < kFlatBelow ? 1 : vector_width<T>(s, 4 / kWords, {yv, dyv, dxv});
 #define H2X_BWD(V, CM)                                                                             \
     do                                                                                             \
     {                                                                                              \
@@ -924,7 +972,8 @@ int backward_impl(int n, int c, size_t s, const void* yv, const void* dyv, void*
         if (c <= 256) return launch_bwd_split<T, 1, 64>(y, dy, dx, n, c, s, st);
     }
 #undef H2X_BWD
-    softmax_bwd_wide_kernel<T><<<wide_grid(s, 1, n), kBlockSize, 0, st>>>(y, dy, dx, c, s);
+    const int flat = flat_samples(n, s);
+    softmax_bwd_wide_kernel<T><<<wide_grid(s, 1, n, flat), kBlockSize, 0, st>>>(y, dy, dx, c, s, flat);
     return launch_status();
 }
 

@@ -39,6 +39,11 @@ CASES = [
     (2, 1024, 3, 3),      # the most eight waves hold forward
     (1, 1025, 2, 2),      # beyond that: the re-reading kernel
     (3, 150, 40, 40),     # several workgroups a sample, the last one partly filled
+    # fewer than 128 pixels a sample: the pixels are counted through all samples, a tile holds several samples
+    (37, 5, 3, 5),
+    (130, 40, 7, 7),
+    (9, 600, 7, 7),
+    (11, 1100, 3, 3),
 ]
 
 
