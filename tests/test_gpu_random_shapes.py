@@ -150,6 +150,32 @@ def _shuffle_cases(count=24, seed=20240611):
     return cases
 
 
+def _bn_halo_cases(count=16, seed=20240612):
+    """Spatially decomposed tensors with halos, for batch-norm on every rank: local tiles from a
+    few elements (the short-segment kernels, slots by rows) to a few thousand (padded rows)."""
+    rng = np.random.default_rng(seed)
+    cases = []
+    while len(cases) < count:
+        nd = int(rng.integers(4, 6))
+        ns = nd - 2
+        locale = _factor(rng, int(rng.choice([2, 4, 8])), ns) + [1, 1]
+        overlap = [int(rng.integers(0, 3)) for _ in range(ns)] + [0, 0]
+        if not any(overlap[:ns - 1]):            # a halo on an inner dimension: the strided layout
+            continue
+        small = len(cases) % 2 == 0
+        shape = [int(locale[d] * rng.integers(max(overlap[d], 1), 9 if small else 40)) for d in range(ns)]
+        shape += [int(np.exp(rng.uniform(0, np.log(40)))), int(rng.integers(1, 6))]
+        if int(np.prod(shape)) > 150_000:
+            continue
+        cases.append((tuple(shape), tuple(locale), tuple(overlap)))
+    return cases
+
+
+@pytest.mark.parametrize("case", _bn_halo_cases())
+def test_batch_norm_on_haloed_tensors(case, oracle_mod):
+    bn_tests.test_haloed_tensors_match_oracle(case, oracle_mod)
+
+
 @pytest.mark.parametrize("case", _halo_cases())
 def test_halo_exchange(case, oracle_mod):
     import test_gpu_halo as halo_tests
