@@ -101,6 +101,8 @@ size_t partials_bytes(int num_channels)
 }
 
 // How one (sample, channel) segment of `spatial` elements is cut into chunks.
+// With vectors, `spatial` is a whole number of them (dense: a condition of the
+// aligned path; strided: rows are padded), and so is every chunk.
 struct Chunking
 {
     size_t chunk;        // elements per workgroup, multiple of the tile
@@ -425,13 +427,6 @@ __global__ __launch_bounds__(kBlockSize) void bn_sums_kernel(
                 if (j >= static_cast<int>(skip))
                     accumulate(v[j]);
         }
-        if constexpr (VEC > 1)
-        {
-            // a segment whose length is no multiple of the vector ends with single elements
-            const size_t rest = (end - begin) % VEC;
-            if (threadIdx.x < rest)
-                accumulate(p[seg_offset<STRIDED>(mx, end - rest + threadIdx.x)]);
-        }
     }
     if (finish_workgroup<2>(acc, partials, c, groups_per_channel_max, always_partials)
         && threadIdx.x == 0)
@@ -562,18 +557,6 @@ __global__ __launch_bounds__(kBlockSize) void bn_apply_kernel(
             v[j] = fma_t((v[j] - m) * inv_stdev, sc, bi);
         store_at<T, VEC, STRIDED>(yp, my, i, v, true);
     }
-    if constexpr (VEC > 1)
-    {
-        // a segment whose length is no multiple of the vector ends with single elements
-        const size_t rest = (end - begin) % VEC;
-        if (threadIdx.x < rest)
-        {
-            const size_t i = end - rest + threadIdx.x;
-            T v[1] = {xp[seg_offset<STRIDED>(mx, i)]};
-            v[0] = fma_t((v[0] - m) * inv_stdev, sc, bi);
-            store_vec<T, 1>(yp + seg_offset<STRIDED>(my, i), v);
-        }
-    }
 }
 
 // ---- backward: per-channel sums ----------------------------------------------
@@ -647,16 +630,6 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop1_kernel(
             for (int j = 0; j < VEC; ++j)
                 if (j >= static_cast<int>(skip))
                     accumulate(xv[j], dv[j]);
-        }
-        if constexpr (VEC > 1)
-        {
-            // a segment whose length is no multiple of the vector ends with single elements
-            const size_t rest = (end - begin) % VEC;
-            if (threadIdx.x < rest)
-            {
-                const size_t i = end - rest + threadIdx.x;
-                accumulate(xp[seg_offset<STRIDED>(mx, i)], dp[seg_offset<STRIDED>(md, i)]);
-            }
         }
     }
     if (finish_workgroup<4>(acc, partials, c, groups_per_channel_max, always_partials)
@@ -756,18 +729,6 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop2_kernel(
             xv[j] = fma_t(xv[j] - m, dvar_term, r);
         }
         store_at<T, VEC, STRIDED>(op, mo, i, xv, disjoint);
-    }
-    if constexpr (VEC > 1)
-    {
-        // a segment whose length is no multiple of the vector ends with single elements
-        const size_t rest = (end - begin) % VEC;
-        if (threadIdx.x < rest)
-        {
-            const size_t i = end - rest + threadIdx.x;
-            const T r = fma_t(dp[seg_offset<STRIDED>(md, i)] * sc, inv_stdev, dmean_term);
-            T v[1] = {fma_t(xp[seg_offset<STRIDED>(mx, i)] - m, dvar_term, r)};
-            store_vec<T, 1>(op + seg_offset<STRIDED>(mo, i), v);
-        }
     }
 }
 
