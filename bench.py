@@ -381,21 +381,21 @@ def cpu_baseline(repeats: int = 5):
 # TCC_EA0_WRREQ_64B), request counts summed over the L2 channels, per dispatch.
 # label -> (bytes read, bytes written) per launch
 PMC_TRAFFIC = {
-    "bn_sums": (268460544, 131072),
-    "bn_apply": (268466176, 268483200),
-    "bn_backprop1": (536915328, 131072),
-    "bn_backprop2": (536907776, 268435456),
-    "halo_dim0_pack": (149477968, 8652800),    # 4 faces (2 ranks) a launch, four launches a step
-    "halo_dim0_unpack": (9218224, 43264000),
+    "bn_sums": (268451328, 131072),
+    "bn_apply": (268466176, 268496512),
+    "bn_backprop1": (536913344, 131072),
+    "bn_backprop2": (536904704, 268435968),
+    "halo_dim0_pack": (149623936, 8652800),    # 4 faces (2 ranks) a launch, four launches a step
+    "halo_dim0_unpack": (9219232, 43264000),
     "halo_dim1_pack": (42624768, 34611200),
-    "halo_dim1_unpack": (34637504, 36216128),
+    "halo_dim1_unpack": (34637440, 36216768),
     "halo_dim2_pack": (34694400, 34611200),
-    "halo_dim2_unpack": (34637568, 34619488),
+    "halo_dim2_unpack": (34637568, 34619392),
 }
 # sha256 (first 16 hex digits) of the kernel sources the table was measured with, see
 # kernel_sources_sha(); with other sources the traffic fields are omitted
-PMC_SOURCES_SHA = "e8f4000d51cee6f5"
-PMC_COMMIT = "cccf888"
+PMC_SOURCES_SHA = "21c18b723b66d41b"
+PMC_COMMIT = "161583c"
 
 KERNEL_OF = {
     "bn_sums": "bn_sums_kernel<float,4> (+bn_finish_kernel<float,2>)",

@@ -230,5 +230,5 @@ int main()
     }
     errors += test_statistics();
     std::printf("test_algorithms: %d errors\n", errors);
-    return errors ? 1 : 0;
+    leave(errors ? 1 : 0);
 }

@@ -278,5 +278,5 @@ int main()
     errors += test_softmax_instance(Shape({32, 32, 21, 4}));
     errors += test_softmax_instance(Shape({5, 3, 7, 2}));
     std::printf("test_batchnorm_softmax: %d errors\n", errors);
-    return errors ? 1 : 0;
+    leave(errors ? 1 : 0);
 }

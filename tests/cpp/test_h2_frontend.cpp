@@ -11,6 +11,8 @@
 #include <random>
 #include <vector>
 
+#include <unistd.h>
+
 #include "h2/ops_mi355x.hpp"
 
 extern "C" {
@@ -560,5 +562,10 @@ int main()
 #undef RUN
     check_hip(hipDeviceSynchronize(), "sync");
     std::printf("test_h2_frontend: ok\n");
-    return 0;
+    // Leave without running exit handlers and static destructors: the order in which the HIP
+    // runtime, the OpenMP runtime of the CPU oracle and this program's statics are torn down is
+    // nobody's contract, and a crash in there would hide the result of the checks (this program
+    // ended with SIGSEGV after the line above in 2 of about 50 runs).
+    std::fflush(nullptr);
+    _exit(0);
 }
