@@ -382,15 +382,15 @@ def cpu_baseline(repeats: int = 5):
 # label -> (bytes read, bytes written) per launch
 PMC_TRAFFIC = {
     "bn_sums": (268451328, 131072),
-    "bn_apply": (268466176, 268496512),
-    "bn_backprop1": (536913344, 131072),
-    "bn_backprop2": (536904704, 268435968),
-    "halo_dim0_pack": (149623936, 8652800),    # 4 faces (2 ranks) a launch, four launches a step
-    "halo_dim0_unpack": (9219232, 43264000),
-    "halo_dim1_pack": (42624768, 34611200),
-    "halo_dim1_unpack": (34637440, 36216768),
+    "bn_apply": (268466176, 268486912),
+    "bn_backprop1": (536913408, 131072),
+    "bn_backprop2": (536904704, 268435456),
+    "halo_dim0_pack": (149576448, 8652800),    # 4 faces (2 ranks) a launch, four launches a step
+    "halo_dim0_unpack": (9218592, 43264000),
+    "halo_dim1_pack": (42624704, 34611200),
+    "halo_dim1_unpack": (34637568, 36217600),
     "halo_dim2_pack": (34694400, 34611200),
-    "halo_dim2_unpack": (34637568, 34619392),
+    "halo_dim2_unpack": (34637568, 34619552),
 }
 # steps of the timed region whose dominant-kernel launches are bracketed by events: every EVENT_EVERY-th
 EVENT_EVERY = 4
@@ -398,7 +398,7 @@ EVENT_EVERY = 4
 # sha256 (first 16 hex digits) of the kernel sources the table was measured with, see
 # kernel_sources_sha(); with other sources the traffic fields are omitted
 PMC_SOURCES_SHA = "21c18b723b66d41b"
-PMC_COMMIT = "161583c"
+PMC_COMMIT = "dab733e"
 
 KERNEL_OF = {
     "bn_sums": "bn_sums_kernel<float,4> (+bn_finish_kernel<float,2>)",
