@@ -1181,9 +1181,10 @@ __global__ __launch_bounds__(kBlockSize) void softmax_inst_map_kernel(
     P::store(out + off, v);
 }
 
-// Samples of at most 64 * CPL elements (the softmax behind a classifier: 10 to
-// a few thousand classes): a wave takes a sample, holds it in registers and
-// combines its lanes with shuffles, so a reduction is one launch without
+// Samples of at most 8192 elements (the softmax behind a classifier: 10 to
+// a few thousand classes): a wave -- beyond 2048 elements a workgroup -- takes a
+// sample, holds it in registers (CPL elements a lane) and combines its lanes with
+// shuffles (and its waves through LDS), so a reduction is one launch without
 // partials, and the whole forward pass of samples that are whole on this rank is
 // one launch too (N 4096, 10 elements a sample: 18 us in five launches before).
 // Sums are accumulated in fp64, lane by lane and then across the lanes as a
@@ -1197,25 +1198,28 @@ enum InstSmall : int
     kSmallForward = 4  // result[n] = max, result2[n] = sum, out = max(exp(x - max) / sum, min_output)
 };
 
-template <typename T, int CPL, int MODE>
+template <typename T, int CPL, int MODE, int LANES>
 __global__ __launch_bounds__(kBlockSize) void softmax_inst_small_kernel(
     const T* __restrict__ a, const T* __restrict__ b, T* __restrict__ out,
     const T* __restrict__ sample_param, T* __restrict__ result, T* __restrict__ result2,
     int sample_size, int num_samples, T min_output)
 {
-    const int lane = threadIdx.x % kWaveSize;
-    const int n = blockIdx.x * kWavesPerBlock + threadIdx.x / kWaveSize;
+    // LANES lanes serve a sample: a wave, or the whole workgroup (whose waves are then
+    // combined through LDS in wave order; every thread of the workgroup has the same n)
+    __shared__ double lds[kWavesPerBlock];
+    const int lane = threadIdx.x % LANES;
+    const int n = (blockIdx.x * kBlockSize + threadIdx.x) / LANES;
     if (n >= num_samples)
         return;
     const size_t base = static_cast<size_t>(n) * sample_size;
     T va[CPL], vb[CPL];
 #pragma unroll
     for (int k = 0; k < CPL; ++k)
-        if (lane + k * kWaveSize < sample_size)
+        if (lane + k * LANES < sample_size)
         {
-            va[k] = a[base + lane + k * kWaveSize];
+            va[k] = a[base + lane + k * LANES];
             if constexpr (MODE == kSmallDot)
-                vb[k] = b[base + lane + k * kWaveSize];
+                vb[k] = b[base + lane + k * LANES];
         }
     T shift = T(0);
     if constexpr (MODE == kSmallMax || MODE == kSmallForward)
@@ -1223,9 +1227,12 @@ __global__ __launch_bounds__(kBlockSize) void softmax_inst_small_kernel(
         T mx = Limits<T>::min_normal; // softmax.cu:88-99: the maximum starts at min_normal
 #pragma unroll
         for (int k = 0; k < CPL; ++k)
-            if (lane + k * kWaveSize < sample_size)
+            if (lane + k * LANES < sample_size)
                 mx = va[k] >= mx ? va[k] : mx;
-        mx = wave_max(mx);
+        if constexpr (LANES == kWaveSize)
+            mx = wave_max(mx);
+        else
+            mx = static_cast<T>(block_combine(static_cast<double>(mx), true, lds));
         if (lane == 0)
             result[n] = mx;
         if constexpr (MODE == kSmallMax)
@@ -1239,7 +1246,7 @@ __global__ __launch_bounds__(kBlockSize) void softmax_inst_small_kernel(
     double acc = 0.0;
 #pragma unroll
     for (int k = 0; k < CPL; ++k)
-        if (lane + k * kWaveSize < sample_size)
+        if (lane + k * LANES < sample_size)
         {
             if constexpr (MODE == kSmallDot)
             {
@@ -1251,7 +1258,10 @@ __global__ __launch_bounds__(kBlockSize) void softmax_inst_small_kernel(
                 acc += static_cast<double>(va[k]);
             }
         }
-    acc = wave_butterfly_sum(acc);
+    if constexpr (LANES == kWaveSize)
+        acc = wave_butterfly_sum(acc);
+    else
+        acc = block_combine(acc, false, lds);
     const T total = static_cast<T>(acc);
     if (lane == 0)
         (MODE == kSmallForward ? result2 : result)[n] = total;
@@ -1259,40 +1269,43 @@ __global__ __launch_bounds__(kBlockSize) void softmax_inst_small_kernel(
     {
 #pragma unroll
         for (int k = 0; k < CPL; ++k)
-            if (lane + k * kWaveSize < sample_size)
+            if (lane + k * LANES < sample_size)
             {
                 if constexpr (MODE == kSmallForward)
                 {
                     const T r = va[k] / total;
                     va[k] = r > min_output ? r : min_output;
                 }
-                out[base + lane + k * kWaveSize] = va[k];
+                out[base + lane + k * LANES] = va[k];
             }
     }
 }
 
-constexpr size_t kInstSmallSample = 32 * kWaveSize;
+constexpr size_t kInstSmallSample = 32 * kBlockSize;
 
 template <typename T, int MODE>
 int inst_small(int n, size_t sample_size, const void* a, const void* b, void* out,
                const void* param, void* result, void* result2, T min_output, hipStream_t st)
 {
-    const unsigned int blocks = (static_cast<unsigned int>(n) + kWavesPerBlock - 1) / kWavesPerBlock;
-#define H2X_INST_SMALL(CP)                                                                         \
+#define H2X_INST_SMALL(CP, LN)                                                                     \
     do                                                                                             \
     {                                                                                              \
-        softmax_inst_small_kernel<T, CP, MODE><<<blocks, kBlockSize, 0, st>>>(                     \
-            static_cast<const T*>(a), static_cast<const T*>(b), static_cast<T*>(out),              \
-            static_cast<const T*>(param), static_cast<T*>(result), static_cast<T*>(result2),       \
-            static_cast<int>(sample_size), n, min_output);                                         \
+        const unsigned int teams = kBlockSize / LN;                                                \
+        softmax_inst_small_kernel<T, CP, MODE, LN>                                                 \
+            <<<(static_cast<unsigned int>(n) + teams - 1) / teams, kBlockSize, 0, st>>>(           \
+                static_cast<const T*>(a), static_cast<const T*>(b), static_cast<T*>(out),          \
+                static_cast<const T*>(param), static_cast<T*>(result), static_cast<T*>(result2),   \
+                static_cast<int>(sample_size), n, min_output);                                     \
         return launch_status();                                                                    \
     } while (0)
-    if (sample_size <= 1 * kWaveSize) H2X_INST_SMALL(1);
-    if (sample_size <= 2 * kWaveSize) H2X_INST_SMALL(2);
-    if (sample_size <= 4 * kWaveSize) H2X_INST_SMALL(4);
-    if (sample_size <= 8 * kWaveSize) H2X_INST_SMALL(8);
-    if (sample_size <= 16 * kWaveSize) H2X_INST_SMALL(16);
-    H2X_INST_SMALL(32);
+    if (sample_size <= 1 * kWaveSize) H2X_INST_SMALL(1, kWaveSize);
+    if (sample_size <= 2 * kWaveSize) H2X_INST_SMALL(2, kWaveSize);
+    if (sample_size <= 4 * kWaveSize) H2X_INST_SMALL(4, kWaveSize);
+    if (sample_size <= 8 * kWaveSize) H2X_INST_SMALL(8, kWaveSize);
+    if (sample_size <= 16 * kWaveSize) H2X_INST_SMALL(16, kWaveSize);
+    if (sample_size <= 32 * kWaveSize) H2X_INST_SMALL(32, kWaveSize);
+    if (sample_size <= 16 * kBlockSize) H2X_INST_SMALL(16, kBlockSize);
+    H2X_INST_SMALL(32, kBlockSize);
 #undef H2X_INST_SMALL
 }
 

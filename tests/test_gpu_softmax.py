@@ -162,7 +162,9 @@ def test_float64(shape, oracle_mod):
 
 INSTANCE_CASES = [(16, 21, 64, 64), (3, 4, 5, 6), (2, 7, 9), (1, 2, 3, 4, 5), (5, 1, 1, 1), (2, 64, 128, 128),
                   # samples of at most 2048 elements: a wave per sample
-                  (300, 10, 1, 1), (7, 1000, 1, 1), (3, 2048, 1, 1), (2, 2049, 1, 1), (130, 5, 13, 1)]
+                  (300, 10, 1, 1), (7, 1000, 1, 1), (3, 2048, 1, 1), (130, 5, 13, 1),
+                  # to 8192 elements: a workgroup per sample
+                  (2, 2049, 1, 1), (5, 4096), (3, 4097), (4, 8192), (2, 8193)]
 
 
 @pytest.mark.parametrize("shape", INSTANCE_CASES)
