@@ -211,7 +211,9 @@ int h2x_bn_backprop1(h2x_dtype dtype,
 
 /**
  * dx = dy * scale * r + dmean / n + dvar * 2 / (n - 1) * (x - mean), with
- * n = num_per_sum.  dx may alias x.  Replaces batchnorm::backprop2
+ * n = num_per_sum.  dx may be x itself (the same elements at the same
+ * addresses, batchnorm.cu:1303-1314); buffers that overlap in any other way
+ * are not supported.  Replaces batchnorm::backprop2
  * (batchnorm.hpp:83-96, batchnorm.cu:1371-1559).
  */
 int h2x_bn_backprop2(h2x_dtype dtype,
@@ -268,7 +270,7 @@ int h2x_bn_forward_local(h2x_dtype dtype,
  * Backward pass likewise: h2x_bn_backprop1 followed by h2x_bn_backprop2 with
  * the sums it produced, bit for bit, in two launches instead of three
  * (BatchNormalization::backward without its allreduce stage,
- * batchnorm.hpp:360-475).  dx may alias x.
+ * batchnorm.hpp:360-475).  dx may be x itself.
  */
 int h2x_bn_backward_local(h2x_dtype dtype,
                           int num_samples,
