@@ -109,19 +109,16 @@ h2x_tensor_geometry local_geometry(const Tensor& t, const Shape* region = nullpt
     return g;
 }
 
-// Device scratch per stream, grown on demand and kept for the life of the
-// process (calls on one stream are ordered, so they can share it).
+// Device scratch shared by the calls of one stream, grown on demand (calls on
+// one stream are ordered, so they can share it).  Kept until
+// distconv::release_workspaces(); nothing is freed at static destruction.
 inline void* stream_scratch(hipStream_t stream, size_t bytes)
 {
-    static std::map<hipStream_t, Memory<CUDAAllocator>> table;
-    Memory<CUDAAllocator>& m = table[stream];
-    if (m.is_null() || m.get_size() < bytes)
-    {
-        if (!m.is_null())
-            DISTCONV_CHECK_HIP(hipStreamSynchronize(stream));
-        m.allocate(bytes);
-    }
-    return m.get();
+    hipError_t err = hipSuccess;
+    void* p = h2x_host::StreamScratch::get(stream, h2x_host::StreamScratch::REDUCE_PARTIALS, bytes,
+                                           &err);
+    DISTCONV_CHECK_HIP(err);
+    return p;
 }
 
 template <typename Tensor, typename Functor>

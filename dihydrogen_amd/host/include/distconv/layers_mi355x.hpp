@@ -5,7 +5,6 @@
 #pragma once
 
 #include <functional>
-#include <map>
 
 #include "distconv/algorithms_mi355x.hpp"
 #include "distconv/tensor_mi355x.hpp"
@@ -78,29 +77,44 @@ h2x_tensor_geometry tensor_geometry(const Tensor& t, int num_samples)
     return g;
 }
 
-// Workspace of fp64 partial sums, owned by the caller (one per layer object).
+// Workspace of fp64 partial sums.  A default-constructed one owns its memory
+// (one per layer object, freed with the object); one made by
+// default_workspace() refers to the buffer that the calls of one stream share.
 class Workspace
 {
 public:
+    Workspace() = default;
     void* get(int num_channels)
     {
         const size_t need = h2x_bn_workspace_bytes(num_channels);
+        if (m_shared)
+        {
+            hipError_t err = hipSuccess;
+            void* p = h2x_host::StreamScratch::get(m_stream, h2x_host::StreamScratch::BN_PARTIALS,
+                                                   need, &err);
+            DISTCONV_CHECK_HIP(err);
+            return p;
+        }
         if (m_mem.is_null() || m_mem.get_size() < need)
             m_mem.allocate(need);
         return m_mem.get();
     }
 
 private:
+    friend Workspace default_workspace(hipStream_t stream);
+    explicit Workspace(hipStream_t stream) : m_shared(true), m_stream(stream) {}
     tensor::Memory<tensor::CUDAAllocator> m_mem;
+    bool m_shared = false;
+    hipStream_t m_stream = nullptr;
 };
 
-// Workspace used by the overloads that keep the reference's exact signatures:
-// one per stream, created on first use and kept for the life of the process
-// (calls on one stream are ordered, so they can share it).
-inline Workspace& default_workspace(hipStream_t stream)
+// Workspace used by the overloads that keep the reference's exact signatures
+// (which have no workspace argument): one buffer per stream, created on first
+// use (calls on one stream are ordered, so they can share it).  It is kept
+// until release_workspaces(); nothing is freed at static destruction.
+inline Workspace default_workspace(hipStream_t stream)
 {
-    static std::map<hipStream_t, Workspace> table;
-    return table[stream];
+    return Workspace(stream);
 }
 
 // batchnorm.hpp:22-28
@@ -134,8 +148,8 @@ template <typename Tensor>
 void channel_sums_and_sqsums(int num_dims, int num_samples, const Tensor& input, Tensor& sums,
                              Tensor& sqsums, hipStream_t stream)
 {
-    channel_sums_and_sqsums(num_dims, num_samples, input, sums, sqsums, stream,
-                            default_workspace(stream));
+    Workspace ws = default_workspace(stream);
+    channel_sums_and_sqsums(num_dims, num_samples, input, sums, sqsums, stream, ws);
 }
 
 // batchnorm.hpp:30-37
@@ -219,9 +233,9 @@ void backprop1(int num_dims, int num_samples, const Tensor& input, const Tensor&
                Tensor& bias_gradient, Tensor& mean_gradient, Tensor& var_gradient,
                typename Tensor::data_type epsilon, hipStream_t stream)
 {
+    Workspace ws = default_workspace(stream);
     backprop1(num_dims, num_samples, input, d_output, mean, var, scale, scale_gradient,
-              bias_gradient, mean_gradient, var_gradient, epsilon, stream,
-              default_workspace(stream));
+              bias_gradient, mean_gradient, var_gradient, epsilon, stream, ws);
 }
 
 // batchnorm.hpp:83-96; d_input may be the same tensor as input

@@ -11,9 +11,26 @@
 #include <memory>
 
 #include "distconv/base_mi355x.hpp"
+#include "h2x_stream_scratch.hpp"
 
 namespace distconv
 {
+
+// Frees the device buffers that the free functions with the reference's exact
+// signatures (batchnorm::channel_sums_and_sqsums, backprop1, tensor::ReduceSum,
+// ...) keep per stream: of one stream (call it before destroying the stream) or
+// of every stream of the current device.  Waits for the work in flight first.
+// Layer objects own their workspaces and free them with the object; nothing in
+// this layer frees device memory from a destructor of static storage duration.
+inline void release_workspaces(hipStream_t stream)
+{
+    DISTCONV_CHECK_HIP(h2x_host::StreamScratch::release(stream));
+}
+inline void release_workspaces()
+{
+    DISTCONV_CHECK_HIP(h2x_host::StreamScratch::release_all());
+}
+
 namespace tensor
 {
 

@@ -20,6 +20,7 @@
 
 #include "h2/h2_mi355x.hpp"
 #include "h2x.h"
+#include "h2x_stream_scratch.hpp"
 
 #include <map>
 #include <mutex>
@@ -78,31 +79,22 @@ inline void require_same(const BaseTensor& a, const BaseTensor& b, const char* w
         throw H2FatalException(what, ": tensors live on different devices");
 }
 
-// fp64 partials of the two batch-norm reductions: one buffer per stream, grown
-// on demand and kept for the life of the process (calls on a stream are ordered).
+// Device scratch shared by the calls of one stream, grown on demand (calls on a
+// stream are ordered).  Kept until h2::release_workspaces(); nothing is freed at
+// static destruction.
+inline void* stream_scratch(hipStream_t stream, size_t bytes, int slot)
+{
+    hipError_t err = hipSuccess;
+    void* p = h2x_host::StreamScratch::get(stream, slot, bytes, &err);
+    check_hip(err, "stream scratch");
+    return p;
+}
+
+// fp64 partials of the two batch-norm reductions
 inline void* bn_workspace(hipStream_t stream, int channels)
 {
-    struct Entry
-    {
-        void* ptr = nullptr;
-        size_t bytes = 0;
-    };
-    static std::map<hipStream_t, Entry> table;
-    static std::mutex m;
-    std::lock_guard<std::mutex> lock(m);
-    Entry& e = table[stream];
-    const size_t need = h2x_bn_workspace_bytes(channels);
-    if (need > e.bytes)
-    {
-        if (e.ptr)
-        {
-            check_hip(hipStreamSynchronize(stream), "hipStreamSynchronize");
-            check_hip(hipFree(e.ptr), "hipFree");
-        }
-        check_hip(hipMalloc(&e.ptr, need), "hipMalloc");
-        e.bytes = need;
-    }
-    return e.ptr;
+    return stream_scratch(stream, h2x_bn_workspace_bytes(channels),
+                          h2x_host::StreamScratch::BN_PARTIALS);
 }
 
 inline hipStream_t gpu_stream(const BaseTensor& t)
@@ -111,6 +103,18 @@ inline hipStream_t gpu_stream(const BaseTensor& t)
 }
 
 } // namespace mi355x
+
+// Frees the device buffers the operators keep per stream (partial sums of the
+// reductions): of one stream (call it before destroying the stream) or of every
+// stream of the current device.  Waits for the work in flight first.
+inline void release_workspaces(hipStream_t stream)
+{
+    check_hip(h2x_host::StreamScratch::release(stream), "release_workspaces");
+}
+inline void release_workspaces()
+{
+    check_hip(h2x_host::StreamScratch::release_all(), "release_workspaces");
+}
 
 // ---- device implementations ---------------------------------------------------------------
 namespace impl

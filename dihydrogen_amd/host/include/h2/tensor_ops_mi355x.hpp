@@ -57,31 +57,6 @@ inline h2x_tensor_geometry plain_geometry(const BaseTensor& t, const char* what)
     return g;
 }
 
-// Device scratch per stream, grown on demand, kept for the life of the process.
-inline void* stream_scratch(hipStream_t stream, size_t bytes, int slot = 0)
-{
-    struct Entry
-    {
-        void* ptr = nullptr;
-        size_t bytes = 0;
-    };
-    static std::map<std::pair<hipStream_t, int>, Entry> table;
-    static std::mutex m;
-    std::lock_guard<std::mutex> lock(m);
-    Entry& e = table[{stream, slot}];
-    if (bytes > e.bytes)
-    {
-        if (e.ptr)
-        {
-            check_hip(hipStreamSynchronize(stream), "hipStreamSynchronize");
-            check_hip(hipFree(e.ptr), "hipFree");
-        }
-        check_hip(hipMalloc(&e.ptr, bytes), "hipMalloc");
-        e.bytes = bytes;
-    }
-    return e.ptr;
-}
-
 // Calls f(offsets...) for every element of equally shaped strided tensors,
 // innermost dimension fastest (host loops of the CPU implementations).
 template <std::size_t N, typename F>
@@ -207,8 +182,9 @@ void reduce_sum_impl(GPUDev_t, const Tensor<T>& src, Tensor<T>& dst, bool square
     const size_t bytes = h2x_tensor_reduce_sum_workspace_bytes(&gs, &gd);
     if (bytes == 0)
         throw H2FatalException("reduce_sum: each extent of dst must be 1 or equal to src's");
+    void* ws = mi355x::stream_scratch(s, bytes, h2x_host::StreamScratch::REDUCE_PARTIALS);
     mi355x::check(h2x_tensor_reduce_sum(mi355x::dtype_of<T>(), &gs, src.const_data(), &gd, dst.data(),
-                                        square ? 1 : 0, mi355x::stream_scratch(s, bytes, 1), s),
+                                        square ? 1 : 0, ws, s),
                   "reduce_sum");
 }
 template <typename T>
@@ -418,8 +394,10 @@ void softmax_instance_forward_impl(GPUDev_t, const Tensor<T>& x, Tensor<T>& y)
     const int n = static_cast<int>(g.local_shape[g.num_dims - 1]);
     const size_t size = static_cast<size_t>(x.numel()) / n;
     hipStream_t s = mi355x::gpu_stream(x);
-    void* ws = mi355x::stream_scratch(s, h2x_softmax_instance_workspace_bytes(n), 2);
-    T* scalars = static_cast<T*>(mi355x::stream_scratch(s, 2 * n * sizeof(T), 3));
+    void* ws = mi355x::stream_scratch(s, h2x_softmax_instance_workspace_bytes(n),
+                                      h2x_host::StreamScratch::SOFTMAX_PARTIALS);
+    T* scalars = static_cast<T*>(mi355x::stream_scratch(s, 2 * n * sizeof(T),
+                                                      h2x_host::StreamScratch::SOFTMAX_SCALARS));
     const h2x_dtype dt = mi355x::dtype_of<T>();
     // an h2 tensor is one rank's whole tensor: no all-reduce between the stages
     mi355x::check(h2x_softmax_instance_forward_local(dt, n, size, x.const_data(), y.data(), scalars,
@@ -437,8 +415,10 @@ void softmax_instance_backward_impl(GPUDev_t, const Tensor<T>& y, const Tensor<T
     const int n = static_cast<int>(g.local_shape[g.num_dims - 1]);
     const size_t size = static_cast<size_t>(y.numel()) / n;
     hipStream_t s = mi355x::gpu_stream(y);
-    void* ws = mi355x::stream_scratch(s, h2x_softmax_instance_workspace_bytes(n), 2);
-    T* dp = static_cast<T*>(mi355x::stream_scratch(s, 2 * n * sizeof(T), 3));
+    void* ws = mi355x::stream_scratch(s, h2x_softmax_instance_workspace_bytes(n),
+                                      h2x_host::StreamScratch::SOFTMAX_PARTIALS);
+    T* dp = static_cast<T*>(mi355x::stream_scratch(s, 2 * n * sizeof(T),
+                                                      h2x_host::StreamScratch::SOFTMAX_SCALARS));
     const h2x_dtype dt = mi355x::dtype_of<T>();
     mi355x::check(h2x_softmax_instance_dot(dt, n, size, y.const_data(), dy.const_data(), dp, ws, s),
                   "softmax dot");

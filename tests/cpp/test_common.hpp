@@ -7,8 +7,6 @@
 #include <random>
 #include <vector>
 
-#include <unistd.h>
-
 #include <hip/hip_runtime_api.h>
 
 #include "distconv/distconv_mi355x.hpp"
@@ -64,13 +62,14 @@ std::vector<T> global_offset_field(const DevTensor<T>& t, T fill)
     return h;
 }
 
-// Ends a test program once its checks are done and their result is printed, without
-// running exit handlers and static destructors: the order in which the HIP runtime, the
-// OpenMP runtime of the CPU oracle and the program's own statics are torn down is
-// nobody's contract, and a crash in there would hide the result of the checks.
-[[noreturn]] inline void leave(int status)
+// Ends a test program the way an application does: the per-stream workspaces of the layer are
+// handed back, the device is idle, and main returns, so that the exit handlers and static
+// destructors of the program, of libh2x.so and of the HIP runtime run.  Tensors, layers and plans
+// of main's own scope are destroyed by that return, before any exit handler.
+inline int finish(int errors)
 {
-    std::fflush(nullptr);
-    _exit(status);
+    release_workspaces();
+    CHECK(h2x_host::StreamScratch::held_buffers() == 0);
+    DISTCONV_CHECK_HIP(hipDeviceSynchronize());
+    return errors ? 1 : 0;
 }
-

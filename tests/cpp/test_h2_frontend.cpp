@@ -117,6 +117,18 @@ static DTTuple channel_types(int nd)
     return t;
 }
 
+// A strided tensor holding `values` at its elements (natural order), everything else `fill`.
+template <typename T>
+static std::vector<T> scatter_strided(const ShapeTuple& shape, const StrideTuple& strides, size_t span,
+                                      const std::vector<T>& values, T fill)
+{
+    std::vector<T> h(span, fill);
+    size_t i = 0;
+    const StrideTuple s[1] = {strides};
+    mi355x::for_each_element(shape, s, [&](const DataIndexType* o) { h[o[0]] = values[i++]; });
+    return h;
+}
+
 // Batch norm forward + backward through the type-erased operators.
 static void test_batchnorm(const ShapeTuple& shape)
 {
@@ -298,7 +310,14 @@ static void test_errors()
     Tensor<double> ds(Device::GPU, ShapeTuple{3}, DTTuple{DT::Channel}, stream);
     BaseTensor &bx = x, &bds = ds, &bq = q;
     CHECK_THROWS(batchnorm_channel_sums(bx, bds, bq));
-    // registry: register, call, unregister
+}
+
+// The dispatch registry: register, call, unregister (test/unit_test/core/unit_test_dispatch.cpp).
+// Needs no device: keys are made from element types.
+static void test_registry()
+{
+    const ShapeTuple shape{8, 4, 3, 2};
+    Tensor<float> x(Device::CPU, shape, channel_types(4));
     static int calls = 0;
     struct Probe
     {
@@ -318,16 +337,102 @@ static void test_errors()
     CHECK_THROWS(internal::call_dispatch_entry("probe_gpu", key, cbx, five));
 }
 
-// A strided tensor holding `values` at its elements (natural order), everything else `fill`.
-template <typename T>
-static std::vector<T> scatter_strided(const ShapeTuple& shape, const StrideTuple& strides, size_t span,
-                                      const std::vector<T>& values, T fill)
+// The host arms of the operators against plain arithmetic, the operators without a host arm
+// raising for a host tensor, and the OpenMP oracle at work: everything this program does that
+// needs no GPU.  With --host-only the program runs only this and returns from main, so that the
+// exit handlers of a process that has libh2x.so (and with it the HIP runtime) and the OpenMP
+// runtime loaded are exercised where there is no GPU as well.
+static void test_host_arms()
 {
-    std::vector<T> h(span, fill);
-    size_t i = 0;
-    const StrideTuple s[1] = {strides};
-    mi355x::for_each_element(shape, s, [&](const DataIndexType* o) { h[o[0]] = values[i++]; });
-    return h;
+    const ComputeStream cs(Device::CPU);
+    const ShapeTuple shape{7, 5, 3, 2};
+    const StrideTuple halo_strides{1, 9, 9 * 8, 9 * 8 * 3}; // a 7 x 5 interior inside 9 x 8 rows
+    const size_t span = 9 * 8 * 3 * 2;
+    const DTTuple types = channel_types(4);
+    const size_t n = product<size_t>(shape);
+    std::vector<double> vals(n);
+    for (size_t i = 0; i < n; ++i)
+        vals[i] = 0.25 * (double) i - 3.0;
+    const std::vector<double> image = scatter_strided(shape, halo_strides, span, vals, -99.0);
+    std::vector<double> host_a = image, host_b(n, 0.0);
+    Tensor<double> ca(Device::CPU, host_a.data(), shape, types, halo_strides, cs);
+    Tensor<double> cb(Device::CPU, host_b.data(), shape, types, get_contiguous_strides(shape), cs);
+    scale(ca, 2.0);
+    for (size_t i = 0; i < span; ++i)
+        CHECK(host_a[i] == (image[i] == -99.0 ? -99.0 : 2.0 * image[i])); // the gaps are not touched
+    copy_values(ca, cb);
+    for (size_t i = 0; i < n; ++i)
+        CHECK(host_b[i] == 2.0 * vals[i]);
+    BaseTensor &bca = ca, &bcb = cb;
+    scale_bias(bca, bcb, 0.5, 1.0); // type-erased front
+    for (size_t i = 0; i < n; ++i)
+        CHECK(host_b[i] == vals[i] + 1.0);
+    const ShapeTuple rshape{1, 1, 3, 1};
+    std::vector<double> host_r(3, 10.0);
+    Tensor<double> cr(Device::CPU, host_r.data(), rshape, types, get_contiguous_strides(rshape), cs);
+    reduce_sum(ca, cr, true);
+    for (int c = 0; c < 3; ++c)
+    {
+        double want = 10.0;
+        for (int s = 0; s < 2; ++s)
+            for (int i = 0; i < 35; ++i)
+            {
+                const double x = 2.0 * vals[(s * 3 + c) * 35 + i];
+                want += x * x;
+            }
+        CHECK(std::fabs(host_r[c] - want) <= 1e-12 * want);
+    }
+    // halo operators on contiguous tensors whose shape includes the halo
+    const ShapeTuple hshape{10, 6, 3, 2};
+    const size_t ht = product<size_t>(hshape);
+    std::vector<double> c1(ht), c2(ht), cbuf(ht, 0.0);
+    for (size_t i = 0; i < ht; ++i)
+    {
+        c1[i] = 1.0 + (double) i;
+        c2[i] = -2.0 * (double) i;
+    }
+    const std::vector<double> h1 = c1, h2v = c2;
+    Tensor<double> t1(Device::CPU, c1.data(), hshape, types, get_contiguous_strides(hshape), cs);
+    Tensor<double> t2(Device::CPU, c2.data(), hshape, types, get_contiguous_strides(hshape), cs);
+    Tensor<double> tbuf(Device::CPU, cbuf.data(), ShapeTuple{(DimType) ht}, DTTuple{DT::Any}, StrideTuple{1}, cs);
+    clear_halo(t2, 1, 1);
+    for (size_t i = 0; i < ht; ++i)
+    {
+        const size_t h = (i / 10) % 6;
+        CHECK(c2[i] == ((h == 0 || h == 5) ? 0.0 : h2v[i]));
+    }
+    // the RHS boundary column of t1 (w = 8) lands in the LHS halo column of t2 (w = 0)
+    halo_pack(t1, 0, H2X_RHS, 1, tbuf);
+    halo_unpack(t2, 0, H2X_LHS, 1, tbuf);
+    for (size_t row = 0; row < ht / 10; ++row)
+        CHECK(c2[row * 10] == h1[row * 10 + 8]);
+    // a transfer is that pack and unpack in one
+    std::vector<double> c3 = h2v;
+    Tensor<double> t3(Device::CPU, c3.data(), hshape, types, get_contiguous_strides(hshape), cs);
+    halo_transfer(t1, t3, 0, H2X_RHS, 1);
+    for (size_t row = 0; row < ht / 10; ++row)
+        for (int w = 0; w < 10; ++w)
+            CHECK(c3[row * 10 + w] == (w == 0 ? h1[row * 10 + 8] : h2v[row * 10 + w]));
+    Tensor<double> bad(Device::CPU, ShapeTuple{1, 2, 3, 1}, types, cs);
+    CHECK_THROWS(reduce_sum(ca, bad)); // extent 2 is neither 1 nor 5
+
+    // operators without a host arm raise for a host tensor
+    const ShapeTuple fshape{8, 4, 3, 2};
+    Tensor<float> cx(Device::CPU, fshape, channel_types(4)), cy(Device::CPU, fshape, channel_types(4)),
+        csum(Device::CPU, ShapeTuple{3}, DTTuple{DT::Channel}), cq(Device::CPU, ShapeTuple{3}, DTTuple{DT::Channel});
+    CHECK_THROWS(batchnorm_channel_sums(cx, csum, cq));
+    CHECK_THROWS(softmax_channel_forward(cx, cy));
+    CHECK_THROWS(softmax_instance_forward(cx, cy));
+
+    // the oracle on a tensor large enough for its OpenMP team to start: mean 0.3, variance 1
+    const int N = 8, C = 16;
+    const size_t S = 32 * 32;
+    const std::vector<float> hx = randn((size_t) N * C * S, 11, 1.0f, 0.3f);
+    std::vector<float> sums(C), sqsums(C), rm(C, 0.0f), rv(C, 1.0f);
+    orc_bn_channel_sums_and_sqsums_f32(N, C, S, S, hx.data(), sums.data(), sqsums.data());
+    orc_bn_sums_to_statistics_f32(C, (size_t) N * S, 0.9f, sums.data(), sqsums.data(), rm.data(), rv.data());
+    for (int c = 0; c < C; ++c)
+        CHECK(std::fabs(sums[c] - 0.3f) < 0.05f && std::fabs(sqsums[c] - 1.0f) < 0.05f);
 }
 
 // Every operator of tensor_ops_mi355x.hpp on a GPU tensor and on a CPU tensor with the
@@ -540,7 +645,7 @@ static void test_softmax_instance()
         CHECK(std::fabs(gdx[i] - wdx[i]) <= 1e-5 * (std::fabs(gy[i] * hdy[i]) + std::fabs(gy[i])));
 }
 
-int main()
+int main(int argc, char** argv)
 {
     std::setvbuf(stdout, nullptr, _IONBF, 0); // what was printed survives a crash
 #define RUN(call)                                                                                  \
@@ -549,6 +654,13 @@ int main()
         std::printf("%s\n", #call);                                                                \
         call;                                                                                      \
     } while (0)
+    RUN(test_host_arms());
+    RUN(test_registry());
+    if (argc > 1 && std::strcmp(argv[1], "--host-only") == 0)
+    {
+        std::printf("test_h2_frontend: host-only ok\n");
+        return 0;
+    }
     RUN(test_both_arms());
     RUN(test_shuffle());
     RUN(test_softmax_instance());
@@ -560,12 +672,18 @@ int main()
     RUN(test_halo());
     RUN(test_errors());
 #undef RUN
+    release_workspaces();
     check_hip(hipDeviceSynchronize(), "sync");
     std::printf("test_h2_frontend: ok\n");
-    // Leave without running exit handlers and static destructors: the order in which the HIP
-    // runtime, the OpenMP runtime of the CPU oracle and this program's statics are torn down is
-    // nobody's contract, and a crash in there would hide the result of the checks (this program
-    // ended with SIGSEGV after the line above in 2 of about 50 runs).
+    // The GPU run of this one program leaves without exit handlers.  It ended with SIGSEGV after
+    // the line above, i.e. inside the exit handlers, in 2 of about 50 runs on the GPU, and the
+    // cause is not established.  Ruled out: every object of this program that owns device memory,
+    // a plan or a stream has function scope and is gone by now; the headers free nothing from
+    // static destructors; the same exit path with the HIP runtime loaded but not initialised and
+    // the OpenMP team of the oracle alive (--host-only, which returns from main) is clean under
+    // ASan, UBSan and TSan and in hundreds of plain runs.  What is left needs an initialised
+    // runtime: its own teardown beside its helper threads.  The other test programs return from
+    // main and so exercise that path.
     std::fflush(nullptr);
     _exit(0);
 }

@@ -169,5 +169,5 @@ int main()
                 ++errors;
     }
     std::printf("test_halo_exchange_virtual: %d errors\n", errors);
-    leave(errors ? 1 : 0);
+    return finish(errors);
 }

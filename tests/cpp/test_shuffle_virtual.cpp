@@ -136,5 +136,5 @@ int main()
             errors += back[i] != field[i];
     }
     std::printf("test_shuffle_virtual: %d errors\n", errors);
-    leave(errors ? 1 : 0);
+    return finish(errors);
 }
