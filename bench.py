@@ -60,8 +60,8 @@ def _time_events(fn, iters: int, warmup: int, inner: int = 4):
 
 
 def _time_graph(fn, iters: int, warmup: int, inner: int = 4):
-    """Median and minimum milliseconds of one fn() on the GPU, free of host
-    enqueue cost: `inner` calls are captured into one HIP graph and 2 x `inner`
+    """Median and minimum (of the per-iteration differences) milliseconds of one fn() on
+    the GPU, free of host enqueue cost: `inner` calls are captured into one HIP graph and 2 x `inner`
     calls into another, both are replayed between two events, and the difference
     of the two replay times is divided by `inner`.  The difference removes what a
     replay costs besides its kernels (8-25 us between the first event and the
@@ -91,9 +91,49 @@ def _time_graph(fn, iters: int, warmup: int, inner: int = 4):
             e1.synchronize()
             times[which].append(e0.elapsed_time(e1))
     del graphs
-    median = (statistics.median(times[1]) - statistics.median(times[0])) / inner
-    minimum = (min(times[1]) - min(times[0])) / inner
-    return median, minimum
+    # one difference per iteration (the long and the short replay run back to back): their
+    # median, and their minimum, which is the minimum of a difference and not a lower bound
+    diffs = [(b - a) / inner for a, b in zip(*times)]
+    return statistics.median(diffs), min(diffs)
+
+
+def _time_graph_cold(fn, flush, iters: int, warmup: int, inner: int = 2):
+    """GPU time of one fn() whose working set is in no cache when it starts: `flush` (a
+    read-only pass over a buffer twice the size of the 256 MB memory-side cache, launched by
+    the library's own sum kernel) runs before every call inside the graph.  One graph holds
+    `inner` x (flush, fn), the other `inner` x flush; the difference of the two replay times
+    divided by `inner` is the call, free of host enqueue cost and of the flush.  What the call
+    leaves dirty in the caches is written back under the next flush, which both graphs pay
+    alike only in part: the figure is an upper estimate of the cold call."""
+    import torch
+    for _ in range(max(warmup, 1)):
+        flush()
+        fn()
+    torch.cuda.synchronize()
+    graphs = []
+    for with_fn in (False, True):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for _ in range(inner):
+                flush()
+                if with_fn:
+                    fn()
+        for _ in range(2):
+            graph.replay()
+        graphs.append(graph)
+    torch.cuda.synchronize()
+    times = ([], [])
+    for _ in range(iters):
+        for which, graph in enumerate(graphs):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            graph.replay()
+            e1.record()
+            e1.synchronize()
+            times[which].append(e0.elapsed_time(e1))
+    del graphs
+    diffs = [(b - a) / inner for a, b in zip(*times)]
+    return statistics.median(diffs), min(diffs)
 
 
 def _time_events_cold(fn, flush, iters: int, warmup: int):
@@ -234,6 +274,148 @@ class ShuffleWorkload:
 
     def backward(self):
         self.sh.shuffle_backward()
+
+
+# ---------------------------------------------------------------------------------------------
+# Parity gate: every timed configuration's outputs are checked on the GPU before its timing is
+# taken, against the definition of the operation evaluated in float64 by library routines
+# (batch-norm, softmax; bound 1e-5 of the terms of each expression, the bound an fp32 result
+# can meet where terms cancel) or bit for bit against the closed form (halo: every cell of
+# every rank equals the periodic global field; shuffle: every element sits at its global
+# position, and the round trip restores the source).  The full comparison with the CPU oracle
+# is in tests/; this gate keeps a wrong kernel from being timed.
+# ---------------------------------------------------------------------------------------------
+GATE_TOL = 1e-5
+
+
+class ParityError(RuntimeError):
+    pass
+
+
+def _gate(ok: bool, what: str):
+    if not ok:
+        raise ParityError(f"parity gate failed: {what}")
+
+
+def _within(got, want, terms, what):
+    """|got - want| <= GATE_TOL * terms everywhere (terms: sum of the magnitudes of the
+    addends of the expression, the conditioning of its fp32 evaluation)."""
+    import torch
+    err = (got.double() - want).abs()
+    bound = GATE_TOL * terms + 1e-30
+    bad = int((~(err <= bound)).sum())
+    _gate(bad == 0, f"{what}: {bad} of {err.numel()} elements beyond {GATE_TOL:g} of their terms "
+                    f"(largest error {float(err.max()):.3g})")
+    return float((err / (terms + 1e-30)).max())
+
+
+def gate_batchnorm(w: "BatchNormWorkload", backward: bool = True):
+    """mean, var, y (and dscale, dbias, dmean, dvar, dx) of the last forward() / backward()."""
+    import torch
+    x = w.x.interior_view().double()
+    dims = [0] + list(range(2, x.dim()))
+    bshape = [1, -1] + [1] * (x.dim() - 2)
+    n = x.numel() // x.shape[1]
+    m64, v64 = x.mean(dims), x.var(dims, unbiased=True)
+    q64 = (x * x).mean(dims)
+    worst = {}
+    worst["mean"] = _within(w.mean, m64, x.abs().mean(dims), "batch-norm mean")
+    worst["var"] = _within(w.var, v64, q64 + m64 * m64, "batch-norm var")
+    mean, var = w.mean.double(), w.var.double()
+    r = torch.rsqrt(var + 1e-5)
+    scale, bias = w.scale.double(), w.bias.double()
+    xm = x - mean.view(bshape)
+    a = xm * (r * scale).view(bshape)
+    worst["y"] = _within(w.y.interior_view(), a + bias.view(bshape), a.abs() + bias.abs().view(bshape), "batch-norm y")
+    del a
+    if backward:
+        dy = w.dy.interior_view().double()
+        dscale, dbias, dmean, dvar = (g.double() for g in w.grads)
+        t = dy * xm
+        s_dyxm, a_dyxm = t.sum(dims), t.abs().sum(dims)
+        del t
+        s_dy, a_dy = dy.sum(dims), dy.abs().sum(dims)
+        worst["dscale"] = _within(w.grads[0], s_dyxm * r, a_dyxm * r, "batch-norm dscale")
+        worst["dbias"] = _within(w.grads[1], s_dy, a_dy, "batch-norm dbias")
+        worst["dmean"] = _within(w.grads[2], -s_dy * scale * r, a_dy * scale * r, "batch-norm dmean")
+        worst["dvar"] = _within(w.grads[3], -s_dyxm * scale * r ** 3 / 2, a_dyxm * scale * r ** 3 / 2,
+                                "batch-norm dvar")
+        t1 = dy * (scale * r).view(bshape)
+        t2 = (dmean / n).view(bshape)
+        t3 = xm * (dvar * 2 / (n - 1)).view(bshape)
+        worst["dx"] = _within(w.dx.interior_view(), t1 + t2 + t3, t1.abs() + t2.abs() + t3.abs(), "batch-norm dx")
+    return worst
+
+
+def gate_halo(w: "HaloWorkload"):
+    """After an exchange on the periodic grid every cell of every rank, halo cells included,
+    holds the value of the global field at its wrapped global index
+    (legacy/tests/tensor/test_halo_exchange_cuda.cu:104-233), bit for bit."""
+    import torch
+    ranks = w.ranks
+    t0 = ranks[0]
+    nd = len(t0.local_shape)
+    gshape_np = [t0.shape[d] for d in range(nd - 1, -1, -1)]
+    field = torch.empty(gshape_np, dtype=t0.data.dtype, device="cuda")
+    for t in ranks:
+        sl = tuple(slice(g, g + l) for g, l in zip(reversed(t.global_index), reversed(t.local_shape)))
+        field[sl] = t.interior_view()
+    ov = list(reversed(t0.overlap))            # numpy order
+    pad = []
+    for o in reversed(ov[2:]):                 # F.pad takes the last dimension first
+        pad += [o, o]
+    padded = torch.nn.functional.pad(field, pad, mode="circular")
+    del field
+    for r, t in enumerate(ranks):
+        sl = tuple(slice(g, g + l + 2 * o)
+                   for g, l, o in zip(reversed(t.global_index), reversed(t.local_shape), ov))
+        _gate(torch.equal(t.real_view(), padded[sl]), f"halo exchange: rank {r} differs from the periodic field")
+    return {"ranks": len(ranks), "cells_per_rank": int(ranks[0].real_view().numel())}
+
+
+def gate_softmax(w: "SoftmaxWorkload", instance: bool = False):
+    import torch
+    x = w.x.interior_view().double()
+    y = w.y.interior_view()
+    if instance:
+        want = torch.softmax(x.flatten(1), 1).view_as(x)
+    else:
+        want = torch.softmax(x, 1)
+    # the reference clamps y to FLT_MIN from below (softmax.cu:565,590)
+    want = want.clamp_min(1.1754943508222875e-38)
+    worst = {"y": _within(y, want, want, "softmax y")}
+    y64, dy = y.double(), w.dy.interior_view().double()
+    if instance:
+        dp = (y64 * dy).flatten(1).sum(1).view([-1] + [1] * (x.dim() - 1))
+    else:
+        dp = (y64 * dy).sum(1, keepdim=True)
+    want_dx = y64 * (dy - dp)
+    terms = (y64 * dy).abs() + (y64 * dp).abs()
+    # y at the clamp gives dx = 0 in the reference (softmax.cu:666); N(0, 2) logits never get there
+    worst["dx"] = _within(w.dx.interior_view(), want_dx, terms, "softmax dx")
+    return worst
+
+
+def gate_shuffle(w: "ShuffleWorkload"):
+    """forward: every destination rank holds its part of the global tensor; backward into
+    cleared sources: the sources are back, bit for bit
+    (legacy/tests/tensor/test_tensor_mpi_shuffle.cpp:26-154)."""
+    import torch
+    nd = len(w.src[0].local_shape)
+    gshape_np = [w.src[0].shape[d] for d in range(nd - 1, -1, -1)]
+    field = torch.empty(gshape_np, dtype=w.src[0].data.dtype, device="cuda")
+    part = lambda t: tuple(slice(g, g + l) for g, l in zip(reversed(t.global_index), reversed(t.local_shape)))
+    for t in w.src:
+        field[part(t)] = t.interior_view()
+    w.forward()
+    for r, t in enumerate(w.dst):
+        _gate(torch.equal(t.interior_view(), field[part(t)]), f"shuffle forward: destination rank {r}")
+    for t in w.src:
+        t.data.zero_()
+    w.backward()
+    for r, t in enumerate(w.src):
+        _gate(torch.equal(t.interior_view(), field[part(t)]), f"shuffle backward: source rank {r}")
+    return {"elements": int(field.numel())}
 
 
 def _cpu_model() -> str:
@@ -624,6 +806,9 @@ def main() -> int:
     step()  # the fused entry points once, untimed (first-use allocations)
     torch.cuda.synchronize()
     events.clear()
+    # parity gate of the step's two configurations, before the timed region
+    parity = {"C3_bn3d_fwd_bwd": gate_batchnorm(bn3), "C2_halo_8ranks": gate_halo(halo)}
+    torch.cuda.synchronize()
 
     # timed region: only the dominant kernel's launches carry events, and only in every
     # EVENT_EVERY-th step (a pair of timing events costs the stream 2-3 us: bracketing all four
@@ -706,10 +891,28 @@ def main() -> int:
                 e["ms_eager_median"] = _time_events(fn, it, wu, inner)[0]
             return e
 
+        evict = torch.empty(1 << 27, device="cuda").fill_(1.0)   # 512 MB: twice the memory-side cache
+        from dihydrogen_amd import layers as L
+        from dihydrogen_amd.tensor import Distribution as _D, LocaleVirtual as _LV, Tensor as _T
+        evict_t = _T([1 << 21, 1, 1, 64, 1], _LV(0, 1), _D.make_localized_distribution(5))
+        evict_t.data = evict
+        evict_stat = _T([1, 1, 1, 64, 1], _LV(0, 1), _D.make_localized_distribution(5)).allocate()
+        flush_in_graph = lambda: L.reduce_sum(evict_t, evict_stat)   # a read-only pass, the library's own kernel
+
+        def cold_entry(nbytes, elems, fn, inner=2):
+            med, mn = _time_graph_cold(fn, flush_in_graph, it, wu, inner)
+            return {"bytes": nbytes, "ms_median": med, "ms_min": mn, "GB/s": _gbs(nbytes, med),
+                    "frac_of_peak": _gbs(nbytes, med) / HBM_PEAK_GBS, "Gelem/s": elems / (med * 1e-3) / 1e9,
+                    "timing": "HIP-graph replay of (512 MB read-only flush, call) pairs minus the replay of the "
+                              "flushes alone (GPU time, caches cold)"}
+
         breakdown["C3_bn3d_fwd"] = entry(3 * S3 * 4, S3, bn3.forward)
         breakdown["C3_bn3d_bwd"] = entry(5 * S3 * 4, S3, bn3.backward)
         breakdown["C3_bn3d_fwd_bwd"] = entry(8 * S3 * 4, S3, lambda: (bn3.forward(), bn3.backward()), inner=2)
+        breakdown["C3_bn3d_fwd_bwd_cold"] = cold_entry(8 * S3 * 4, S3, lambda: (bn3.forward(), bn3.backward()), inner=1)
         bn3.bn.fuse_local = False
+        bn3.forward(), bn3.backward()
+        parity["C3_bn3d_fwd_bwd_staged"] = gate_batchnorm(bn3)
         breakdown["C3_bn3d_fwd_bwd_staged"] = entry(8 * S3 * 4, S3, lambda: (bn3.forward(), bn3.backward()), inner=2)
         bn3.bn.fuse_local = True
         breakdown["C2_halo_8ranks"] = entry(halo.bytes, halo.elems, halo.run, inner=2)
@@ -717,7 +920,16 @@ def main() -> int:
             ov = [1 if k == d else 0 for k in range(5)]
             fn = lambda ov=ov: halo.xch.exchange(ov, ov, ov, ov)
             breakdown[f"C2_halo_{name}"] = entry(halo.bytes // 3, halo.elems // 3, fn)
+            breakdown[f"C2_halo_{name}_cold"] = cold_entry(halo.bytes // 3, halo.elems // 3, fn)
+        breakdown["C2_halo_8ranks_cold"] = cold_entry(halo.bytes, halo.elems, halo.run, inner=1)
         # the same exchange as tensor-to-tensor transfers (no buffers): half the bytes per strip
+        for t in halo.ranks:          # poison the halos: the fused exchange has to fill every cell again
+            keep = t.interior_view().clone()
+            t.real_view().fill_(float("nan"))
+            t.interior_view().copy_(keep)
+        del keep
+        halo.xch.exchange(fused=True)
+        parity["C2_halo_8ranks_fused"] = gate_halo(halo)
         breakdown["C2_halo_8ranks_fused"] = entry(halo.bytes // 2, halo.elems // 2,
                                                   lambda: halo.xch.exchange(fused=True), inner=2)
         for d, name in enumerate(("dim0_W", "dim1_H", "dim2_D")):
@@ -742,12 +954,16 @@ def main() -> int:
             lambda: halo.xch.exchange(is_reverse=True, op=HaloExchangeAccumOp.SUM), inner=2)
         # tensor::Transform / ReduceSum at the config 3 shape: scale in place (read + write), copy into a
         # second tensor (read + write), per-channel sums and sums of squares (one read each)
-        from dihydrogen_amd import layers as L
-        from dihydrogen_amd.tensor import Distribution as _D, LocaleVirtual as _LV, Tensor as _T
         breakdown["C3_transform_scale"] = entry(2 * S3 * 4, S3, lambda: L.transform(capi.TRANSFORM_SCALE, [bn3.y], [1.0]))
         breakdown["C3_transform_copy"] = entry(2 * S3 * 4, S3, lambda: L.transform(capi.TRANSFORM_COPY, [bn3.x, bn3.y]))
         stat = _T([1, 1, 1, 64, 1], _LV(0, 1), _D.make_localized_distribution(5)).allocate()
+        stat.data.zero_()
+        L.reduce_sum(bn3.x, stat)
+        want = bn3.x.interior_view().double().sum((0, 2, 3, 4))
+        parity["C3_reduce_sum_per_channel"] = {"sum": _within(
+            stat.data.view(-1), want, bn3.x.interior_view().double().abs().sum((0, 2, 3, 4)), "reduce_sum")}
         breakdown["C3_reduce_sum_per_channel"] = entry(S3 * 4, S3, lambda: L.reduce_sum(bn3.x, stat))
+        breakdown["C3_reduce_sum_per_channel_cold"] = cold_entry(S3 * 4, S3, lambda: L.reduce_sum(bn3.x, stat))
         breakdown["C3_reduce_sqsum_per_channel"] = entry(S3 * 4, S3, lambda: L.reduce_sum(bn3.x, stat, square=True))
         # what a convolution does before it runs (convolution.hpp:400-411): clear the halos, exchange.
         # Bytes: the exchange's; the clearing is overhead.  On the periodic grid every strip is overwritten
@@ -771,20 +987,25 @@ def main() -> int:
         torch.cuda.empty_cache()
         # strided batch-norm: the config 3 shard with a halo of 1 on all three spatial dimensions
         bn3h = BatchNormWorkload((4, 64, 64, 64, 64), SEED + 6, overlap=1)
+        bn3h.forward(), bn3h.backward()
+        parity["C3_bn3d_haloed_fwd_bwd"] = gate_batchnorm(bn3h)
         breakdown["C3_bn3d_haloed_fwd_bwd"] = entry(8 * bn3h.elems * 4, bn3h.elems,
                                                     lambda: (bn3h.forward(), bn3h.backward()), inner=2)
         del bn3h
         torch.cuda.empty_cache()
         # short segments (the last stage of a ResNet): a workgroup serves a window of whole channels
         bn7 = BatchNormWorkload((256, 2048, 7, 7), SEED + 7)
+        bn7.forward(), bn7.backward()
+        parity["bn2d_7x7_N256_C2048"] = gate_batchnorm(bn7)
         breakdown["bn2d_7x7_N256_C2048_fwd"] = entry(3 * bn7.elems * 4, bn7.elems, bn7.forward)
         breakdown["bn2d_7x7_N256_C2048_bwd"] = entry(5 * bn7.elems * 4, bn7.elems, bn7.backward)
         del bn7
         torch.cuda.empty_cache()
         # configs 1 and 4 fit in the memory-side cache: warm = back to back, cold = after a 512 MB read
-        evict = torch.empty(1 << 27, device="cuda").fill_(1.0)
         flush = lambda: evict.sum()
         bn1 = BatchNormWorkload((8, 64, 56, 56), SEED + 1)
+        bn1.forward()
+        parity["C1_bn2d_fwd"] = gate_batchnorm(bn1, backward=False)
         breakdown["C1_bn2d_fwd"] = entry(3 * bn1.elems * 4, bn1.elems, bn1.forward)
         med, mn = _time_events_cold(bn1.forward, flush, it, wu)
         breakdown["C1_bn2d_fwd_cold"] = {
@@ -792,10 +1013,13 @@ def main() -> int:
             "frac_of_peak": _gbs(3 * bn1.elems * 4, med) / HBM_PEAK_GBS,
             "timing": "events around one eager call after a cache-evicting read (2 launches)"}
         bn1.bn.fuse_local = False
+        bn1.forward()
+        parity["C1_bn2d_fwd_staged"] = gate_batchnorm(bn1, backward=False)
         breakdown["C1_bn2d_fwd_staged"] = entry(3 * bn1.elems * 4, bn1.elems, bn1.forward)
         del bn1
         sm = SoftmaxWorkload((16, 21, 256, 256), SEED + 4)
-        sm.forward()
+        sm.forward(), sm.backward()
+        parity["C4_softmax"] = gate_softmax(sm)
         breakdown["C4_softmax_fwd"] = entry(2 * sm.elems * 4, sm.elems, sm.forward)
         breakdown["C4_softmax_bwd"] = entry(3 * sm.elems * 4, sm.elems, sm.backward)
         for name, fn, nb in (("fwd", sm.forward, 2), ("bwd", sm.backward, 3)):
@@ -809,30 +1033,38 @@ def main() -> int:
         # times and writes y once (max, sum of exponentials, y from x), backward reads y and dy twice
         # and writes dx
         smi = SoftmaxWorkload((16, 21, 256, 256), SEED + 4, instance=True)
-        smi.forward()
+        smi.forward(), smi.backward()
+        parity["C4_softmax_instance"] = gate_softmax(smi, instance=True)
         breakdown["C4_softmax_instance_fwd"] = entry(4 * smi.elems * 4, smi.elems, smi.forward)
         breakdown["C4_softmax_instance_bwd"] = entry(5 * smi.elems * 4, smi.elems, smi.backward)
-        del smi, evict
+        del smi
         torch.cuda.empty_cache()
         shf = ShuffleWorkload((128, 128, 64, 32), SEED + 5)
+        parity["C5_shuffle"] = gate_shuffle(shf)
         breakdown["C5_shuffle_fwd"] = entry(4 * shf.elems * 4, shf.elems, shf.forward)
         breakdown["C5_shuffle_bwd"] = entry(4 * shf.elems * 4, shf.elems, shf.backward)
         breakdown["C5_shuffle_round_trip"] = entry(8 * shf.elems * 4, 2 * shf.elems,
                                                    lambda: (shf.forward(), shf.backward()), inner=2)
+        breakdown["C5_shuffle_fwd_cold"] = cold_entry(4 * shf.elems * 4, shf.elems, shf.forward)
+        breakdown["C5_shuffle_bwd_cold"] = cold_entry(4 * shf.elems * 4, shf.elems, shf.backward)
+        breakdown["C5_shuffle_round_trip_cold"] = cold_entry(8 * shf.elems * 4, 2 * shf.elems,
+                                                             lambda: (shf.forward(), shf.backward()), inner=1)
         del shf
         torch.cuda.empty_cache()
         # the spatial side with a halo of 1 (what a convolution behind the shuffle needs): the unpack
         # writes rows of 64 floats into rows of 66, the backward pack reads them
         shfh = ShuffleWorkload((128, 128, 64, 32), SEED + 5, dst_overlap=1)
+        parity["C5_shuffle_haloed_dst"] = gate_shuffle(shfh)
         breakdown["C5_shuffle_haloed_dst_round_trip"] = entry(8 * shfh.elems * 4, 2 * shfh.elems,
                                                               lambda: (shfh.forward(), shfh.backward()), inner=2)
         del shfh
         torch.cuda.empty_cache()
         # the same tensor between 16 ranks: 256 boxes a direction, one launch each for pack and unpack
         shf16 = ShuffleWorkload((128, 128, 64, 32), SEED + 5, ranks=16, grid=(4, 4))
+        parity["C5_shuffle_16ranks"] = gate_shuffle(shf16)
         breakdown["C5_shuffle_16ranks_round_trip"] = entry(8 * shf16.elems * 4, 2 * shf16.elems,
                                                            lambda: (shf16.forward(), shf16.backward()), inner=2)
-        del shf16
+        del shf16, evict, evict_t, evict_stat
         torch.cuda.empty_cache()
 
     out = {
@@ -858,6 +1090,8 @@ def main() -> int:
         "frac_of_hbm_peak": value / HBM_PEAK_GBS,
         "elements_per_s": step_elems / (ms_per_step * 1e-3),
         "kernel_sources": sources_sha,
+        "parity_gate": "ok",
+        "parity": parity,
         "roofline": roofline,
         "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline(),
         "launches": launches,
@@ -868,4 +1102,8 @@ def main() -> int:
 
 
 if __name__ == "__main__":
-    sys.exit(main())
+    try:
+        sys.exit(main())
+    except ParityError as e:
+        print(f"bench.py: {e}", file=sys.stderr)
+        sys.exit(1)

@@ -33,6 +33,66 @@ def bn_inputs(shape_ncs, seed, dtype=np.float32):
     return x, dy, scale, bias
 
 
+def glibc_rand(seed: int, count: int) -> np.ndarray:
+    """The first ``count`` values of ``srand(seed); rand()`` of the GNU C library (its
+    additive-feedback generator of degree 31; ``RAND_MAX`` = 2**31 - 1), restated here so
+    that the values do not depend on the C library of the machine and drawing them leaves
+    the process's own generator alone.  tests/test_oracle_bn.py pins it on the C library."""
+    seed = seed or 1                     # srand(0) seeds with 1
+    r = [0] * (344 + count)
+    r[0] = seed
+    for i in range(1, 31):
+        # 16807 * r[i-1] mod (2**31 - 1) on the signed 32-bit value, by Schrage's method
+        prev = _to_signed(r[i - 1])
+        hi = int(prev / 127773)          # C division: towards zero
+        lo = prev - hi * 127773
+        word = 16807 * lo - 2836 * hi
+        r[i] = (word + 2147483647 if word < 0 else word) & 0xffffffff
+    for i in range(31, 34):
+        r[i] = r[i - 31]
+    for i in range(34, 344 + count):
+        r[i] = (r[i - 31] + r[i - 3]) & 0xffffffff
+    return np.array([v >> 1 for v in r[344:]], dtype=np.int64)
+
+
+def _to_signed(v: int) -> int:
+    return v - (1 << 32) if v & 0x80000000 else v
+
+
+def reference_initializer(shape_ncs, seed, num_rands=100, global_shape=None, global_index=None,
+                          dtype=np.float32):
+    """The input generator of the reference's benchmarks and validation runs
+    (legacy/benchmarks/benchmark_common.hpp:46-79, used by distconv_benchmark_bn.cpp:200-213
+    with seeds 0 for the input and 2 for d_output): a table of ``num_rands`` values of
+    ``rand()``; the element at global index i gets
+    (table[sum(i) % num_rands] + table[offset(i) % num_rands]) / 2 / RAND_MAX, its offset taken
+    in the global tensor, innermost dimension fastest.  Values lie in [0, 1) with mean 1/2.
+    ``shape_ncs``, ``global_shape`` and ``global_index`` are in numpy order (N, C, *spatial)."""
+    table = glibc_rand(seed, num_rands).astype(np.float64) / 2147483647.0
+    nd = len(shape_ncs)
+    gshape = tuple(global_shape) if global_shape is not None else tuple(shape_ncs)
+    gidx = tuple(global_index) if global_index is not None else (0,) * nd
+    # both table indices are sums of per-axis terms taken modulo num_rands: small integers
+    total = np.zeros((1,) * nd, np.int16)
+    offset = np.zeros((1,) * nd, np.int16)
+    stride = 1
+    for axis in range(nd - 1, -1, -1):
+        view = [1] * nd
+        view[axis] = shape_ncs[axis]
+        i = np.arange(shape_ncs[axis], dtype=np.int64) + gidx[axis]
+        total = total + (i % num_rands).astype(np.int16).reshape(view)
+        offset = offset + ((i * stride) % num_rands).astype(np.int16).reshape(view)
+        stride *= gshape[axis]
+    # one gather from the table of all pairs, each pair averaged in double and rounded once
+    pairs = ((table[:, None] + table[None, :]) / 2).astype(dtype).ravel()
+    total %= num_rands
+    offset %= num_rands
+    index = total.astype(np.int32)
+    index *= num_rands
+    index += offset
+    return pairs[index]
+
+
 # ---------------------------------------------------------------------------
 # virtual ranks on the CPU, driven through the oracle
 # ---------------------------------------------------------------------------

@@ -281,3 +281,73 @@ def test_strided_equals_dense_on_the_interior(shape, halo):
     oracle.bn_backprop2_strided(xf, lshape, xs, df, ds, dx_real.reshape(-1)[xb:], xs, n, mean, var, scale,
                                 g0[2], g0[3], EPS)
     assert np.array_equal(dx_real[inner], dx0)
+
+
+def test_glibc_rand_restated_equals_the_c_library():
+    """helpers.glibc_rand against srand() / rand() of the C library of this machine."""
+    import ctypes
+    from helpers import glibc_rand
+    libc = ctypes.CDLL("libc.so.6")
+    for seed in (0, 1, 2, 12345, 2 ** 31 + 5):
+        libc.srand(seed)
+        assert [libc.rand() for _ in range(400)] == list(glibc_rand(seed, 400))
+
+
+def test_reference_initializer_by_brute_force():
+    """helpers.reference_initializer against the loop of
+    legacy/benchmarks/benchmark_common.hpp:56-72 on a rank's part of a global tensor."""
+    from helpers import glibc_rand, reference_initializer
+    table = glibc_rand(2, 100) / 2147483647.0
+    local, gshape, gidx = (2, 3, 4, 5), (4, 3, 8, 10), (2, 0, 4, 5)
+    got = reference_initializer(local, 2, global_shape=gshape, global_index=gidx)
+    for i in np.ndindex(*local):
+        g = [a + b for a, b in zip(i, gidx)]
+        offset = g[3] + gshape[3] * (g[2] + gshape[2] * (g[1] + gshape[1] * g[0]))
+        assert got[i] == np.float32((table[sum(g) % 100] + table[offset % 100]) / 2)
+
+
+@pytest.mark.parametrize("offset_case", [False, True])
+def test_inputs_whose_variance_cancels(offset_case):
+    """The reference validates on values in [0, 1) with scale 1, bias 0 (variance cancels 4x);
+    with x ~ N(10, 1) it cancels 100x.  The oracle's fp32 formulas against float64, each
+    bounded by the conditioning of its own expression."""
+    from helpers import reference_initializer
+    shape = (4, 6, 10, 12)
+    if offset_case:
+        rng = np.random.default_rng(8)
+        x = (10 + rng.standard_normal(shape)).astype(np.float32)
+        dy = rng.standard_normal(shape).astype(np.float32)
+    else:
+        x, dy = reference_initializer(shape, 0), reference_initializer(shape, 2)
+    c = shape[1]
+    scale, bias = np.ones(c, np.float32), np.zeros(c, np.float32)
+    rm, rv = np.zeros(c, np.float32), np.ones(c, np.float32)
+    y, mean, var = oracle.bn_forward(x, scale, bias, rm, rv, EPS, 0.9)
+    ax, n = _axes(x), x.size // c
+    x64, dy64 = x.astype(np.float64), dy.astype(np.float64)
+    m64, q64 = x64.mean(axis=ax), (x64 * x64).mean(axis=ax)
+    v64 = (q64 - m64 * m64) * n / (n - 1)
+    u = 2.0 ** -24
+    assert (np.abs(mean - m64) <= 2 * u * np.abs(m64)).all()
+    # var = (q/n - mean^2) * n/(n-1): the error of either term, not of their difference
+    assert (np.abs(var - v64) <= 6 * u * (q64 + m64 * m64)).all()
+    cancel = (q64 + m64 * m64) / v64
+    assert cancel.min() > (50 if offset_case else 4)
+    assert (np.abs(rm - 0.1 * m64) <= 4 * u * np.abs(m64)).all()
+    assert (np.abs(rv - (0.9 + 0.1 * v64)) <= 6 * u * (1 + q64 + m64 * m64)).all()
+    # elementwise outputs against float64 from the oracle's own (rounded) statistics
+    r = 1 / np.sqrt(var.astype(np.float64) + EPS)
+    mb, rb = mean.astype(np.float64).reshape(_bshape(x)), r.reshape(_bshape(x))
+    assert np.abs(y - (x64 - mb) * rb).max() <= 8 * u * np.abs((x64 - mb) * rb).max()
+    dx, dscale, dbias, dmean, dvar = oracle.bn_backward(x, dy, mean, var, scale, EPS)
+    xm = x64 - mb
+    assert (np.abs(dbias - dy64.sum(axis=ax)) <= 4 * u * np.abs(dy64).sum(axis=ax)).all()
+    assert (np.abs(dscale - (dy64 * xm).sum(axis=ax) * r) <= 8 * u * np.abs(dy64 * xm).sum(axis=ax) * r).all()
+    assert (np.abs(dmean + dy64.sum(axis=ax) * r) <= 8 * u * np.abs(dy64).sum(axis=ax) * r).all()
+    assert (np.abs(dvar + (dy64 * xm).sum(axis=ax) * r ** 3 / 2)
+            <= 8 * u * np.abs(dy64 * xm).sum(axis=ax) * r ** 3 / 2).all()
+    want_dx = (dy64 * rb + dmean.astype(np.float64).reshape(_bshape(x)) / n
+               + dvar.astype(np.float64).reshape(_bshape(x)) * 2 / (n - 1) * xm)
+    terms = (np.abs(dy64 * rb) + np.abs(dmean.reshape(_bshape(x))) / n
+             + np.abs(dvar.reshape(_bshape(x)) * 2 / (n - 1) * xm))
+    assert (np.abs(dx - want_dx) <= 8 * u * terms).all()
