@@ -385,12 +385,14 @@ def gate_softmax(w: "SoftmaxWorkload", instance: bool = False):
     want = want.clamp_min(1.1754943508222875e-38)
     worst = {"y": _within(y, want, want, "softmax y")}
     y64, dy = y.double(), w.dy.interior_view().double()
+    ydy = y64 * dy
     if instance:
-        dp = (y64 * dy).flatten(1).sum(1).view([-1] + [1] * (x.dim() - 1))
+        dp = ydy.flatten(1).sum(1).view([-1] + [1] * (x.dim() - 1))
+        adp = ydy.abs().flatten(1).sum(1).view([-1] + [1] * (x.dim() - 1))
     else:
-        dp = (y64 * dy).sum(1, keepdim=True)
+        dp, adp = ydy.sum(1, keepdim=True), ydy.abs().sum(1, keepdim=True)
     want_dx = y64 * (dy - dp)
-    terms = (y64 * dy).abs() + (y64 * dp).abs()
+    terms = ydy.abs() + y64 * adp       # dp itself is a sum that cancels: its terms count, not its value
     # y at the clamp gives dx = 0 in the reference (softmax.cu:666); N(0, 2) logits never get there
     worst["dx"] = _within(w.dx.interior_view(), want_dx, terms, "softmax dx")
     return worst
