@@ -232,58 +232,79 @@ __device__ __forceinline__ int64_t chain(uint32_t i, int nd, const FastDiv* div,
 // element's addends; neighbouring threads read neighbouring addends, VEC at a
 // time (VEC > 1: the innermost reduced dimension is contiguous and a multiple of
 // VEC long, and so is the group size), four loads in flight per thread.
-template <typename T, int VEC>
+// RUN: every group lies within one run of the innermost reduced dimension, which
+// is contiguous: the group's first addend is located once and the others follow
+// it in memory (no index splitting per load).
+template <typename T, int VEC, bool SQUARE, bool RUN>
 __global__ __launch_bounds__(kBlockSize) void reduce_inner_kernel(const ReduceArgs a)
 {
     typedef T Vec __attribute__((ext_vector_type(VEC), aligned(sizeof(T))));
     constexpr int kInFlight = 4;
     __shared__ double lds[kWavesPerBlock];
-    const uint32_t k = blockIdx.x, g = blockIdx.y;
-    const T* src = reinterpret_cast<const T*>(a.src)
-                   + chain(k, a.num_kept, a.kept_div, a.kept_src, nullptr, nullptr);
+    // Groups count fastest (blockIdx.x): workgroups that start together then read
+    // neighbouring chunks of one output's addends.  With the outputs fastest they
+    // would start a whole kept-dimension stride apart, a power of two at the usual
+    // shapes, and crowd a few memory channels.
+    const uint32_t g = blockIdx.x;
     const uint32_t begin = g * a.chunk;
     const uint32_t end = begin + a.chunk < a.red_count ? begin + a.chunk : a.red_count;
-    double acc[1] = {0.0};
-    auto add = [&](T v) {
-        const double x = static_cast<double>(v);
-        acc[0] += a.square ? x * x : x;
-    };
     constexpr uint32_t kStep = kBlockSize * VEC;
-    uint32_t r = begin + threadIdx.x * VEC;
-    for (; r + (kInFlight - 1) * kStep < end; r += kInFlight * kStep)
+    const int64_t run_start =
+        RUN ? chain(begin, a.num_reduced, a.red_div, a.red_src, nullptr, nullptr) - begin : 0;
+    auto locate = [&](uint32_t r) -> int64_t {
+        if constexpr (RUN)
+            return run_start + r;
+        else
+            return chain(r, a.num_reduced, a.red_div, a.red_src, nullptr, nullptr);
+    };
+    for (uint32_t k = blockIdx.y; k < a.kept_count; k += gridDim.y)
     {
-        Vec v[kInFlight];
+        const T* src = reinterpret_cast<const T*>(a.src)
+                       + chain(k, a.num_kept, a.kept_div, a.kept_src, nullptr, nullptr);
+        double acc[1] = {0.0};
+        auto add = [&](T v) {
+            const double x = static_cast<double>(v);
+            if constexpr (SQUARE && sizeof(T) == 4)
+                acc[0] = __builtin_fma(x, x, acc[0]); // the product of two floats is exact in fp64
+            else if constexpr (SQUARE)
+                acc[0] += x * x;
+            else
+                acc[0] += x;
+        };
+        uint32_t r = begin + threadIdx.x * VEC;
+        for (; r + (kInFlight - 1) * kStep < end; r += kInFlight * kStep)
+        {
+            Vec v[kInFlight];
 #pragma unroll
-        for (int u = 0; u < kInFlight; ++u)
-            v[u] = *reinterpret_cast<const Vec*>(
-                src + chain(r + u * kStep, a.num_reduced, a.red_div, a.red_src, nullptr, nullptr));
+            for (int u = 0; u < kInFlight; ++u)
+                v[u] = *reinterpret_cast<const Vec*>(src + locate(r + u * kStep));
 #pragma unroll
-        for (int u = 0; u < kInFlight; ++u)
+            for (int u = 0; u < kInFlight; ++u)
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+                    add(v[u][j]);
+        }
+        for (; r < end; r += kStep)
+        {
+            const Vec v = *reinterpret_cast<const Vec*>(src + locate(r));
 #pragma unroll
             for (int j = 0; j < VEC; ++j)
-                add(v[u][j]);
-    }
-    for (; r < end; r += kStep)
-    {
-        const Vec v = *reinterpret_cast<const Vec*>(
-            src + chain(r, a.num_reduced, a.red_div, a.red_src, nullptr, nullptr));
-#pragma unroll
-        for (int j = 0; j < VEC; ++j)
-            add(v[j]);
-    }
-    block_sum<1>(acc, lds);
-    if (threadIdx.x == 0)
-    {
-        if (a.groups == 1) // the only group of its output: no finishing launch
-        {
-            int64_t dst_off;
-            chain(k, a.num_kept, a.kept_div, a.kept_src, a.kept_dst, &dst_off);
-            T* p = reinterpret_cast<T*>(a.dst) + dst_off;
-            *p = *p + static_cast<T>(acc[0]);
+                add(v[j]);
         }
-        else
+        block_sum<1>(acc, lds);
+        if (threadIdx.x == 0)
         {
-            a.partials[static_cast<size_t>(k) * a.groups + g] = acc[0];
+            if (a.groups == 1) // the only group of its output: no finishing launch
+            {
+                int64_t dst_off;
+                chain(k, a.num_kept, a.kept_div, a.kept_src, a.kept_dst, &dst_off);
+                T* p = reinterpret_cast<T*>(a.dst) + dst_off;
+                *p = *p + static_cast<T>(acc[0]);
+            }
+            else
+            {
+                a.partials[static_cast<size_t>(k) * a.groups + g] = acc[0];
+            }
         }
     }
 }
@@ -401,18 +422,23 @@ __global__ __launch_bounds__(kBlockSize) void reduce_finish_wide_kernel(const Re
 {
     __shared__ double lds[kWavesPerBlock];
     const uint32_t k = blockIdx.x;
+    // the value to add to is asked for first, so that its latency passes with the partials'
+    T* p = nullptr;
+    T before = T(0);
+    if (threadIdx.x == 0)
+    {
+        int64_t dst_off;
+        chain(k, a.num_kept, a.kept_div, a.kept_src, a.kept_dst, &dst_off);
+        p = reinterpret_cast<T*>(a.dst) + dst_off;
+        before = *p;
+    }
     double t[1] = {0.0};
     for (uint32_t g = threadIdx.x; g < a.groups; g += kBlockSize)
         t[0] += inner ? a.partials[static_cast<size_t>(k) * a.groups + g]
                       : a.partials[static_cast<size_t>(g) * a.kept_count + k];
     block_sum<1>(t, lds);
     if (threadIdx.x == 0)
-    {
-        int64_t dst_off;
-        chain(k, a.num_kept, a.kept_div, a.kept_src, a.kept_dst, &dst_off);
-        T* p = reinterpret_cast<T*>(a.dst) + dst_off;
-        *p = *p + static_cast<T>(t[0]);
-    }
+        *p = before + static_cast<T>(t[0]);
 }
 
 // ---- host ---------------------------------------------------------------------
@@ -608,10 +634,27 @@ int reduce_typed(const ReducePlan& plan, hipStream_t stream)
     }
     if (plan.inner)
     {
+        const dim3 grid(a.groups, std::min<uint32_t>(a.kept_count, 65535u));
+        // every group within one contiguous run of the innermost reduced dimension?
+        const bool run = a.num_reduced > 0 && a.red_src[0] == 1
+                         && (a.num_reduced == 1 || a.red_div[0].divisor % a.chunk == 0);
+#define H2X_REDUCE_INNER(VEC)                                                                      \
+    do                                                                                             \
+    {                                                                                              \
+        if (a.square && run)                                                                       \
+            reduce_inner_kernel<T, VEC, true, true><<<grid, kBlockSize, 0, stream>>>(a);           \
+        else if (a.square)                                                                         \
+            reduce_inner_kernel<T, VEC, true, false><<<grid, kBlockSize, 0, stream>>>(a);          \
+        else if (run)                                                                              \
+            reduce_inner_kernel<T, VEC, false, true><<<grid, kBlockSize, 0, stream>>>(a);          \
+        else                                                                                       \
+            reduce_inner_kernel<T, VEC, false, false><<<grid, kBlockSize, 0, stream>>>(a);         \
+    } while (0)
         if (plan.vec == kVec)
-            reduce_inner_kernel<T, kVec><<<dim3(a.kept_count, a.groups), kBlockSize, 0, stream>>>(a);
+            H2X_REDUCE_INNER(kVec);
         else
-            reduce_inner_kernel<T, 1><<<dim3(a.kept_count, a.groups), kBlockSize, 0, stream>>>(a);
+            H2X_REDUCE_INNER(1);
+#undef H2X_REDUCE_INNER
     }
     else if (plan.outer_vec == kVec)
     {
