@@ -600,7 +600,7 @@ KERNEL_OF = {
 
 
 # the sources of the kernels of the step (batch-norm and box copy), whose traffic PMC_TRAFFIC holds
-STEP_KERNEL_SOURCES = ("h2x_bn.hip", "h2x_copy.hip", "h2x_copy_acc.hip", "h2x_copy_kernel.hpp", "h2x_device.hpp")
+STEP_KERNEL_SOURCES = ("h2x_bn.hip", "h2x_bn_maps.hpp", "h2x_copy.hip", "h2x_copy_acc.hip", "h2x_copy_kernel.hpp", "h2x_device.hpp")
 
 
 def kernel_sources_sha() -> str:

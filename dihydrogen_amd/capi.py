@@ -7,7 +7,7 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import POINTER, c_double, c_int, c_int32, c_int64, c_size_t, c_void_p
+from ctypes import POINTER, c_double, c_int, c_int32, c_int64, c_size_t, c_uint32, c_uint64, c_void_p
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libh2x.so")
@@ -68,6 +68,34 @@ class TensorGeometry(ctypes.Structure):
     ]
 
 
+BN_STAGE_SUMS, BN_STAGE_NORMALIZE, BN_STAGE_BACKPROP1, BN_STAGE_BACKPROP2 = 0, 1, 2, 3
+BN_STAGE_FORWARD_LOCAL, BN_STAGE_BACKWARD_LOCAL = 4, 5
+BN_AUDIT_MAX_LAUNCHES = 8
+
+
+class BnAuditTensor(ctypes.Structure):
+    """struct h2x_bn_audit_tensor"""
+    _fields_ = [("loads", c_uint64), ("stores", c_uint64), ("outside", c_uint64), ("missed", c_uint64),
+                ("owned_twice", c_uint64)]
+
+
+class BnAuditLaunch(ctypes.Structure):
+    """struct h2x_bn_audit_launch"""
+    _fields_ = [
+        ("kernel", c_int32), ("family", c_int32), ("vector_width", c_int32), ("tail", c_int32),
+        ("folded", c_int32), ("fused", c_int32), ("grid_x", c_uint32), ("grid_y", c_uint32),
+        ("partials_bytes", c_uint64), ("partials_capacity", c_uint64),
+        ("num_tensors", c_int32), ("reserved", c_int32),
+        ("tensor", BnAuditTensor * 3),
+    ]
+
+
+class BnAuditReport(ctypes.Structure):
+    """struct h2x_bn_audit_report"""
+    _fields_ = [("num_launches", c_int32), ("reserved", c_int32), ("workspace_bytes", c_uint64),
+                ("launch", BnAuditLaunch * BN_AUDIT_MAX_LAUNCHES)]
+
+
 class ShuffleGeometry(ctypes.Structure):
     """struct h2x_shuffle_geometry"""
     _fields_ = [
@@ -121,6 +149,8 @@ SIGNATURES = {
                                          POINTER(TensorGeometry), POINTER(TensorGeometry), c_void_p,
                                          c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                          c_void_p, c_double, c_void_p]),
+    "h2x_bn_audit": (c_int, [c_int, c_int, c_int, POINTER(POINTER(TensorGeometry)), POINTER(c_uint64),
+                             POINTER(BnAuditReport)]),
     "h2x_tensor_transform": (c_int, [c_int, c_int, c_int, POINTER(POINTER(TensorGeometry)), POINTER(c_void_p),
                                      POINTER(c_double), c_void_p]),
     "h2x_tensor_reduce_sum_workspace_bytes": (c_size_t, [POINTER(TensorGeometry), POINTER(TensorGeometry)]),

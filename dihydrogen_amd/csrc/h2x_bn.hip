@@ -33,6 +33,8 @@
 // 10x slower than the whole stream).  All orders are fixed, so results are
 // deterministic; the reference's float atomics are not
 // (batchnorm.cu:127-131,1047-1053).
+#include "h2x_bn_maps.hpp"
+#include "h2x_bn_plan.hpp"
 #include "h2x_device.hpp"
 
 #include <algorithm>
@@ -50,6 +52,37 @@ namespace h2x
 {
 namespace
 {
+
+using namespace bn;
+
+// The log the calling thread has installed (h2x_bn_plan.hpp): launches are then
+// described instead of issued.
+thread_local LaunchLog* t_launch_log = nullptr;
+
+// Appends a planned launch to the installed log; false: no log, issue it.
+bool logged(const LaunchRecord& r)
+{
+    if (!t_launch_log)
+        return false;
+    t_launch_log->records.push_back(r);
+    return true;
+}
+
+// Status of the launches just issued (none while a log is installed).
+int issued()
+{
+    return t_launch_log ? static_cast<int>(H2X_SUCCESS) : launch_status();
+}
+
+// Installs a log for the lifetime of the object and puts the previous one back.
+struct ScopedLaunchLog
+{
+    explicit ScopedLaunchLog(LaunchLog* log) : before(t_launch_log) { t_launch_log = log; }
+    ~ScopedLaunchLog() { t_launch_log = before; }
+    ScopedLaunchLog(const ScopedLaunchLog&) = delete;
+    ScopedLaunchLog& operator=(const ScopedLaunchLog&) = delete;
+    LaunchLog* before;
+};
 
 // Device address of `scratch` on the current device, looked up once per device.
 constexpr int kMaxDevices = 64;
@@ -124,60 +157,6 @@ Chunking make_chunking(size_t spatial, size_t segments, size_t budget, size_t ti
     if (c.chunks_per_seg < 1)
         c.chunks_per_seg = 1;
     return c;
-}
-
-// Where the elements of one tensor live.  Element i of segment (n, c) is at
-// base[n*stride_n + c*stride_c + offset(i)]; offset(i) = i for the dense layout.
-// Strided layout (tensors with halos inside their segments, samples folded into
-// rows, dense tensors that vectors cannot address aligned): element by element,
-// i is the flat index over the interior extents, innermost first.  With vectors,
-// every row (the `width` contiguous interior elements) is padded to `spr`
-// vectors and i counts the elements of the padded rows: vector k of a row
-// starts at element min(k * VEC, width - VEC), so the last vector of a row that
-// is no multiple of VEC long overlaps the one before it instead of running into
-// the next row, and every vector is contiguous in every tensor of the launch.
-// The `skip` leading elements of such a vector belong to its neighbour:
-// reductions leave them out; elementwise kernels store them twice (the same
-// values) where the output shares no memory with an input, else one by one.
-struct TensorMap
-{
-    int64_t stride_n, stride_c;
-    FastDiv w, h;     // interior extents of spatial dimensions 0 and 1 (strided layout)
-    int64_t sy, sz;   // strides of spatial dimensions 1 and 2 (strided layout)
-    FastDiv spr;      // vectors a row is padded to (strided layout with vectors)
-    uint32_t width;   // elements of a row (strided layout with vectors)
-};
-
-template <bool STRIDED>
-__device__ __forceinline__ size_t seg_offset(const TensorMap& m, size_t i)
-{
-    if constexpr (!STRIDED)
-    {
-        return i;
-    }
-    else
-    {
-        const uint32_t t = fastdiv(static_cast<uint32_t>(i), m.w);
-        const uint32_t x = static_cast<uint32_t>(i) - t * m.w.divisor;
-        const uint32_t z = fastdiv(t, m.h);
-        const uint32_t y = t - z * m.h.divisor;
-        return x + y * static_cast<size_t>(m.sy) + z * static_cast<size_t>(m.sz);
-    }
-}
-
-// Offset of the vector at padded index i (a multiple of VEC) and the number of
-// its leading elements that the vector before it owns.
-template <int VEC>
-__device__ __forceinline__ size_t row_vector_offset(const TensorMap& m, size_t i, uint32_t* skip)
-{
-    const uint32_t slot = static_cast<uint32_t>(i) / VEC;
-    const uint32_t r = fastdiv(slot, m.spr);
-    const uint32_t x = (slot - r * m.spr.divisor) * VEC;
-    const uint32_t last = m.width - VEC;
-    *skip = x > last ? x - last : 0;
-    const uint32_t z = fastdiv(r, m.h);
-    const uint32_t y = r - z * m.h.divisor;
-    return (x > last ? last : x) + y * static_cast<size_t>(m.sy) + z * static_cast<size_t>(m.sz);
 }
 
 // ALIGNED: the address is a multiple of the vector size (dense layout); rows
@@ -762,94 +741,6 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop2_kernel(
 // channels and many samples would leave a reduction with too few workgroups,
 // the lanes of a workgroup form `rows` rows that take every rows-th sample of
 // a narrower window.
-struct ShortGeometry
-{
-    int num_samples, num_channels, spatial;
-    int row;                // elements that are contiguous in every tensor of the launch: the
-                            // whole segment, or a row of it when some tensor has halos inside
-    int slots_per_row;      // vectors a row is padded to
-    int slots;              // vectors a segment is padded to: its rows * slots_per_row
-    int rows_per_plane;     // rows in a plane of the segment (launches that go row by row)
-    int rows;               // rows of lanes, each on samples of its own
-    int channels_per_group; // whole channels one workgroup serves: kBlockSize / rows / slots
-    int samples_per_group;  // samples one workgroup walks through (blockIdx.y counts these ranges)
-};
-
-// One tensor of a short-segment launch: where sample n, channel c starts and
-// where the rows of its segment lie.
-struct ShortTensor
-{
-    int64_t stride_n, stride_c;
-    int h;          // rows per plane (interior extent of spatial dimension 1)
-    int64_t sy, sz; // strides of spatial dimensions 1 and 2
-};
-
-enum ShortTail : int
-{
-    kTailNone = 0,    // segments are whole vectors
-    kTailOverlap = 1, // the last vector of a segment overlaps the one before it
-    kTailScalar = 2   // segments shorter than a vector
-};
-
-struct ShortLane
-{
-    int row;    // row of lanes: its samples are row, row + rows, ... of the workgroup's range
-    int q;      // channel within the workgroup's window
-    int slot;   // slot of the channel's segment
-    int c;      // channel
-    int line;   // row of the segment the slot lies in
-    int first;  // first element of the slot's vector within its row
-    int valid;  // elements the slot owns; 0: an idle lane
-    int skip;   // leading elements of its vector that the slot before it owns (kTailOverlap)
-    bool heads; // first lane of its channel in its row
-    bool leads; // first lane of its channel in row 0
-};
-
-template <int VEC, int TAIL>
-__device__ __forceinline__ ShortLane short_lane(const ShortGeometry& g)
-{
-    ShortLane l;
-    const int lanes_per_row = kBlockSize / g.rows;
-    l.row = static_cast<int>(threadIdx.x) / lanes_per_row;
-    const int t = static_cast<int>(threadIdx.x) - l.row * lanes_per_row;
-    l.q = t / g.slots;
-    const int v = t - l.q * g.slots;
-    l.slot = v;
-    l.c = static_cast<int>(blockIdx.x) * g.channels_per_group + l.q;
-    l.line = v / g.slots_per_row;
-    const int k = v - l.line * g.slots_per_row;
-    const int left = g.row - k * VEC;
-    const bool active = l.q < g.channels_per_group && l.c < g.num_channels;
-    l.valid = active ? (left < VEC ? left : VEC) : 0;
-    l.skip = TAIL == kTailOverlap && active ? VEC - l.valid : 0;
-    l.first = k * VEC - l.skip;
-    l.heads = active && v == 0;
-    l.leads = l.heads && l.row == 0;
-    return l;
-}
-
-// Whether element j of the lane's vector is one the lane owns.
-template <int VEC, int TAIL>
-__device__ __forceinline__ bool slot_owns(const ShortLane& l, int j)
-{
-    if constexpr (TAIL == kTailNone)
-        return true;
-    else if constexpr (TAIL == kTailOverlap)
-        return j >= l.skip;
-    else
-        return j < l.valid;
-}
-
-// Where a lane's slot starts in one tensor, relative to the start of the
-// (sample, channel) segment.  The lane's place in the segment never changes, so
-// this is worked out once.
-__device__ __forceinline__ int slot_offset(const ShortLane& l, const ShortTensor& t)
-{
-    const int z = l.line / t.h;
-    const int y = l.line - z * t.h;
-    return static_cast<int>(l.first + y * t.sy + z * t.sz);
-}
-
 template <typename T, int VEC, int TAIL, bool STREAM = false>
 __device__ __forceinline__ void load_slot(const T* p, const ShortLane& l, T (&r)[VEC])
 {
@@ -1008,7 +899,7 @@ __global__ __launch_bounds__(kBlockSize) void bn_sums_short_kernel(
     const T* __restrict__ x, T* __restrict__ sums, T* __restrict__ sqsums, double* partials,
     const ShortTensor tx, const ShortGeometry g, bool always_partials)
 {
-    const ShortLane l = short_lane<VEC, TAIL>(g);
+    const ShortLane l = short_lane<VEC, TAIL>(g, static_cast<int>(threadIdx.x), static_cast<int>(blockIdx.x));
     double acc[2] = {0.0, 0.0};
     if (l.valid > 0)
     {
@@ -1060,7 +951,7 @@ __global__ __launch_bounds__(kBlockSize) void bn_apply_short_kernel(
     const T* __restrict__ scale, const T* __restrict__ bias, T* __restrict__ y, T epsilon,
     const ShortTensor tx, const ShortTensor ty, const ShortGeometry g, const FusedStats<T> fused)
 {
-    const ShortLane l = short_lane<VEC, TAIL>(g);
+    const ShortLane l = short_lane<VEC, TAIL>(g, static_cast<int>(threadIdx.x), static_cast<int>(blockIdx.x));
     T m = T(0), variance = T(0);
     if constexpr (FUSED)
     {
@@ -1139,7 +1030,7 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop1_short_kernel(
     double* partials, const ShortTensor tx, const ShortTensor td, const ShortGeometry g,
     bool always_partials)
 {
-    const ShortLane l = short_lane<VEC, TAIL>(g);
+    const ShortLane l = short_lane<VEC, TAIL>(g, static_cast<int>(threadIdx.x), static_cast<int>(blockIdx.x));
     double acc[4] = {0.0, 0.0, 0.0, 0.0};
     if (l.valid > 0)
     {
@@ -1209,7 +1100,7 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop2_short_kernel(
     T epsilon, size_t num_per_sum, const ShortTensor tx, const ShortTensor td,
     const ShortTensor to, const ShortGeometry g, bool disjoint, const FusedStats<T> fused)
 {
-    const ShortLane l = short_lane<VEC, TAIL>(g);
+    const ShortLane l = short_lane<VEC, TAIL>(g, static_cast<int>(threadIdx.x), static_cast<int>(blockIdx.x));
     T dmean_c = T(0), dvar_c = T(0);
     if constexpr (FUSED)
     {
@@ -1699,16 +1590,70 @@ int short_elementwise_groups(ShortGeometry* g, int unroll, size_t prologue_bytes
         }                                                                                          \
     } while (0)
 
+// ---- what a launch looks like to the log ----------------------------------------
+
+LaunchRecord short_record(int kernel, const ShortGeometry& sg, dim3 grid, int vec,
+                          std::initializer_list<const HostTensor*> ts, bool last_is_output)
+{
+    LaunchRecord r;
+    r.kernel = kernel;
+    r.family = kFamilyShort;
+    r.vec = vec;
+    r.tail = sg.row % vec == 0 ? kTailNone : sg.row > vec ? kTailOverlap : kTailScalar;
+    r.grid_x = grid.x;
+    r.grid_y = grid.y;
+    r.num_samples = sg.num_samples;
+    r.num_channels = sg.num_channels;
+    r.spatial = static_cast<size_t>(sg.spatial);
+    r.geometry = sg;
+    r.last_is_output = last_is_output;
+    for (const HostTensor* t : ts)
+        r.tensor[r.num_tensors++] = short_tensor(*t, sg);
+    return r;
+}
+
+LaunchRecord long_record(int kernel, bool strided, int vw, dim3 grid, int num_samples,
+                         int num_channels, size_t spatial, const Chunking& ch,
+                         std::initializer_list<const HostTensor*> ts, bool last_is_output)
+{
+    LaunchRecord r;
+    r.kernel = kernel;
+    r.family = strided ? kFamilyStrided : kFamilyDense;
+    r.vec = vw;
+    r.grid_x = grid.x;
+    r.grid_y = grid.y;
+    r.num_samples = num_samples;
+    r.num_channels = num_channels;
+    r.spatial = spatial;
+    r.chunk = ch.chunk;
+    r.chunks_per_seg = ch.chunks_per_seg;
+    r.last_is_output = last_is_output;
+    for (const HostTensor* t : ts)
+        r.map[r.num_tensors++] = t->map;
+    return r;
+}
+
+LaunchRecord small_record(int kernel, unsigned int grid_x, int num_channels, int num_sums = 0)
+{
+    LaunchRecord r;
+    r.kernel = kernel;
+    r.grid_x = grid_x;
+    r.num_channels = num_channels;
+    r.num_sums = num_sums;
+    return r;
+}
+
 template <typename T>
 int zero_outputs(std::initializer_list<void*> outs, int num_channels, hipStream_t stream)
 {
     const int blocks = (num_channels + kBlockSize - 1) / kBlockSize;
     for (void* p : outs)
-        fill_kernel<T><<<blocks, kBlockSize, 0, stream>>>(static_cast<T*>(p), num_channels, T(0));
-    return launch_status();
+        if (!logged(small_record(kKernelFill, blocks, num_channels)))
+            fill_kernel<T><<<blocks, kBlockSize, 0, stream>>>(static_cast<T*>(p), num_channels, T(0));
+    return issued();
 }
 
-// `groups_out` non-null: the caller finishes the reduction itself (a fused
+// `fused_out` non-null: the caller finishes the reduction itself (a fused
 // consumer kernel): every workgroup stores partials, no finishing launch.
 template <typename T>
 int sums_impl(int num_samples, int num_channels, size_t spatial, const HostTensor& tx_in,
@@ -1728,24 +1673,29 @@ int sums_impl(int num_samples, int num_channels, size_t spatial, const HostTenso
         const int groups = short_reduction_groups(&sg, gmax, kUnroll, sizeof(T));
         double* partials = static_cast<double*>(workspace);
         const dim3 grid(short_windows(sg), groups);
-        H2X_DISPATCH_SHORT(bn_sums_short_kernel, grid, static_cast<const T*>(x),
-                           static_cast<T*>(sums), static_cast<T*>(sqsums), partials,
-                           short_tensor(tx_in, sg), sg, fused_out != nullptr);
+        LaunchRecord rec = short_record(kKernelSums, sg, grid, full_vec<T>(), {&tx_in}, false);
+        rec.num_sums = 2;
+        rec.groups_max = gmax;
+        rec.partials = groups > 1 || fused_out != nullptr;
+        if (!logged(rec))
+            H2X_DISPATCH_SHORT(bn_sums_short_kernel, grid, static_cast<const T*>(x),
+                               static_cast<T*>(sums), static_cast<T*>(sqsums), partials,
+                               short_tensor(tx_in, sg), sg, fused_out != nullptr);
         if (fused_out)
         {
             fused_out->groups = groups;
             fused_out->sequential = true;
-            return launch_status();
+            return issued();
         }
-        if (groups > 1)
-            bn_finish_short_kernel<T, 2>
-                <<<(num_channels + kBlockSize - 1) / kBlockSize, kBlockSize, 0, stream>>>(
-                    partials, groups, num_channels, static_cast<T*>(sums),
-                    static_cast<T*>(sqsums), nullptr, nullptr);
-        return launch_status();
+        const unsigned int blocks = (num_channels + kBlockSize - 1) / kBlockSize;
+        if (groups > 1 && !logged(small_record(kKernelFinish, blocks, num_channels, 2)))
+            bn_finish_short_kernel<T, 2><<<blocks, kBlockSize, 0, stream>>>(
+                partials, groups, num_channels, static_cast<T*>(sums), static_cast<T*>(sqsums),
+                nullptr, nullptr);
+        return issued();
     }
     HostTensor tx = tx_in;
-    fold_samples(&num_samples, &spatial, {&tx});
+    const bool folded = fold_samples(&num_samples, &spatial, {&tx});
     if (spatial >= (1ull << 31) && tx.strided)
         return H2X_ERR_TOO_LARGE;
     bool strided;
@@ -1763,19 +1713,28 @@ int sums_impl(int num_samples, int num_channels, size_t spatial, const HostTenso
     const size_t groups = std::min<size_t>(units, gmax);
     double* partials = static_cast<double*>(workspace);
     const dim3 grid(static_cast<unsigned int>(groups), num_channels);
-    H2X_DISPATCH(bn_sums_kernel, grid, static_cast<const T*>(x), static_cast<T*>(sums),
-                 static_cast<T*>(sqsums), partials, tx.map, spatial, ch.chunk, ch.chunks_per_seg,
-                 static_cast<unsigned int>(units), gmax, fused_out != nullptr);
+    LaunchRecord rec = long_record(kKernelSums, strided, vw, grid, num_samples, num_channels,
+                                   spatial, ch, {&tx}, false);
+    rec.folded = folded;
+    rec.num_units = static_cast<unsigned int>(units);
+    rec.num_sums = 2;
+    rec.groups_max = gmax;
+    rec.partials = groups > 1 || fused_out != nullptr;
+    if (!logged(rec))
+        H2X_DISPATCH(bn_sums_kernel, grid, static_cast<const T*>(x), static_cast<T*>(sums),
+                     static_cast<T*>(sqsums), partials, tx.map, spatial, ch.chunk,
+                     ch.chunks_per_seg, static_cast<unsigned int>(units), gmax,
+                     fused_out != nullptr);
     if (fused_out != nullptr)
     {
         fused_out->groups = static_cast<int>(groups);
-        return launch_status();
+        return issued();
     }
-    if (groups > 1)
+    if (groups > 1 && !logged(small_record(kKernelFinish, num_channels, num_channels, 2)))
         bn_finish_kernel<T, 2><<<num_channels, kBlockSize, 0, stream>>>(
             partials, static_cast<int>(groups), gmax, static_cast<T*>(sums),
             static_cast<T*>(sqsums), nullptr, nullptr);
-    return launch_status();
+    return issued();
 }
 
 template <typename T>
@@ -1785,10 +1744,11 @@ int statistics_impl(int num_channels, size_t num_per_sum, double decay, void* me
     if (num_channels == 0)
         return H2X_SUCCESS;
     const int blocks = std::min((num_channels + kBlockSize - 1) / kBlockSize, 1024);
-    bn_statistics_kernel<T><<<blocks, kBlockSize, 0, stream>>>(
-        num_channels, num_per_sum, static_cast<T>(decay), static_cast<T*>(mean),
-        static_cast<T*>(var), static_cast<T*>(running_mean), static_cast<T*>(running_var));
-    return launch_status();
+    if (!logged(small_record(kKernelStatistics, blocks, num_channels)))
+        bn_statistics_kernel<T><<<blocks, kBlockSize, 0, stream>>>(
+            num_channels, num_per_sum, static_cast<T>(decay), static_cast<T*>(mean),
+            static_cast<T*>(var), static_cast<T*>(running_mean), static_cast<T*>(running_var));
+    return issued();
 }
 
 // Chunking of an elementwise pass over N*C segments: at least one full vector
@@ -1819,6 +1779,11 @@ int apply_impl(int num_samples, int num_channels, size_t spatial, const HostTens
                         short_elementwise_groups(&sg, kUnroll,
                                                  fused ? fused->groups * 2 * sizeof(double) : 0,
                                                  spatial * sizeof(T) * 2));
+        LaunchRecord rec =
+            short_record(kKernelApply, sg, grid, full_vec<T>(), {&tx_in, &ty_in}, true);
+        rec.fused = fused != nullptr;
+        if (logged(rec))
+            return H2X_SUCCESS;
         if (fused)
             H2X_DISPATCH_SHORT_FUSED(bn_apply_short_kernel, true, grid, static_cast<const T*>(x),
                                      nullptr, nullptr, static_cast<const T*>(scale),
@@ -1831,10 +1796,10 @@ int apply_impl(int num_samples, int num_channels, size_t spatial, const HostTens
                                      static_cast<const T*>(scale), static_cast<const T*>(bias),
                                      static_cast<T*>(y), static_cast<T>(epsilon),
                                      short_tensor(tx_in, sg), short_tensor(ty_in, sg), sg, FusedStats<T>());
-        return launch_status();
+        return issued();
     }
     HostTensor tx = tx_in, ty = ty_in;
-    fold_samples(&num_samples, &spatial, {&tx, &ty});
+    const bool folded = fold_samples(&num_samples, &spatial, {&tx, &ty});
     if (spatial >= (1ull << 31) && (tx.strided || ty.strided))
         return H2X_ERR_TOO_LARGE;
     const size_t segments = static_cast<size_t>(num_samples) * num_channels;
@@ -1849,6 +1814,12 @@ int apply_impl(int num_samples, int num_channels, size_t spatial, const HostTens
     if (!grid_ok(blocks))
         return H2X_ERR_TOO_LARGE;
     const unsigned int grid = static_cast<unsigned int>(blocks);
+    LaunchRecord rec = long_record(kKernelApply, strided, vw, dim3(grid), num_samples, num_channels,
+                                   spatial, ch, {&tx, &ty}, true);
+    rec.folded = folded;
+    rec.fused = fused != nullptr;
+    if (logged(rec))
+        return H2X_SUCCESS;
     if (fused)
         H2X_DISPATCH_FUSED(bn_apply_kernel, grid, static_cast<const T*>(x), nullptr, nullptr,
                            static_cast<const T*>(scale), static_cast<const T*>(bias),
@@ -1859,7 +1830,7 @@ int apply_impl(int num_samples, int num_channels, size_t spatial, const HostTens
                      static_cast<const T*>(var), static_cast<const T*>(scale),
                      static_cast<const T*>(bias), static_cast<T*>(y), static_cast<T>(epsilon),
                      num_channels, spatial, tx.map, ty.map, ch.chunk, ch.chunks_per_seg);
-    return launch_status();
+    return issued();
 }
 
 template <typename T>
@@ -1882,27 +1853,34 @@ int backprop1_impl(int num_samples, int num_channels, size_t spatial, const Host
         const int groups = short_reduction_groups(&sg, gmax, kUnroll / 2, sizeof(T));
         double* partials = static_cast<double*>(workspace);
         const dim3 grid(short_windows(sg), groups);
-        H2X_DISPATCH_SHORT(bn_backprop1_short_kernel, grid, static_cast<const T*>(x),
-                           static_cast<const T*>(dy), static_cast<const T*>(mean),
-                           static_cast<const T*>(var), static_cast<const T*>(scale),
-                           static_cast<T*>(dscale), static_cast<T*>(dbias), static_cast<T*>(dmean),
-                           static_cast<T*>(dvar), static_cast<T>(epsilon), partials,
-                           short_tensor(tx_in, sg), short_tensor(td_in, sg), sg, fused_out != nullptr);
+        LaunchRecord rec =
+            short_record(kKernelBackprop1, sg, grid, full_vec<T>(), {&tx_in, &td_in}, false);
+        rec.num_sums = 4;
+        rec.groups_max = gmax;
+        rec.partials = groups > 1 || fused_out != nullptr;
+        if (!logged(rec))
+            H2X_DISPATCH_SHORT(bn_backprop1_short_kernel, grid, static_cast<const T*>(x),
+                               static_cast<const T*>(dy), static_cast<const T*>(mean),
+                               static_cast<const T*>(var), static_cast<const T*>(scale),
+                               static_cast<T*>(dscale), static_cast<T*>(dbias),
+                               static_cast<T*>(dmean), static_cast<T*>(dvar),
+                               static_cast<T>(epsilon), partials, short_tensor(tx_in, sg),
+                               short_tensor(td_in, sg), sg, fused_out != nullptr);
         if (fused_out)
         {
             fused_out->groups = groups;
             fused_out->sequential = true;
-            return launch_status();
+            return issued();
         }
-        if (groups > 1)
-            bn_finish_short_kernel<T, 4>
-                <<<(num_channels + kBlockSize - 1) / kBlockSize, kBlockSize, 0, stream>>>(
-                    partials, groups, num_channels, static_cast<T*>(dscale),
-                    static_cast<T*>(dbias), static_cast<T*>(dmean), static_cast<T*>(dvar));
-        return launch_status();
+        const unsigned int blocks = (num_channels + kBlockSize - 1) / kBlockSize;
+        if (groups > 1 && !logged(small_record(kKernelFinish, blocks, num_channels, 4)))
+            bn_finish_short_kernel<T, 4><<<blocks, kBlockSize, 0, stream>>>(
+                partials, groups, num_channels, static_cast<T*>(dscale), static_cast<T*>(dbias),
+                static_cast<T*>(dmean), static_cast<T*>(dvar));
+        return issued();
     }
     HostTensor tx = tx_in, td = td_in;
-    fold_samples(&num_samples, &spatial, {&tx, &td});
+    const bool folded = fold_samples(&num_samples, &spatial, {&tx, &td});
     if (spatial >= (1ull << 31) && (tx.strided || td.strided))
         return H2X_ERR_TOO_LARGE;
     bool strided;
@@ -1920,22 +1898,31 @@ int backprop1_impl(int num_samples, int num_channels, size_t spatial, const Host
     const size_t groups = std::min<size_t>(units, gmax);
     double* partials = static_cast<double*>(workspace);
     const dim3 grid(static_cast<unsigned int>(groups), num_channels);
-    H2X_DISPATCH(bn_backprop1_kernel, grid, static_cast<const T*>(x), static_cast<const T*>(dy),
-                 static_cast<const T*>(mean), static_cast<const T*>(var),
-                 static_cast<const T*>(scale), static_cast<T*>(dscale), static_cast<T*>(dbias),
-                 static_cast<T*>(dmean), static_cast<T*>(dvar), static_cast<T>(epsilon), partials,
-                 spatial, tx.map, td.map, ch.chunk, ch.chunks_per_seg,
-                 static_cast<unsigned int>(units), gmax, fused_out != nullptr);
+    LaunchRecord rec = long_record(kKernelBackprop1, strided, vw, grid, num_samples, num_channels,
+                                   spatial, ch, {&tx, &td}, false);
+    rec.folded = folded;
+    rec.num_units = static_cast<unsigned int>(units);
+    rec.num_sums = 4;
+    rec.groups_max = gmax;
+    rec.partials = groups > 1 || fused_out != nullptr;
+    if (!logged(rec))
+        H2X_DISPATCH(bn_backprop1_kernel, grid, static_cast<const T*>(x),
+                     static_cast<const T*>(dy), static_cast<const T*>(mean),
+                     static_cast<const T*>(var), static_cast<const T*>(scale),
+                     static_cast<T*>(dscale), static_cast<T*>(dbias), static_cast<T*>(dmean),
+                     static_cast<T*>(dvar), static_cast<T>(epsilon), partials, spatial, tx.map,
+                     td.map, ch.chunk, ch.chunks_per_seg, static_cast<unsigned int>(units), gmax,
+                     fused_out != nullptr);
     if (fused_out != nullptr)
     {
         fused_out->groups = static_cast<int>(groups);
-        return launch_status();
+        return issued();
     }
-    if (groups > 1)
+    if (groups > 1 && !logged(small_record(kKernelFinish, num_channels, num_channels, 4)))
         bn_finish_kernel<T, 4><<<num_channels, kBlockSize, 0, stream>>>(
             partials, static_cast<int>(groups), gmax, static_cast<T*>(dscale),
             static_cast<T*>(dbias), static_cast<T*>(dmean), static_cast<T*>(dvar));
-    return launch_status();
+    return issued();
 }
 
 template <typename T>
@@ -1967,6 +1954,12 @@ int backprop2_impl(int num_samples, int num_channels, size_t spatial, size_t num
                         short_elementwise_groups(&sg, kUnroll / 2,
                                                  fused ? fused->groups * 4 * sizeof(double) : 0,
                                                  spatial * sizeof(T) * 3));
+        LaunchRecord rec = short_record(kKernelBackprop2, sg, grid, full_vec<T>(),
+                                        {&tx_in, &td_in, &to_in}, true);
+        rec.fused = fused != nullptr;
+        rec.rewrite = disjoint;
+        if (logged(rec))
+            return H2X_SUCCESS;
         if (fused)
             H2X_DISPATCH_SHORT_FUSED(bn_backprop2_short_kernel, true, grid,
                                      static_cast<const T*>(x), static_cast<const T*>(dy),
@@ -1984,10 +1977,10 @@ int backprop2_impl(int num_samples, int num_channels, size_t spatial, size_t num
                                      static_cast<T>(epsilon), num_per_sum, short_tensor(tx_in, sg),
                                      short_tensor(td_in, sg), short_tensor(to_in, sg), sg, disjoint,
                                      FusedStats<T>());
-        return launch_status();
+        return issued();
     }
     HostTensor tx = tx_in, td = td_in, to = to_in;
-    fold_samples(&num_samples, &spatial, {&tx, &td, &to});
+    const bool folded = fold_samples(&num_samples, &spatial, {&tx, &td, &to});
     if (spatial >= (1ull << 31) && (tx.strided || td.strided || to.strided))
         return H2X_ERR_TOO_LARGE;
     const size_t segments = static_cast<size_t>(num_samples) * num_channels;
@@ -2002,6 +1995,13 @@ int backprop2_impl(int num_samples, int num_channels, size_t spatial, size_t num
     if (!grid_ok(blocks))
         return H2X_ERR_TOO_LARGE;
     const unsigned int grid = static_cast<unsigned int>(blocks);
+    LaunchRecord rec = long_record(kKernelBackprop2, strided, vw, dim3(grid), num_samples,
+                                   num_channels, spatial, ch, {&tx, &td, &to}, true);
+    rec.folded = folded;
+    rec.fused = fused != nullptr;
+    rec.rewrite = disjoint;
+    if (logged(rec))
+        return H2X_SUCCESS;
     if (fused)
         H2X_DISPATCH_FUSED(bn_backprop2_kernel, grid, static_cast<const T*>(x),
                            static_cast<const T*>(dy), static_cast<const T*>(mean),
@@ -2016,7 +2016,7 @@ int backprop2_impl(int num_samples, int num_channels, size_t spatial, size_t num
                      static_cast<const T*>(dvar), static_cast<T*>(dx), static_cast<T>(epsilon),
                      num_per_sum, num_channels, spatial, tx.map, td.map, to.map, ch.chunk,
                      ch.chunks_per_seg, disjoint);
-    return launch_status();
+    return issued();
 }
 
 bool bad_geometry(int num_samples, int num_channels, size_t spatial, size_t real)
@@ -2143,6 +2143,17 @@ int forward_local(int n, int c, size_t s, size_t x_real, size_t y_real, const vo
     f.out[1] = static_cast<T*>(var);
     f.out[2] = static_cast<T*>(running_mean);
     f.out[3] = static_cast<T*>(running_var);
+    {
+        // both launches are planned before the first is issued: a call that is rejected writes nothing
+        LaunchLog plan;
+        ScopedLaunchLog scope(&plan);
+        FusedStats<T> g = f;
+        int err = sums_impl<T>(n, c, s, tx, x, nullptr, nullptr, ws, st, &g);
+        if (!err)
+            err = apply_impl<T>(n, c, s, tx, ty, x, nullptr, nullptr, scale, bias, y, eps, st, &g);
+        if (err)
+            return err;
+    }
     const int err = sums_impl<T>(n, c, s, tx, x, nullptr, nullptr, ws, st, &f);
     return err ? err : apply_impl<T>(n, c, s, tx, ty, x, nullptr, nullptr, scale, bias, y, eps, st, &f);
 }
@@ -2172,6 +2183,19 @@ int backward_local(int n, int c, size_t s, size_t x_real, size_t dy_real, size_t
     f.out[1] = static_cast<T*>(dbias);
     f.out[2] = static_cast<T*>(dmean);
     f.out[3] = static_cast<T*>(dvar);
+    {
+        // both launches are planned before the first is issued: a call that is rejected writes nothing
+        LaunchLog plan;
+        ScopedLaunchLog scope(&plan);
+        FusedStats<T> g = f;
+        int err = backprop1_impl<T>(n, c, s, tx, td, x, dy, mean, var, scale, nullptr, nullptr,
+                                    nullptr, nullptr, eps, ws, st, &g);
+        if (!err)
+            err = backprop2_impl<T>(n, c, s, num_per_sum, tx, td, to, x, dy, mean, var, scale,
+                                    nullptr, nullptr, dx, eps, st, &g);
+        if (err)
+            return err;
+    }
     const int err = backprop1_impl<T>(n, c, s, tx, td, x, dy, mean, var, scale, nullptr, nullptr,
                                       nullptr, nullptr, eps, ws, st, &f);
     return err ? err
@@ -2180,6 +2204,16 @@ int backward_local(int n, int c, size_t s, size_t x_real, size_t dy_real, size_t
 }
 
 } // namespace
+
+namespace bn
+{
+LaunchLog* install_launch_log(LaunchLog* log)
+{
+    LaunchLog* before = t_launch_log;
+    t_launch_log = log;
+    return before;
+}
+} // namespace bn
 } // namespace h2x
 
 using namespace h2x;

@@ -376,6 +376,78 @@ int h2x_bn_backprop2_strided(h2x_dtype dtype,
                              double epsilon,
                              h2x_stream_t stream);
 
+/**
+ * Launch audit, on the host: no GPU call is made and no pointer is followed.
+ * No counterpart in the reference, whose kernels check nothing of the kind;
+ * it exists so that the choice of kernels and their indexing can be verified
+ * on a machine without a GPU.  The entry point named by `stage` plans its
+ * launches for tensors of the given geometries (x; y or dy; dx - as many as
+ * the stage takes) at the given base addresses (only their alignment and
+ * whether x and dx share memory matter), and every workgroup and lane of
+ * every planned launch is then played on the CPU through the index maps the
+ * kernels use.  Per launch and tensor the report says how many elements are
+ * loaded and stored, how many of those accesses fall outside the interior
+ * elements of the tensor (`outside`: must be 0; halo cells and anything beyond
+ * the allocation count), how many interior elements no lane owns (`missed`:
+ * must be 0) and how many are owned by more than one (`owned_twice`: must be
+ * 0; a reduction would add them twice).  Owning an element means adding it
+ * into a sum or storing its result; elements that two overlapping vectors
+ * share are loaded, and where allowed stored, by both but owned by one.
+ * The two-launch stages take dense tensors only: geometries of three
+ * dimensions {spatial, channels, samples} with strides {1, real, real *
+ * channels}.  Returns what the entry point returns; H2X_ERR_TOO_LARGE if it
+ * plans more than H2X_BN_AUDIT_MAX_LAUNCHES launches.  Cost: proportional to
+ * the elements of the tensors; meant for tests.
+ */
+typedef enum h2x_bn_stage
+{
+    H2X_BN_STAGE_SUMS = 0,          /* h2x_bn_channel_sums_and_sqsums_strided */
+    H2X_BN_STAGE_NORMALIZE = 1,     /* h2x_bn_batch_normalization_strided */
+    H2X_BN_STAGE_BACKPROP1 = 2,     /* h2x_bn_backprop1_strided */
+    H2X_BN_STAGE_BACKPROP2 = 3,     /* h2x_bn_backprop2_strided */
+    H2X_BN_STAGE_FORWARD_LOCAL = 4, /* h2x_bn_forward_local */
+    H2X_BN_STAGE_BACKWARD_LOCAL = 5 /* h2x_bn_backward_local */
+} h2x_bn_stage;
+
+#define H2X_BN_AUDIT_MAX_LAUNCHES 8
+
+typedef struct h2x_bn_audit_tensor
+{
+    uint64_t loads, stores; /* elements */
+    uint64_t outside, missed, owned_twice;
+} h2x_bn_audit_tensor;
+
+typedef struct h2x_bn_audit_launch
+{
+    int32_t kernel; /* 0 sums, 1 normalise, 2 backprop1, 3 backprop2, 4 finish, 5 statistics, 6 fill */
+    int32_t family; /* 0 dense, 1 strided (padded rows, folded samples), 2 short segments */
+    int32_t vector_width; /* elements per access */
+    int32_t tail;         /* short family: 0 whole vectors, 1 overlapping last vector, 2 element by element */
+    int32_t folded;       /* samples folded into the rows of one segment */
+    int32_t fused;        /* finishes the preceding reduction itself */
+    uint32_t grid_x, grid_y;
+    uint64_t partials_bytes;    /* reductions: bytes of partial sums the launch can write in the workspace */
+    uint64_t partials_capacity; /* reductions: bytes the library reserves for them */
+    int32_t num_tensors;
+    int32_t reserved;
+    h2x_bn_audit_tensor tensor[3];
+} h2x_bn_audit_launch;
+
+typedef struct h2x_bn_audit_report
+{
+    int32_t num_launches;
+    int32_t reserved;
+    uint64_t workspace_bytes; /* h2x_bn_workspace_bytes of the channel count */
+    h2x_bn_audit_launch launch[H2X_BN_AUDIT_MAX_LAUNCHES];
+} h2x_bn_audit_report;
+
+int h2x_bn_audit(h2x_bn_stage stage,
+                 h2x_dtype dtype,
+                 int num_samples,
+                 const h2x_tensor_geometry* const* geometry,
+                 const uint64_t* address,
+                 h2x_bn_audit_report* report);
+
 /* ------------------------------------------------------------------------ */
 /* Elementwise transforms and sums over dimensions                           */
 /* ------------------------------------------------------------------------ */
