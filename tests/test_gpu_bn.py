@@ -202,6 +202,75 @@ def test_backprop2_in_place(shape, oracle_mod):
     assert max_rel(xin.real_view().cpu().numpy(), dx_o) <= TOL
 
 
+@pytest.mark.parametrize("fuse", [True, False])
+@pytest.mark.parametrize("shape", [(3, 5, 57, 57), (2, 3, 1027, 1031), (4, 6, 19, 19), (2, 4, 9, 11, 13)])
+def test_backprop2_in_place_on_segments_that_end_in_an_overlapping_vector(shape, fuse, oracle_mod):
+    """Dense segments that are no multiple of the vector long go through the padded-row
+    kernels, whose last vector of a row overlaps the one before it; with dx == x the
+    shared elements must be stored by their owner only.  Both the two-launch
+    backward() and the staged calls."""
+    import torch
+    from dihydrogen_amd.tensor import Distribution, LocaleVirtual, Tensor
+
+    x, dy, scale, bias = bn_inputs(shape, seed=17)
+    bn, xin, yout, mean, var, rm, rv = _run_forward(x, scale, bias)
+    bn.fuse_local = fuse
+    dist = Distribution.make_localized_distribution(len(shape))
+    dyt = Tensor(list(shape[::-1]), LocaleVirtual(0, 1), dist).allocate()
+    dyt.real_view().copy_(torch.from_numpy(dy))
+    outs = [torch.empty(shape[1], device="cuda") for _ in range(4)]
+    sc = torch.from_numpy(scale).cuda()
+    assert bn.backward(xin, dyt, mean, var, sc, *outs, xin) == 0  # d_input aliases input
+    torch.cuda.synchronize()
+    dx_o, dscale_o, dbias_o, dmean_o, dvar_o = oracle_mod.bn_backward(
+        x, dy, mean.cpu().numpy(), var.cpu().numpy(), scale, 1e-5)
+    assert max_rel(xin.real_view().cpu().numpy(), dx_o) <= TOL
+    for got, want in zip(outs, (dscale_o, dbias_o, dmean_o, dvar_o)):
+        assert max_rel(got.cpu().numpy(), want) <= TOL
+
+
+@pytest.mark.parametrize("case", [
+    ((134, 6, 3, 2), (2, 2, 1, 1), (1, 1, 0, 0)),          # haloed rows of 67 elements
+    ((130, 4, 6, 2, 2), (2, 1, 2, 1, 1), (2, 0, 1, 0, 0)),  # 5-D, rows of 65
+    ((14, 14, 70, 5), (2, 2, 1, 1), (1, 1, 0, 0)),          # 7 x 7 tiles in 9 x 9: short-segment kernels
+    ((18, 10, 14, 3, 2), (2, 2, 2, 1, 1), (1, 1, 1, 0, 0)),  # 9 x 5 x 7 tiles in 11 x 7 x 9
+])
+def test_backprop2_in_place_on_haloed_tensors(case, oracle_mod):
+    """dx == x on every rank of a decomposition whose local parts carry halos: interior
+    equal to the oracle's, halo cells untouched (they keep the input's halo values)."""
+    import torch
+    from dihydrogen_amd.layers import BatchNormalization
+    from dihydrogen_amd.tensor import Distribution, LocaleVirtual, Tensor
+    gshape, locale, overlap = case
+    nd = len(gshape)
+    nranks = int(np.prod(locale))
+    dist = Distribution.make_overlapped_distribution(locale, overlap)
+    c = gshape[nd - 2]
+    rng = np.random.default_rng(23)
+    scale = rng.uniform(0.5, 1.5, c).astype(np.float32)
+    bias = (0.1 * rng.standard_normal(c)).astype(np.float32)
+    for r in range(nranks):
+        loc = LocaleVirtual(r, nranks)
+        x, y, dy = (Tensor(gshape, loc, dist).allocate() for _ in range(3))
+        for t in (x, y, dy):
+            t.real_view().fill_(float("nan"))
+        xi = rng.standard_normal(x.local_shape[::-1]).astype(np.float32)
+        di = rng.standard_normal(x.local_shape[::-1]).astype(np.float32)
+        x.interior_view().copy_(torch.from_numpy(xi))
+        dy.interior_view().copy_(torch.from_numpy(di))
+        dev = lambda a: torch.from_numpy(a.copy()).cuda()
+        mean, var = torch.empty(c, device="cuda"), torch.empty(c, device="cuda")
+        rm, rv = torch.zeros(c, device="cuda"), torch.ones(c, device="cuda")
+        grads = [torch.empty(c, device="cuda") for _ in range(4)]
+        bn = BatchNormalization(nd, 0.9, 1e-5)
+        assert bn.forward(x, mean, var, rm, rv, dev(scale), dev(bias), y, True) == 0
+        assert bn.backward(x, dy, mean, var, dev(scale), *grads, x) == 0  # d_input aliases input
+        torch.cuda.synchronize()
+        dx_o = oracle_mod.bn_backward(xi, di, mean.cpu().numpy(), var.cpu().numpy(), scale)[0]
+        assert max_rel(x.interior_view().cpu().numpy(), dx_o) <= TOL
+        assert int(torch.isnan(x.real_view()).sum()) == x.get_local_real_size() - x.get_local_size()
+
+
 def test_inference_uses_running_statistics(oracle_mod):
     import torch
     shape = (2, 4, 6, 6)
