@@ -202,49 +202,68 @@ __device__ __forceinline__ void store_vec(T* p, const T (&r)[VEC])
     }
 }
 
-// The VEC elements at index i; returns how many of the leading ones belong to
-// the vector before (strided layout with vectors, else 0).
-template <typename T, int VEC, bool STRIDED, bool STREAM = false>
-__device__ __forceinline__ uint32_t load_at(const T* p, const TensorMap& m, size_t i, T (&r)[VEC])
+// How a kernel walks a tensor: as it lies (dense) or row by row in vectors
+// that start on any element (rows; see Place in h2x_bn_maps.hpp).
+enum Layout : int
 {
-    if constexpr (!STRIDED || VEC == 1)
+    kLayoutDense = 0,
+    kLayoutRows = 1
+};
+
+// Where the vector at index i lies.  Worked out once per vector, from the map
+// of one tensor of the launch, and shared by all of them (index splitting costs
+// two multiply-high divisions; done per tensor it was a third of the
+// instructions of the strided kernels).  Without vectors or index splitting
+// the place is not used.
+template <typename T, int VEC, int LAYOUT>
+__device__ __forceinline__ Place place_at(const TensorMap& m, size_t i)
+{
+    Place pl{0, 0, 0, 0};
+    if constexpr (VEC > 1 && LAYOUT == kLayoutRows)
+        place_vector<VEC>(m, row_split<VEC>(m, i, &pl), &pl);
+    return pl;
+}
+
+// The VEC elements of tensor p at index i / place pl.
+template <typename T, int VEC, int LAYOUT, bool STREAM = false>
+__device__ __forceinline__ void load_in(const T* p, const TensorMap& m, size_t i, const Place& pl,
+                                        T (&r)[VEC])
+{
+    if constexpr (VEC == 1 || LAYOUT == kLayoutDense)
     {
-        load_vec<T, VEC, !STRIDED, STREAM>(p + seg_offset<STRIDED>(m, i), r);
-        return 0;
+        load_vec<T, VEC, LAYOUT == kLayoutDense, STREAM>(
+            p + seg_offset<LAYOUT != kLayoutDense>(m, i), r);
     }
     else
     {
-        uint32_t skip;
-        const size_t off = row_vector_offset<VEC>(m, i, &skip);
-        load_vec<T, VEC, false, STREAM>(p + off, r);
-        return skip;
+        load_vec<T, VEC, false, STREAM>(p + (row_offset(m, pl) + pl.first), r);
     }
 }
 
-// rewrite: the elements a vector shares with the one before it may be stored
-// by both (the output shares no memory with the inputs they were made from).
-template <typename T, int VEC, bool STRIDED>
-__device__ __forceinline__ void store_at(T* p, const TensorMap& m, size_t i, const T (&r)[VEC],
-                                         bool rewrite)
+// rewrite (rows layout): the elements a vector shares with the one before it
+// may be stored by both (the output shares no memory with the inputs they were
+// made from).
+template <typename T, int VEC, int LAYOUT>
+__device__ __forceinline__ void store_out(T* p, const TensorMap& m, size_t i, const Place& pl,
+                                          const T (&r)[VEC], bool rewrite)
 {
-    if constexpr (!STRIDED || VEC == 1)
+    if constexpr (VEC == 1 || LAYOUT == kLayoutDense)
     {
-        store_vec<T, VEC, !STRIDED>(p + seg_offset<STRIDED>(m, i), r);
+        store_vec<T, VEC, LAYOUT == kLayoutDense>(p + seg_offset<LAYOUT != kLayoutDense>(m, i), r);
     }
     else
     {
-        uint32_t skip;
-        const size_t off = row_vector_offset<VEC>(m, i, &skip);
-        if (skip == 0 || rewrite)
+        T* q = p + (row_offset(m, pl) + pl.first);
+        if (pl.skip == 0 || rewrite)
         {
-            store_vec<T, VEC, false>(p + off, r);
+            store_vec<T, VEC, false>(q, r);
         }
         else
         {
 #pragma unroll
             for (int j = 1; j < VEC; ++j)
-                if (j >= static_cast<int>(skip))
-                    __builtin_nontemporal_store(r[j], p + off + j);
+                if (j >= static_cast<int>(pl.skip))
+                    __builtin_nontemporal_store(r[j], q + j);
         }
     }
 }
@@ -361,6 +380,7 @@ __global__ __launch_bounds__(kBlockSize) void bn_sums_kernel(
     int groups_per_channel_max, bool always_partials)
 {
     const int c = blockIdx.y;
+    constexpr int LAYOUT = STRIDED ? kLayoutRows : kLayoutDense;
     constexpr size_t kStride = static_cast<size_t>(kBlockSize) * VEC;
     constexpr size_t kTile = kStride * kUnroll;
     double acc[2] = {0.0, 0.0};
@@ -389,7 +409,12 @@ __global__ __launch_bounds__(kBlockSize) void bn_sums_kernel(
             uint32_t skip[kUnroll];
 #pragma unroll
             for (int u = 0; u < kUnroll; ++u)
-                skip[u] = load_at<T, VEC, STRIDED>(p, mx, tile + u * kStride + threadIdx.x * VEC, v[u]);
+            {
+                const size_t i = tile + u * kStride + threadIdx.x * VEC;
+                const Place pl = place_at<T, VEC, LAYOUT>(mx, i);
+                load_in<T, VEC, LAYOUT>(p, mx, i, pl, v[u]);
+                skip[u] = pl.skip;
+            }
 #pragma unroll
             for (int u = 0; u < kUnroll; ++u)
 #pragma unroll
@@ -400,10 +425,11 @@ __global__ __launch_bounds__(kBlockSize) void bn_sums_kernel(
         for (size_t i = tile + threadIdx.x * VEC; i + VEC <= end; i += kStride)
         {
             T v[VEC];
-            const uint32_t skip = load_at<T, VEC, STRIDED>(p, mx, i, v);
+            const Place pl = place_at<T, VEC, LAYOUT>(mx, i);
+            load_in<T, VEC, LAYOUT>(p, mx, i, pl, v);
 #pragma unroll
             for (int j = 0; j < VEC; ++j)
-                if (j >= static_cast<int>(skip))
+                if (j >= static_cast<int>(pl.skip))
                     accumulate(v[j]);
         }
     }
@@ -469,7 +495,7 @@ struct FusedStats
 // Replaces batch_normalization_opt_kernel, batchnorm.cu:420-455.  FUSED: mean
 // and variance are not read but made from the partial sums of bn_sums_kernel
 // (bn_finish_kernel + bn_statistics_kernel folded in).
-template <typename T, int VEC, bool STRIDED, bool FUSED = false>
+template <typename T, int VEC, int LAYOUT, bool FUSED = false>
 __global__ __launch_bounds__(kBlockSize) void bn_apply_kernel(
     const T* __restrict__ x, const T* __restrict__ mean, const T* __restrict__ var,
     const T* __restrict__ scale, const T* __restrict__ bias, T* __restrict__ y, T epsilon,
@@ -515,26 +541,32 @@ __global__ __launch_bounds__(kBlockSize) void bn_apply_kernel(
     for (; tile + kTile <= end; tile += kTile)
     {
         T v[kUnroll][VEC];
+        Place pl[kUnroll];
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u)
-            load_at<T, VEC, STRIDED>(xp, mx, tile + u * kStride + threadIdx.x * VEC, v[u]);
+        {
+            const size_t i = tile + u * kStride + threadIdx.x * VEC;
+            pl[u] = place_at<T, VEC, LAYOUT>(my, i);
+            load_in<T, VEC, LAYOUT>(xp, mx, i, pl[u], v[u]);
+        }
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u)
         {
 #pragma unroll
             for (int j = 0; j < VEC; ++j)
                 v[u][j] = fma_t((v[u][j] - m) * inv_stdev, sc, bi);
-            store_at<T, VEC, STRIDED>(yp, my, tile + u * kStride + threadIdx.x * VEC, v[u], true);
+            store_out<T, VEC, LAYOUT>(yp, my, tile + u * kStride + threadIdx.x * VEC, pl[u], v[u], true);
         }
     }
     for (size_t i = tile + threadIdx.x * VEC; i + VEC <= end; i += kStride)
     {
         T v[VEC];
-        load_at<T, VEC, STRIDED>(xp, mx, i, v);
+        const Place pl = place_at<T, VEC, LAYOUT>(my, i);
+        load_in<T, VEC, LAYOUT>(xp, mx, i, pl, v);
 #pragma unroll
         for (int j = 0; j < VEC; ++j)
             v[j] = fma_t((v[j] - m) * inv_stdev, sc, bi);
-        store_at<T, VEC, STRIDED>(yp, my, i, v, true);
+        store_out<T, VEC, LAYOUT>(yp, my, i, pl, v, true);
     }
 }
 
@@ -556,6 +588,7 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop1_kernel(
     const double neg_inv = -static_cast<double>(inv_stdev);
     const double neg_fac = -static_cast<double>(dvar_factor);
 
+    constexpr int LAYOUT = STRIDED ? kLayoutRows : kLayoutDense;
     constexpr size_t kStride = static_cast<size_t>(kBlockSize) * VEC;
     constexpr int kUnroll2 = kUnroll / 2; // two streams: same bytes in flight
     constexpr size_t kTile = kStride * kUnroll2;
@@ -590,8 +623,10 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop1_kernel(
             for (int u = 0; u < kUnroll2; ++u)
             {
                 const size_t i = tile + u * kStride + threadIdx.x * VEC;
-                skip[u] = load_at<T, VEC, STRIDED>(xp, mx, i, xv[u]);
-                load_at<T, VEC, STRIDED, true>(dp, md, i, dv[u]);
+                const Place pl = place_at<T, VEC, LAYOUT>(mx, i);
+                load_in<T, VEC, LAYOUT>(xp, mx, i, pl, xv[u]);
+                load_in<T, VEC, LAYOUT, true>(dp, md, i, pl, dv[u]);
+                skip[u] = pl.skip;
             }
 #pragma unroll
             for (int u = 0; u < kUnroll2; ++u)
@@ -603,11 +638,12 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop1_kernel(
         for (size_t i = tile + threadIdx.x * VEC; i + VEC <= end; i += kStride)
         {
             T xv[VEC], dv[VEC];
-            const uint32_t skip = load_at<T, VEC, STRIDED>(xp, mx, i, xv);
-            load_at<T, VEC, STRIDED, true>(dp, md, i, dv);
+            const Place pl = place_at<T, VEC, LAYOUT>(mx, i);
+            load_in<T, VEC, LAYOUT>(xp, mx, i, pl, xv);
+            load_in<T, VEC, LAYOUT, true>(dp, md, i, pl, dv);
 #pragma unroll
             for (int j = 0; j < VEC; ++j)
-                if (j >= static_cast<int>(skip))
+                if (j >= static_cast<int>(pl.skip))
                     accumulate(xv[j], dv[j]);
         }
     }
@@ -625,7 +661,7 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop1_kernel(
 // Replaces backprop2_opt_kernel, batchnorm.cu:1371-1418.  x and dx may alias:
 // each thread reads its elements before it writes them, so neither is
 // restrict-qualified (`disjoint`: they share no memory).
-template <typename T, int VEC, bool STRIDED, bool FUSED = false>
+template <typename T, int VEC, int LAYOUT, bool FUSED = false>
 __global__ __launch_bounds__(kBlockSize) void bn_backprop2_kernel(
     const T* x, const T* __restrict__ dy, const T* __restrict__ mean,
     const T* __restrict__ var, const T* __restrict__ scale, const T* __restrict__ dmean,
@@ -677,12 +713,14 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop2_kernel(
     for (; tile + kTile <= end; tile += kTile)
     {
         T xv[kUnroll2][VEC], dv[kUnroll2][VEC];
+        Place pl[kUnroll2];
 #pragma unroll
         for (int u = 0; u < kUnroll2; ++u)
         {
             const size_t i = tile + u * kStride + threadIdx.x * VEC;
-            load_at<T, VEC, STRIDED>(xp, mx, i, xv[u]);
-            load_at<T, VEC, STRIDED, true>(dp, md, i, dv[u]);
+            pl[u] = place_at<T, VEC, LAYOUT>(mo, i);
+            load_in<T, VEC, LAYOUT>(xp, mx, i, pl[u], xv[u]);
+            load_in<T, VEC, LAYOUT, true>(dp, md, i, pl[u], dv[u]);
         }
 #pragma unroll
         for (int u = 0; u < kUnroll2; ++u)
@@ -693,21 +731,22 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop2_kernel(
                 T r = fma_t(dv[u][j] * sc, inv_stdev, dmean_term);
                 xv[u][j] = fma_t(xv[u][j] - m, dvar_term, r);
             }
-            store_at<T, VEC, STRIDED>(op, mo, tile + u * kStride + threadIdx.x * VEC, xv[u], disjoint);
+            store_out<T, VEC, LAYOUT>(op, mo, tile + u * kStride + threadIdx.x * VEC, pl[u], xv[u], disjoint);
         }
     }
     for (size_t i = tile + threadIdx.x * VEC; i + VEC <= end; i += kStride)
     {
         T xv[VEC], dv[VEC];
-        load_at<T, VEC, STRIDED>(xp, mx, i, xv);
-        load_at<T, VEC, STRIDED, true>(dp, md, i, dv);
+        const Place pl = place_at<T, VEC, LAYOUT>(mo, i);
+        load_in<T, VEC, LAYOUT>(xp, mx, i, pl, xv);
+        load_in<T, VEC, LAYOUT, true>(dp, md, i, pl, dv);
 #pragma unroll
         for (int j = 0; j < VEC; ++j)
         {
             T r = fma_t(dv[j] * sc, inv_stdev, dmean_term);
             xv[j] = fma_t(xv[j] - m, dvar_term, r);
         }
-        store_at<T, VEC, STRIDED>(op, mo, i, xv, disjoint);
+        store_out<T, VEC, LAYOUT>(op, mo, i, pl, xv, disjoint);
     }
 }
 
@@ -1276,8 +1315,10 @@ int strided_tensor(const h2x_tensor_geometry* g, const void* p, int num_samples,
         t.row = static_cast<size_t>(g->local_shape[0]);
         t.map.w = make_fastdiv(static_cast<uint32_t>(g->local_shape[0]));
         t.map.h = make_fastdiv(ns > 1 ? static_cast<uint32_t>(g->local_shape[1]) : 1u);
-        t.map.sy = ns > 1 ? g->strides[1] : 0;
-        t.map.sz = ns > 2 ? g->strides[2] : 0;
+        if ((ns > 1 && g->strides[1] > 0xffffffffll) || (ns > 2 && g->strides[2] > 0xffffffffll))
+            return H2X_ERR_TOO_LARGE; // strides inside a segment are kept as 32-bit integers
+        t.map.sy = ns > 1 ? static_cast<uint32_t>(g->strides[1]) : 0;
+        t.map.sz = ns > 2 ? static_cast<uint32_t>(g->strides[2]) : 0;
         t.map.spr = make_fastdiv(1);
         t.map.width = 0;
         t.aligned = false;
@@ -1347,8 +1388,8 @@ size_t pad_rows(std::initializer_list<HostTensor*> ts, size_t spatial)
         if (!t->strided)
         {
             t->map.h = make_fastdiv(rows_per_plane);
-            t->map.sy = static_cast<int64_t>(width);
-            t->map.sz = static_cast<int64_t>(width) * rows_per_plane;
+            t->map.sy = static_cast<uint32_t>(width);
+            t->map.sz = static_cast<uint32_t>(width * rows_per_plane); // below 2^31: a segment's elements
         }
         t->map.spr = make_fastdiv(static_cast<uint32_t>(spr));
         t->map.width = static_cast<uint32_t>(width);
@@ -1373,15 +1414,15 @@ bool fold_samples(int* num_samples, size_t* spatial, std::initializer_list<HostT
     if (*num_samples <= 1 || *spatial >= kFoldBelow)
         return false;
     for (const HostTensor* t : ts)
-        if (t->strided)
-            return false; // rows are already split
+        if (t->strided || t->map.stride_n > 0xffffffffll)
+            return false; // rows are already split, or lie further apart than a 32-bit stride
     for (HostTensor* t : ts)
     {
         t->strided = true;
         t->row = *spatial;
         t->map.w = make_fastdiv(static_cast<uint32_t>(*spatial));
         t->map.h = make_fastdiv(static_cast<uint32_t>(*num_samples));
-        t->map.sy = t->map.stride_n;
+        t->map.sy = static_cast<uint32_t>(t->map.stride_n);
         t->map.sz = 0;
         t->aligned = false;
     }
@@ -1570,24 +1611,20 @@ int short_elementwise_groups(ShortGeometry* g, int unroll, size_t prologue_bytes
         }                                                                                          \
     } while (0)
 
-// The same for the variants that finish the preceding reduction themselves.
-#define H2X_DISPATCH_FUSED(KERNEL, GRID, ...)                                                      \
+// Launches an elementwise kernel<T, V, LAYOUT, FUSED>.
+#define H2X_DISPATCH_ELEMENTWISE(KERNEL, FUSED, GRID, ...)                                         \
     do                                                                                             \
     {                                                                                              \
-        if (strided)                                                                               \
-        {                                                                                          \
-            if (vw > 1)                                                                            \
-                KERNEL<T, full_vec<T>(), true, true><<<GRID, kBlockSize, 0, stream>>>(__VA_ARGS__); \
-            else                                                                                   \
-                KERNEL<T, 1, true, true><<<GRID, kBlockSize, 0, stream>>>(__VA_ARGS__);            \
-        }                                                                                          \
+        if (vw > 1 && strided)                                                                     \
+            KERNEL<T, full_vec<T>(), kLayoutRows, FUSED>                                           \
+                <<<GRID, kBlockSize, 0, stream>>>(__VA_ARGS__);                                    \
+        else if (vw > 1)                                                                           \
+            KERNEL<T, full_vec<T>(), kLayoutDense, FUSED>                                          \
+                <<<GRID, kBlockSize, 0, stream>>>(__VA_ARGS__);                                    \
+        else if (strided)                                                                          \
+            KERNEL<T, 1, kLayoutRows, FUSED><<<GRID, kBlockSize, 0, stream>>>(__VA_ARGS__);        \
         else                                                                                       \
-        {                                                                                          \
-            if (vw > 1)                                                                            \
-                KERNEL<T, full_vec<T>(), false, true><<<GRID, kBlockSize, 0, stream>>>(__VA_ARGS__); \
-            else                                                                                   \
-                KERNEL<T, 1, false, true><<<GRID, kBlockSize, 0, stream>>>(__VA_ARGS__);           \
-        }                                                                                          \
+            KERNEL<T, 1, kLayoutDense, FUSED><<<GRID, kBlockSize, 0, stream>>>(__VA_ARGS__);       \
     } while (0)
 
 // ---- what a launch looks like to the log ----------------------------------------
@@ -1757,8 +1794,17 @@ Chunking elementwise_chunking(size_t spatial, size_t segments, int vw, int unrol
 {
     const size_t tile = static_cast<size_t>(kBlockSize) * vw * unroll;
     const size_t one_pass = static_cast<size_t>(kBlockSize) * vw;
-    return make_chunking(spatial, segments, kElementwiseBlocks, one_pass,
-                         one_pass * 2 > tile ? one_pass : one_pass * 2);
+    Chunking c = make_chunking(spatial, segments, kElementwiseBlocks, one_pass,
+                               one_pass * 2 > tile ? one_pass : one_pass * 2);
+    // A chunk of more than a tile is cut down to whole tiles: the passes beyond the
+    // last whole tile run with one load in flight per lane instead of `unroll`
+    // (5 passes as 4 + 1 took a quarter longer than 4 on the haloed C3 shard).
+    if (c.chunk > tile && c.chunk % tile != 0)
+    {
+        c.chunk = c.chunk / tile * tile;
+        c.chunks_per_seg = static_cast<int>((spatial + c.chunk - 1) / c.chunk);
+    }
+    return c;
 }
 
 template <typename T>
@@ -1810,10 +1856,10 @@ int apply_impl(int num_samples, int num_channels, size_t spatial, const HostTens
     if (spatial >= (1ull << 31) && strided)
         return H2X_ERR_TOO_LARGE;
     const Chunking ch = elementwise_chunking(spatial, segments, vw, kUnroll);
-    const size_t blocks = segments * ch.chunks_per_seg;
-    if (!grid_ok(blocks))
+    const size_t workgroups = segments * ch.chunks_per_seg;
+    if (!grid_ok(workgroups))
         return H2X_ERR_TOO_LARGE;
-    const unsigned int grid = static_cast<unsigned int>(blocks);
+    const unsigned int grid = static_cast<unsigned int>(workgroups);
     LaunchRecord rec = long_record(kKernelApply, strided, vw, dim3(grid), num_samples, num_channels,
                                    spatial, ch, {&tx, &ty}, true);
     rec.folded = folded;
@@ -1821,15 +1867,16 @@ int apply_impl(int num_samples, int num_channels, size_t spatial, const HostTens
     if (logged(rec))
         return H2X_SUCCESS;
     if (fused)
-        H2X_DISPATCH_FUSED(bn_apply_kernel, grid, static_cast<const T*>(x), nullptr, nullptr,
-                           static_cast<const T*>(scale), static_cast<const T*>(bias),
-                           static_cast<T*>(y), static_cast<T>(epsilon), num_channels, spatial,
-                           tx.map, ty.map, ch.chunk, ch.chunks_per_seg, *fused);
+        H2X_DISPATCH_ELEMENTWISE(bn_apply_kernel, true, grid, static_cast<const T*>(x), nullptr,
+                                 nullptr, static_cast<const T*>(scale), static_cast<const T*>(bias),
+                                 static_cast<T*>(y), static_cast<T>(epsilon), num_channels, spatial,
+                                 tx.map, ty.map, ch.chunk, ch.chunks_per_seg, *fused);
     else
-        H2X_DISPATCH(bn_apply_kernel, grid, static_cast<const T*>(x), static_cast<const T*>(mean),
-                     static_cast<const T*>(var), static_cast<const T*>(scale),
-                     static_cast<const T*>(bias), static_cast<T*>(y), static_cast<T>(epsilon),
-                     num_channels, spatial, tx.map, ty.map, ch.chunk, ch.chunks_per_seg);
+        H2X_DISPATCH_ELEMENTWISE(bn_apply_kernel, false, grid, static_cast<const T*>(x),
+                                 static_cast<const T*>(mean), static_cast<const T*>(var),
+                                 static_cast<const T*>(scale), static_cast<const T*>(bias),
+                                 static_cast<T*>(y), static_cast<T>(epsilon), num_channels, spatial,
+                                 tx.map, ty.map, ch.chunk, ch.chunks_per_seg);
     return issued();
 }
 
@@ -1991,10 +2038,10 @@ int backprop2_impl(int num_samples, int num_channels, size_t spatial, size_t num
     if (spatial >= (1ull << 31) && strided)
         return H2X_ERR_TOO_LARGE;
     const Chunking ch = elementwise_chunking(spatial, segments, vw, kUnroll / 2);
-    const size_t blocks = segments * ch.chunks_per_seg;
-    if (!grid_ok(blocks))
+    const size_t workgroups = segments * ch.chunks_per_seg;
+    if (!grid_ok(workgroups))
         return H2X_ERR_TOO_LARGE;
-    const unsigned int grid = static_cast<unsigned int>(blocks);
+    const unsigned int grid = static_cast<unsigned int>(workgroups);
     LaunchRecord rec = long_record(kKernelBackprop2, strided, vw, dim3(grid), num_samples,
                                    num_channels, spatial, ch, {&tx, &td, &to}, true);
     rec.folded = folded;
@@ -2003,19 +2050,20 @@ int backprop2_impl(int num_samples, int num_channels, size_t spatial, size_t num
     if (logged(rec))
         return H2X_SUCCESS;
     if (fused)
-        H2X_DISPATCH_FUSED(bn_backprop2_kernel, grid, static_cast<const T*>(x),
-                           static_cast<const T*>(dy), static_cast<const T*>(mean),
-                           static_cast<const T*>(var), static_cast<const T*>(scale), nullptr,
-                           nullptr, static_cast<T*>(dx), static_cast<T>(epsilon), num_per_sum,
-                           num_channels, spatial, tx.map, td.map, to.map, ch.chunk,
-                           ch.chunks_per_seg, disjoint, *fused);
+        H2X_DISPATCH_ELEMENTWISE(bn_backprop2_kernel, true, grid, static_cast<const T*>(x),
+                                 static_cast<const T*>(dy), static_cast<const T*>(mean),
+                                 static_cast<const T*>(var), static_cast<const T*>(scale), nullptr,
+                                 nullptr, static_cast<T*>(dx), static_cast<T>(epsilon), num_per_sum,
+                                 num_channels, spatial, tx.map, td.map, to.map, ch.chunk,
+                                 ch.chunks_per_seg, disjoint, *fused);
     else
-        H2X_DISPATCH(bn_backprop2_kernel, grid, static_cast<const T*>(x), static_cast<const T*>(dy),
-                     static_cast<const T*>(mean), static_cast<const T*>(var),
-                     static_cast<const T*>(scale), static_cast<const T*>(dmean),
-                     static_cast<const T*>(dvar), static_cast<T*>(dx), static_cast<T>(epsilon),
-                     num_per_sum, num_channels, spatial, tx.map, td.map, to.map, ch.chunk,
-                     ch.chunks_per_seg, disjoint);
+        H2X_DISPATCH_ELEMENTWISE(bn_backprop2_kernel, false, grid, static_cast<const T*>(x),
+                                 static_cast<const T*>(dy), static_cast<const T*>(mean),
+                                 static_cast<const T*>(var), static_cast<const T*>(scale),
+                                 static_cast<const T*>(dmean), static_cast<const T*>(dvar),
+                                 static_cast<T*>(dx), static_cast<T>(epsilon), num_per_sum,
+                                 num_channels, spatial, tx.map, td.map, to.map, ch.chunk,
+                                 ch.chunks_per_seg, disjoint);
     return issued();
 }
 

@@ -120,25 +120,29 @@ void walk_long(const LaunchRecord& r, TensorCount* count)
     const auto visit_chunk = [&](size_t n, int c, int k) {
         const size_t begin = static_cast<size_t>(k) * r.chunk;
         const size_t end = std::min(begin + r.chunk, r.spatial);
+        // the kernels place a vector by the map of the output (elementwise) or of x (reductions)
+        const TensorMap& placing = r.map[r.last_is_output ? r.num_tensors - 1 : 0];
         for (size_t i = begin; i + VEC <= end; i += VEC)
         {
+            Place pl{0, 0, 0, 0};
+            if constexpr (STRIDED && VEC > 1)
+                place_vector<VEC>(placing, row_split<VEC>(placing, i, &pl), &pl);
             for (int t = 0; t < r.num_tensors; ++t)
             {
                 const TensorMap& m = r.map[t];
-                uint32_t skip = 0;
                 size_t off;
                 if constexpr (!STRIDED || VEC == 1)
                     off = seg_offset<STRIDED>(m, i);
                 else
-                    off = row_vector_offset<VEC>(m, i, &skip);
+                    off = row_offset(m, pl) + pl.first;
                 const int64_t base = static_cast<int64_t>(n) * m.stride_n
                                      + static_cast<int64_t>(c) * m.stride_c + static_cast<int64_t>(off);
                 const bool output = r.last_is_output && t == r.num_tensors - 1;
                 for (int j = 0; j < VEC; ++j)
                 {
-                    const bool owns = j >= static_cast<int>(skip);
-                    if (output && !(skip == 0 || r.rewrite) && !owns)
-                        continue; // store_at leaves the shared elements to their owner
+                    const bool owns = j >= static_cast<int>(pl.skip);
+                    if (output && !(pl.skip == 0 || r.rewrite) && !owns)
+                        continue; // store_out leaves the shared elements to their owner
                     count[t].touch(base + j, output, owns);
                 }
             }

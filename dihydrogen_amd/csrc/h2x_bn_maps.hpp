@@ -29,7 +29,7 @@ struct TensorMap
 {
     int64_t stride_n, stride_c;
     FastDiv w, h;     // interior extents of spatial dimensions 0 and 1 (strided layout)
-    int64_t sy, sz;   // strides of spatial dimensions 1 and 2 (strided layout)
+    uint32_t sy, sz;  // strides of spatial dimensions 1 and 2 (strided layout); the host rejects larger ones
     FastDiv spr;      // vectors a row is padded to (strided layout with vectors)
     uint32_t width;   // elements of a row (strided layout with vectors)
 };
@@ -51,19 +51,41 @@ __host__ __device__ __forceinline__ size_t seg_offset(const TensorMap& m, size_t
     }
 }
 
-// Offset of the vector at padded index i (a multiple of VEC) and the number of
-// its leading elements that the vector before it owns.
+// Where the vector at a padded index lies: the row of the segment and the row
+// element its first lane holds.  Worked out once per vector from one map of the
+// launch (all maps of a launch share extents and padding) and then applied to
+// every tensor through that tensor's own strides.
+// Vector k of a row starts at element min(k * VEC, width - VEC); `skip` leading
+// elements belong to the vector before it.
+struct Place
+{
+    uint32_t y, z; // the row within its segment
+    int first;     // row element of the first lane
+    uint32_t skip; // leading elements that the vector before owns
+};
+
+// Row (y, z) of the vector at padded index i (a multiple of VEC); returns the vector's index within the row.
 template <int VEC>
-__host__ __device__ __forceinline__ size_t row_vector_offset(const TensorMap& m, size_t i, uint32_t* skip)
+__host__ __device__ __forceinline__ uint32_t row_split(const TensorMap& m, size_t i, Place* pl)
 {
     const uint32_t slot = static_cast<uint32_t>(i) / VEC;
     const uint32_t r = fastdiv(slot, m.spr);
-    const uint32_t x = (slot - r * m.spr.divisor) * VEC;
-    const uint32_t last = m.width - VEC;
-    *skip = x > last ? x - last : 0;
-    const uint32_t z = fastdiv(r, m.h);
-    const uint32_t y = r - z * m.h.divisor;
-    return (x > last ? last : x) + y * static_cast<size_t>(m.sy) + z * static_cast<size_t>(m.sz);
+    pl->z = fastdiv(r, m.h);
+    pl->y = r - pl->z * m.h.divisor;
+    return slot - r * m.spr.divisor;
+}
+
+__host__ __device__ __forceinline__ size_t row_offset(const TensorMap& m, const Place& pl)
+{
+    return static_cast<size_t>(pl.y) * m.sy + static_cast<size_t>(pl.z) * m.sz;
+}
+
+template <int VEC>
+__host__ __device__ __forceinline__ void place_vector(const TensorMap& m, uint32_t k, Place* pl)
+{
+    const uint32_t x = k * VEC, last = m.width - VEC;
+    pl->first = static_cast<int>(x > last ? last : x);
+    pl->skip = x > last ? x - last : 0;
 }
 
 struct ShortGeometry
