@@ -11,7 +11,10 @@
 #pragma once
 
 #include <algorithm>
+#include <fstream>
 #include <memory>
+#include <sstream>
+#include <string>
 #include <vector>
 
 #include "distconv/tensor_mi355x.hpp"
@@ -167,6 +170,27 @@ public:
     void* get_send_buffer(int dim, Side side) { return m_halo_send(dim, side).get(); }
     void* get_recv_buffer(int dim, Side side) { return m_halo_recv(dim, side).get(); }
 
+    // :204-255 -- debugging aids: the packed strips of a dimension as text, one
+    // value a line, in send_halo_<rank>_<dim>_<side>.txt and recv_halo_... under
+    // `directory` (the reference writes into the working directory).  They copy
+    // with the blocking hipMemcpy, like the reference's mem_copy; sides without
+    // a peer and buffers that were never allocated are left out.
+    void dump_packed_halo(int dim, const std::string& directory = ".")
+    {
+        for (Side side : SIDES)
+        {
+            if (get_peer(dim, side) == kProcNull)
+                continue;
+            dump_buffer(get_send_buffer(dim, side), "send_halo_", dim, side, directory);
+            dump_buffer(get_recv_buffer(dim, side), "recv_halo_", dim, side, directory);
+        }
+    }
+    void dump_recv_halo(int dim, const std::string& directory = ".")
+    {
+        for (Side side : SIDES)
+            dump_buffer(get_recv_buffer(dim, side), "recv_halo_", dim, side, directory);
+    }
+
     // :285-303 -- buffers are sized for the full halo width and zero-filled
     void ensure_halo_buffers(int dim)
     {
@@ -230,6 +254,21 @@ public:
     }
 
 protected:
+    void dump_buffer(const void* device, const char* prefix, int dim, Side side,
+                     const std::string& directory)
+    {
+        if (!device)
+            return;
+        std::vector<DataType> h(get_halo_size(dim));
+        DISTCONV_CHECK_HIP(hipMemcpy(h.data(), device, h.size() * sizeof(DataType), hipMemcpyDeviceToHost));
+        std::ostringstream path;
+        path << directory << "/" << prefix << m_tensor.get_locale().get_rank() << "_" << dim << "_"
+             << (side == LHS ? "LHS" : "RHS") << ".txt"; // base.hpp:30-36 prints a side by name
+        std::ofstream out(path.str(), std::ios::out | std::ios::trunc);
+        for (const DataType& v : h)
+            out << v << std::endl;
+    }
+
     // :322-357; with `periodic` the grid wraps, which the reference never does
     int find_peer_rank(int dim, Side side) const
     {

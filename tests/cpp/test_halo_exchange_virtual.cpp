@@ -4,6 +4,10 @@
 // global offset of its source.
 #include "test_common.hpp"
 
+#include <cstdlib>
+#include <fstream>
+#include <string>
+
 enum Mode
 {
     kBuffers,        // pack, unpack through receive buffers, one stream
@@ -167,6 +171,45 @@ int main()
         for (int y = 0; y < 6; ++y) // b's LHS halo column holds global x = 3
             if (h[y * 6 + 0] != static_cast<float>(3 + 8 * y))
                 ++errors;
+    }
+    // debugging dumps (halo_exchange_cuda.hpp:204-255): after an exchange of dimension 0 the receive
+    // buffer of rank 1's LHS side holds rank 0's RHS boundary column, one value a line
+    {
+        const Shape shape({8, 6, 2, 1}), locale({2, 1, 1, 1});
+        const Distribution dist = Distribution::make_overlapped_distribution(locale, IntVector({1, 0, 0, 0}));
+        DevTensor<float> a(shape, LocaleVirtual(0, 2), dist), b(shape, LocaleVirtual(1, 2), dist);
+        a.allocate();
+        b.allocate();
+        to_device(a, global_offset_field(a, -1.0f));
+        to_device(b, global_offset_field(b, -1.0f));
+        HaloExchangeVirtual<float> xch({&a, &b});
+        xch.exchange(nullptr);
+        DISTCONV_CHECK_HIP(hipDeviceSynchronize());
+        const char* tmp = std::getenv("TMPDIR");
+        const std::string dir = tmp ? tmp : "/tmp";
+        xch.rank(1).dump_packed_halo(0, dir);
+        std::ifstream in(dir + "/recv_halo_1_0_LHS.txt");
+        CHECK(in.good());
+        int lines = 0;
+        float v;
+        while (in >> v)
+        {
+            const int y = lines % 6, c = lines / 6; // strip of width 1: rows of the plane, then channels
+            if (v != static_cast<float>(3 + 8 * y + 48 * c))
+                ++errors;
+            ++lines;
+        }
+        errors += lines != 12;
+        // the local part of rank 1, raw: its real allocation, which now holds the filled LHS halo column
+        CHECK(dump_local_tensor(b, dir + "/h2x_dump_test", true) == 0);
+        std::ifstream raw(dir + "/h2x_dump_test_1.out", std::ios::binary);
+        std::vector<float> got(b.get_local_real_size());
+        raw.read(reinterpret_cast<char*>(got.data()), got.size() * sizeof(float));
+        CHECK(raw.gcount() == static_cast<std::streamsize>(got.size() * sizeof(float)));
+        errors += got != to_host(b);
+        std::remove((dir + "/h2x_dump_test_1.out").c_str());
+        std::remove((dir + "/recv_halo_1_0_LHS.txt").c_str());
+        std::remove((dir + "/send_halo_1_0_LHS.txt").c_str());
     }
     std::printf("test_halo_exchange_virtual: %d errors\n", errors);
     return finish(errors);
