@@ -993,6 +993,19 @@ def main() -> int:
         parity["C3_bn3d_haloed_fwd_bwd"] = gate_batchnorm(bn3h)
         breakdown["C3_bn3d_haloed_fwd_bwd"] = entry(8 * bn3h.elems * 4, bn3h.elems,
                                                     lambda: (bn3h.forward(), bn3h.backward()), inner=2)
+        # the same shard with clear_output_halo: normalise and the input gradient walk the whole real
+        # tensors in aligned vectors and leave the halos of y and dx cleared (what the convolution that
+        # follows would do with a separate clear_halo per dimension); the gate also looks at the halos
+        bn3h.bn.clear_output_halo = True
+        for t in (bn3h.y, bn3h.dx):
+            t.real_view().fill_(float("nan"))
+        bn3h.forward(), bn3h.backward()
+        parity["C3_bn3d_haloed_clearing_fwd_bwd"] = gate_batchnorm(bn3h)
+        for t, what in ((bn3h.y, "y"), (bn3h.dx, "dx")):
+            halo_sum = t.real_view().double().abs().sum() - t.interior_view().double().abs().sum()
+            _gate(bool(torch.isfinite(halo_sum)) and float(halo_sum) == 0.0, f"clearing batch-norm: halo of {what} is not zero")
+        breakdown["C3_bn3d_haloed_clearing_fwd_bwd"] = entry(8 * bn3h.elems * 4, bn3h.elems,
+                                                             lambda: (bn3h.forward(), bn3h.backward()), inner=2)
         del bn3h
         torch.cuda.empty_cache()
         # short segments (the last stage of a ResNet): a workgroup serves a window of whole channels

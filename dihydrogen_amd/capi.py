@@ -68,6 +68,17 @@ class TensorGeometry(ctypes.Structure):
     ]
 
 
+class HaloedGeometry(ctypes.Structure):
+    """struct h2x_haloed_geometry"""
+    _fields_ = [
+        ("num_dims", c_int32),
+        ("reserved", c_int32),
+        ("local_shape", c_int64 * H2X_MAX_DIMS),
+        ("real_shape", c_int64 * H2X_MAX_DIMS),
+        ("lower_halo", c_int64 * H2X_MAX_DIMS),
+    ]
+
+
 BN_STAGE_SUMS, BN_STAGE_NORMALIZE, BN_STAGE_BACKPROP1, BN_STAGE_BACKPROP2 = 0, 1, 2, 3
 BN_STAGE_FORWARD_LOCAL, BN_STAGE_BACKWARD_LOCAL = 4, 5
 BN_AUDIT_MAX_LAUNCHES = 8
@@ -149,6 +160,10 @@ SIGNATURES = {
                                          POINTER(TensorGeometry), POINTER(TensorGeometry), c_void_p,
                                          c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                          c_void_p, c_double, c_void_p]),
+    "h2x_bn_batch_normalization_clearing": (c_int, [c_int, POINTER(HaloedGeometry), c_void_p, c_void_p, c_void_p,
+                                                    c_void_p, c_void_p, c_void_p, c_double, c_void_p]),
+    "h2x_bn_backprop2_clearing": (c_int, [c_int, c_size_t, POINTER(HaloedGeometry), c_void_p, c_void_p, c_void_p,
+                                          c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_double, c_void_p]),
     "h2x_bn_audit": (c_int, [c_int, c_int, c_int, POINTER(POINTER(TensorGeometry)), POINTER(c_uint64),
                              POINTER(BnAuditReport)]),
     "h2x_tensor_transform": (c_int, [c_int, c_int, c_int, POINTER(POINTER(TensorGeometry)), POINTER(c_void_p),

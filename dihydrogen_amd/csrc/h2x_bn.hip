@@ -750,6 +750,125 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop2_kernel(
     }
 }
 
+// ---- normalise / input gradient that leave the halo of their output cleared ----
+// For tensors that share one haloed geometry.  The kernel walks the REAL local
+// tensor of every (sample, channel) segment - interior and halo cells alike - in
+// aligned 16-byte vectors, computes the interior elements and stores zeros into
+// the halo cells: what the reference's kernel followed by Tensor::clear_halo on
+// every spatial dimension leaves (legacy/src/tensor/tensor_mpi_cuda.cu:14-84;
+// Convolution::forward clears the halos of its input before every exchange,
+// legacy/include/distconv/dnn_backend/convolution.hpp:400-411), in one pass and
+// without the partly written sectors that the gaps between interior rows cost
+// the kernels above.  Halo cells of the inputs are loaded and ignored.
+struct RealBox
+{
+    FastDiv wr, hr;        // real extents of spatial dimensions 0 and 1
+    uint32_t lo[3], hi[3]; // interior: lo <= index < hi, per spatial dimension (real coordinates)
+};
+
+// Whether the elements i ... i + VEC - 1 of a real segment are interior ones.
+template <int VEC>
+__device__ __forceinline__ void interior_mask(const RealBox& b, uint32_t i, bool (&inside)[VEC])
+{
+    uint32_t t = fastdiv(i, b.wr);
+    uint32_t x = i - t * b.wr.divisor;
+    uint32_t z = fastdiv(t, b.hr);
+    uint32_t y = t - z * b.hr.divisor;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j)
+    {
+        inside[j] = x >= b.lo[0] && x < b.hi[0] && y >= b.lo[1] && y < b.hi[1] && z >= b.lo[2] && z < b.hi[2];
+        if (++x == b.wr.divisor)
+        {
+            x = 0;
+            if (++y == b.hr.divisor)
+            {
+                y = 0;
+                ++z;
+            }
+        }
+    }
+}
+
+// BACKWARD: the input gradient (x, dy -> dx); else normalise (x -> y).  Segments
+// are `real` elements long and follow one another (channel stride = real).
+template <typename T, int VEC, bool BACKWARD>
+__global__ __launch_bounds__(kBlockSize) void bn_clearing_kernel(
+    const T* x, const T* __restrict__ dy, const T* __restrict__ mean, const T* __restrict__ var,
+    const T* __restrict__ scale, const T* __restrict__ bias, const T* __restrict__ dmean,
+    const T* __restrict__ dvar, T* out, T epsilon, size_t num_per_sum, int num_channels, size_t real,
+    const RealBox box, size_t chunk, int chunks_per_seg)
+{
+    const size_t seg = blockIdx.x / chunks_per_seg;
+    const int k = blockIdx.x - seg * chunks_per_seg;
+    const int c = seg % num_channels;
+    const T m = mean[c];
+    const T sc = scale[c];
+    const T inv_stdev = inv_sqrt_t(var[c] + epsilon);
+    T bi = T(0), dmean_term = T(0), dvar_term = T(0);
+    if constexpr (BACKWARD)
+    {
+        dmean_term = dmean[c] / static_cast<T>(num_per_sum);
+        dvar_term = dvar[c] * T(2) / static_cast<T>(num_per_sum - 1);
+    }
+    else
+    {
+        bi = bias[c];
+    }
+    const size_t begin = static_cast<size_t>(k) * chunk;
+    const size_t end = begin + chunk < real ? begin + chunk : real;
+    const T* xp = x + seg * real;
+    const T* dp = BACKWARD ? dy + seg * real : nullptr;
+    T* op = out + seg * real;
+
+    auto result = [&](T xv, T dv) {
+        if constexpr (BACKWARD)
+            return fma_t(xv - m, dvar_term, fma_t(dv * sc, inv_stdev, dmean_term));
+        else
+            return fma_t((xv - m) * inv_stdev, sc, bi);
+    };
+    constexpr size_t kStride = static_cast<size_t>(kBlockSize) * VEC;
+    constexpr int kInFlight = BACKWARD ? kUnroll / 2 : kUnroll;
+    constexpr size_t kTile = kStride * kInFlight;
+    size_t tile = begin;
+    for (; tile + kTile <= end; tile += kTile)
+    {
+        T xv[kInFlight][VEC], dv[kInFlight][VEC];
+#pragma unroll
+        for (int u = 0; u < kInFlight; ++u)
+        {
+            const size_t i = tile + u * kStride + threadIdx.x * VEC;
+            load_vec<T, VEC, true>(xp + i, xv[u]);
+            if constexpr (BACKWARD)
+                load_vec<T, VEC, true, true>(dp + i, dv[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < kInFlight; ++u)
+        {
+            const size_t i = tile + u * kStride + threadIdx.x * VEC;
+            bool inside[VEC];
+            interior_mask<VEC>(box, static_cast<uint32_t>(i), inside);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j)
+                xv[u][j] = inside[j] ? result(xv[u][j], BACKWARD ? dv[u][j] : T(0)) : T(0);
+            store_vec<T, VEC, true>(op + i, xv[u]);
+        }
+    }
+    for (size_t i = tile + threadIdx.x * VEC; i + VEC <= end; i += kStride)
+    {
+        T xv[VEC], dv[VEC];
+        load_vec<T, VEC, true>(xp + i, xv);
+        if constexpr (BACKWARD)
+            load_vec<T, VEC, true, true>(dp + i, dv);
+        bool inside[VEC];
+        interior_mask<VEC>(box, static_cast<uint32_t>(i), inside);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j)
+            xv[j] = inside[j] ? result(xv[j], BACKWARD ? dv[j] : T(0)) : T(0);
+        store_vec<T, VEC, true>(op + i, xv);
+    }
+}
+
 // ---- short segments: whole channels side by side in one workgroup ------------
 // A (sample, channel) segment of a few hundred bytes (7 x 7 or 14 x 14
 // activations, 1 x 1 after a fully connected layer) shares its first and last
@@ -2067,6 +2186,81 @@ int backprop2_impl(int num_samples, int num_channels, size_t spatial, size_t num
     return issued();
 }
 
+// Normalise / input gradient over tensors of one haloed geometry, the halo of
+// the output cleared (bn_clearing_kernel).
+template <typename T>
+int clearing_impl(bool backward, size_t num_per_sum, const h2x_haloed_geometry* g, const void* x,
+                  const void* dy, const void* mean, const void* var, const void* scale,
+                  const void* bias, const void* dmean, const void* dvar, void* out, double epsilon,
+                  hipStream_t stream)
+{
+    if (!g || g->num_dims < 3 || g->num_dims > 5)
+        return H2X_ERR_INVALID_ARGUMENT;
+    const int nd = g->num_dims, ns = nd - 2;
+    RealBox box;
+    size_t real = 1, extent[3] = {1, 1, 1};
+    for (int d = 0; d < 3; ++d)
+    {
+        box.lo[d] = 0;
+        box.hi[d] = 1;
+    }
+    for (int d = 0; d < nd; ++d)
+    {
+        if (g->local_shape[d] < 0 || g->lower_halo[d] < 0
+            || g->lower_halo[d] + g->local_shape[d] > g->real_shape[d])
+            return H2X_ERR_INVALID_ARGUMENT;
+        if (d >= ns && (g->lower_halo[d] != 0 || g->real_shape[d] != g->local_shape[d]))
+            return H2X_ERR_UNSUPPORTED; // no halo on the channel and sample dimensions
+    }
+    for (int d = 0; d < ns; ++d)
+    {
+        extent[d] = static_cast<size_t>(g->real_shape[d]);
+        real *= extent[d];
+        if (real >= (1ull << 31))
+            return H2X_ERR_TOO_LARGE;
+        box.lo[d] = static_cast<uint32_t>(g->lower_halo[d]);
+        box.hi[d] = static_cast<uint32_t>(g->lower_halo[d] + g->local_shape[d]);
+    }
+    const int num_channels = static_cast<int>(g->local_shape[nd - 2]);
+    const size_t segments = static_cast<size_t>(g->local_shape[nd - 1]) * num_channels;
+    if (segments == 0 || real == 0)
+        return H2X_SUCCESS;
+    if (!x || !out || (backward && !dy))
+        return H2X_ERR_INVALID_ARGUMENT;
+    box.wr = make_fastdiv(static_cast<uint32_t>(extent[0]));
+    box.hr = make_fastdiv(static_cast<uint32_t>(extent[1]));
+    const bool vectors = real % full_vec<T>() == 0 && aligned16(x) && aligned16(out)
+                         && (!backward || aligned16(dy));
+    const int vw = vectors ? full_vec<T>() : 1;
+    const Chunking ch = elementwise_chunking(real, segments, vw, backward ? kUnroll / 2 : kUnroll);
+    const size_t workgroups = segments * ch.chunks_per_seg;
+    if (!grid_ok(workgroups))
+        return H2X_ERR_TOO_LARGE;
+    const unsigned int grid = static_cast<unsigned int>(workgroups);
+#define H2X_LAUNCH_CLEARING(VEC, BACKWARD)                                                         \
+    bn_clearing_kernel<T, VEC, BACKWARD><<<grid, kBlockSize, 0, stream>>>(                         \
+        static_cast<const T*>(x), static_cast<const T*>(dy), static_cast<const T*>(mean),          \
+        static_cast<const T*>(var), static_cast<const T*>(scale), static_cast<const T*>(bias),     \
+        static_cast<const T*>(dmean), static_cast<const T*>(dvar), static_cast<T*>(out),           \
+        static_cast<T>(epsilon), num_per_sum, num_channels, real, box, ch.chunk, ch.chunks_per_seg)
+    if (backward)
+    {
+        if (vectors)
+            H2X_LAUNCH_CLEARING(full_vec<T>(), true);
+        else
+            H2X_LAUNCH_CLEARING(1, true);
+    }
+    else
+    {
+        if (vectors)
+            H2X_LAUNCH_CLEARING(full_vec<T>(), false);
+        else
+            H2X_LAUNCH_CLEARING(1, false);
+    }
+#undef H2X_LAUNCH_CLEARING
+    return launch_status();
+}
+
 bool bad_geometry(int num_samples, int num_channels, size_t spatial, size_t real)
 {
     return num_samples < 0 || num_channels < 0 || real < spatial;
@@ -2489,6 +2683,39 @@ extern "C" int h2x_bn_backprop2_strided(h2x_dtype dtype, int num_samples, size_t
                  backprop2_strided<double>(num_samples, num_per_sum, x_geometry, dy_geometry,
                                            dx_geometry, x, dy, mean, var, scale, dmean, dvar, dx,
                                            epsilon, as_stream(stream)));
+}
+
+extern "C" int h2x_bn_batch_normalization_clearing(h2x_dtype dtype,
+                                                   const h2x_haloed_geometry* geometry,
+                                                   const void* x_buffer, const void* mean,
+                                                   const void* var, const void* scale,
+                                                   const void* bias, void* y_buffer, double epsilon,
+                                                   h2x_stream_t stream)
+{
+    if (!geometry || !mean || !var || !scale || !bias)
+        return H2X_ERR_INVALID_ARGUMENT;
+    H2X_BY_DTYPE(dtype,
+                 clearing_impl<float>(false, 0, geometry, x_buffer, nullptr, mean, var, scale, bias,
+                                      nullptr, nullptr, y_buffer, epsilon, as_stream(stream)),
+                 clearing_impl<double>(false, 0, geometry, x_buffer, nullptr, mean, var, scale, bias,
+                                       nullptr, nullptr, y_buffer, epsilon, as_stream(stream)));
+}
+
+extern "C" int h2x_bn_backprop2_clearing(h2x_dtype dtype, size_t num_per_sum,
+                                         const h2x_haloed_geometry* geometry, const void* x_buffer,
+                                         const void* dy_buffer, const void* mean, const void* var,
+                                         const void* scale, const void* dmean, const void* dvar,
+                                         void* dx_buffer, double epsilon, h2x_stream_t stream)
+{
+    if (!geometry || !mean || !var || !scale || !dmean || !dvar)
+        return H2X_ERR_INVALID_ARGUMENT;
+    H2X_BY_DTYPE(dtype,
+                 clearing_impl<float>(true, num_per_sum, geometry, x_buffer, dy_buffer, mean, var,
+                                      scale, nullptr, dmean, dvar, dx_buffer, epsilon,
+                                      as_stream(stream)),
+                 clearing_impl<double>(true, num_per_sum, geometry, x_buffer, dy_buffer, mean, var,
+                                       scale, nullptr, dmean, dvar, dx_buffer, epsilon,
+                                       as_stream(stream)));
 }
 
 extern "C" int h2x_bn_forward_local(h2x_dtype dtype, int num_samples, int num_channels,

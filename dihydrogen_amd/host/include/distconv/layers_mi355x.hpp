@@ -77,6 +77,42 @@ h2x_tensor_geometry tensor_geometry(const Tensor& t, int num_samples)
     return g;
 }
 
+// Local and real extents and halo widths, for the entry points that also
+// clear the halo of their output.
+template <typename Tensor>
+h2x_haloed_geometry haloed_geometry(const Tensor& t)
+{
+    h2x_haloed_geometry g = {};
+    g.num_dims = t.get_num_dims();
+    for (int i = 0; i < g.num_dims; ++i)
+    {
+        g.local_shape[i] = static_cast<int64_t>(t.get_local_shape()[i]);
+        g.real_shape[i] = static_cast<int64_t>(t.get_local_real_shape()[i]);
+        g.lower_halo[i] = t.get_halo_width(i);
+    }
+    return g;
+}
+
+// Whether `a` has a halo on a spatial dimension (and none on channel or sample).
+template <typename Tensor>
+bool has_spatial_halo(const Tensor& a)
+{
+    const int nd = a.get_num_dims();
+    bool any = false;
+    for (int i = 0; i < nd - 2; ++i)
+        any = any || a.get_halo_width(i) > 0;
+    return any && a.get_halo_width(nd - 2) == 0 && a.get_halo_width(nd - 1) == 0;
+}
+
+// Whether the local parts of two tensors lie in memory alike.
+template <typename Tensor>
+bool same_haloed_geometry(const Tensor& a, const Tensor& b)
+{
+    return a.get_local_shape() == b.get_local_shape()
+           && a.get_local_real_shape() == b.get_local_real_shape()
+           && a.get_halo_width() == b.get_halo_width();
+}
+
 // Workspace of fp64 partial sums.  A default-constructed one owns its memory
 // (one per layer object, freed with the object); one made by
 // default_workspace() refers to the buffer that the calls of one stream share.
@@ -193,6 +229,42 @@ void batch_normalization(int num_dims, int num_samples, const Tensor& input, con
             mean.get_const_base_ptr(), var.get_const_base_ptr(), scale.get_const_base_ptr(),
             bias.get_const_base_ptr(), output.get_base_ptr(), epsilon, stream));
     }
+}
+
+// No counterpart in the reference: batch_normalization for haloed tensors of one
+// geometry that also clears the halo of `output`, as Tensor::clear_halo on every
+// spatial dimension would (tensor_mpi_cuda.cu:14-84), in one pass.
+template <typename Tensor>
+void batch_normalization_clearing(const Tensor& input, const Tensor& mean, const Tensor& var,
+                                  const Tensor& scale, const Tensor& bias, Tensor& output,
+                                  typename Tensor::data_type epsilon, hipStream_t stream)
+{
+    if (input.get_local_size() == 0)
+        return;
+    assert_always(same_haloed_geometry(input, output));
+    const h2x_haloed_geometry g = haloed_geometry(output);
+    DISTCONV_CHECK_H2X(h2x_bn_batch_normalization_clearing(
+        Tensor::h2x_type(), &g, input.get_const_buffer(), mean.get_const_base_ptr(),
+        var.get_const_base_ptr(), scale.get_const_base_ptr(), bias.get_const_base_ptr(),
+        output.get_buffer(), epsilon, stream));
+}
+
+// Likewise the input gradient; d_input may be the same tensor as input.
+template <typename Tensor>
+void backprop2_clearing(index_t num_per_sum, const Tensor& input, const Tensor& d_output,
+                        const Tensor& mean, const Tensor& var, const Tensor& scale,
+                        const Tensor& mean_gradient, const Tensor& var_gradient, Tensor& d_input,
+                        typename Tensor::data_type epsilon, hipStream_t stream)
+{
+    if (input.get_local_size() == 0)
+        return;
+    assert_always(same_haloed_geometry(input, d_output) && same_haloed_geometry(input, d_input));
+    const h2x_haloed_geometry g = haloed_geometry(d_input);
+    DISTCONV_CHECK_H2X(h2x_bn_backprop2_clearing(
+        Tensor::h2x_type(), num_per_sum, &g, input.get_const_buffer(), d_output.get_const_buffer(),
+        mean.get_const_base_ptr(), var.get_const_base_ptr(), scale.get_const_base_ptr(),
+        mean_gradient.get_const_base_ptr(), var_gradient.get_const_base_ptr(), d_input.get_buffer(),
+        epsilon, stream));
 }
 
 // batchnorm.hpp:68-81
@@ -319,17 +391,16 @@ public:
                        bool is_training)
     {
         if (is_training)
-        {
             batchnorm::sums_to_statistics(num_per_sum(input), m_decay, mean, var, running_mean,
                                           running_var, m_stream);
-            batchnorm::batch_normalization(m_num_dims, m_num_current_samples, input, mean, var,
-                                           scale, bias, output, m_epsilon, m_stream);
-        }
+        const Tensor& m = is_training ? mean : running_mean;
+        const Tensor& v = is_training ? var : running_var;
+        if (clears(input) && batchnorm::same_haloed_geometry(input, output))
+            batchnorm::batch_normalization_clearing(input, m, v, scale, bias, output, m_epsilon,
+                                                    m_stream);
         else
-        {
-            batchnorm::batch_normalization(m_num_dims, m_num_current_samples, input, running_mean,
-                                           running_var, scale, bias, output, m_epsilon, m_stream);
-        }
+            batchnorm::batch_normalization(m_num_dims, m_num_current_samples, input, m, v, scale,
+                                           bias, output, m_epsilon, m_stream);
         return 0;
     }
 
@@ -339,12 +410,19 @@ public:
     // staged calls, bit for bit.  set_fuse_local(false) keeps the staged calls.
     void set_fuse_local(bool on) { m_fuse_local = on; }
 
+    // Haloed tensors of one geometry: normalise and the input gradient also
+    // clear the halo of their output, in one pass over the real tensors (what
+    // Convolution::forward does to its input with a clear_halo per dimension
+    // before every exchange, convolution.hpp:400-411).  Off by default: the
+    // reference's kernels leave halo cells alone.
+    void set_clear_output_halo(bool on) { m_clear_output_halo = on; }
+
     template <typename Tensor>
     int forward(const Tensor& input, Tensor& mean, Tensor& var, Tensor& running_mean,
                 Tensor& running_var, Tensor& scale, Tensor& bias, Tensor& output, bool is_training)
     {
         if (is_training && runs_local(input) && batchnorm::is_dense(input)
-            && batchnorm::is_dense(output))
+            && batchnorm::is_dense(output) && !wants_clearing(input) && !wants_clearing(output))
         {
             set_num_samples(static_cast<int>(input.get_local_shape()[-1]));
             const batchnorm::ChannelGeometry<Tensor> gi(input), go(output);
@@ -396,9 +474,14 @@ public:
                         const Tensor& var, const Tensor& scale, const Tensor& mean_gradient,
                         const Tensor& var_gradient, Tensor& d_input)
     {
-        batchnorm::backprop2(m_num_dims, m_num_current_samples, num_per_sum(input), input, d_output,
-                             mean, var, scale, mean_gradient, var_gradient, d_input, m_epsilon,
-                             m_stream);
+        if (clears(input) && batchnorm::same_haloed_geometry(input, d_output)
+            && batchnorm::same_haloed_geometry(input, d_input))
+            batchnorm::backprop2_clearing(num_per_sum(input), input, d_output, mean, var, scale,
+                                          mean_gradient, var_gradient, d_input, m_epsilon, m_stream);
+        else
+            batchnorm::backprop2(m_num_dims, m_num_current_samples, num_per_sum(input), input,
+                                 d_output, mean, var, scale, mean_gradient, var_gradient, d_input,
+                                 m_epsilon, m_stream);
         return 0;
     }
 
@@ -408,7 +491,7 @@ public:
                  Tensor& mean_gradient, Tensor& var_gradient, Tensor& d_input)
     {
         if (runs_local(input) && batchnorm::is_dense(input) && batchnorm::is_dense(d_output)
-            && batchnorm::is_dense(d_input))
+            && batchnorm::is_dense(d_input) && !wants_clearing(input) && !wants_clearing(d_input))
         {
             set_num_samples(static_cast<int>(input.get_local_shape()[-1]));
             const batchnorm::ChannelGeometry<Tensor> gi(input), go(d_output), gd(d_input);
@@ -439,6 +522,19 @@ private:
     {
         return m_fuse_local && !(m_global_stats && m_allreducer) && input.get_local_size() > 0
                && input.is_split_root();
+    }
+
+    // the clearing entry points serve this tensor: it has a halo on a spatial
+    // dimension and the whole local mini-batch is current
+    template <typename Tensor>
+    bool clears(const Tensor& t) const
+    {
+        return wants_clearing(t) && m_num_current_samples == static_cast<int>(t.get_local_shape()[-1]);
+    }
+    template <typename Tensor>
+    bool wants_clearing(const Tensor& t) const
+    {
+        return m_clear_output_halo && batchnorm::has_spatial_halo(t);
     }
 
     // elements per channel of the global (global statistics) or local shape:
@@ -478,6 +574,7 @@ private:
     BatchnormImpl m_impl;
     bool m_global_stats;
     bool m_fuse_local = true;
+    bool m_clear_output_halo = false;
     Allreduce m_allreducer;
     batchnorm::Workspace m_ws;
 };

@@ -60,6 +60,26 @@ def _tensor_geometry(t: Tensor, num_samples: int) -> capi.TensorGeometry:
     return g
 
 
+def _haloed_geometry(t: Tensor) -> capi.HaloedGeometry:
+    """h2x_haloed_geometry of a local tensor: local and real extents, halo widths."""
+    g = capi.HaloedGeometry()
+    g.num_dims = t.get_num_dims()
+    for i in range(g.num_dims):
+        g.local_shape[i] = t.local_shape[i]
+        g.real_shape[i] = t.local_real_shape[i]
+        g.lower_halo[i] = t.overlap[i]
+    return g
+
+
+def _share_a_haloed_geometry(*tensors: Tensor) -> bool:
+    """Tensors with a halo on a spatial dimension whose local parts lie in memory alike."""
+    t0 = tensors[0]
+    nd = t0.get_num_dims()
+    return (any(t0.overlap[: nd - 2]) and t0.overlap[nd - 2] == 0 and t0.overlap[nd - 1] == 0
+            and all(t.local_shape == t0.local_shape and t.local_real_shape == t0.local_real_shape
+                    and t.overlap == t0.overlap and t.h2x_dtype == t0.h2x_dtype for t in tensors))
+
+
 class BatchNormalization:
     """BatchNormalization<Backend, DataType>
     (legacy/include/distconv/dnn_backend/batchnorm.hpp:100-581).
@@ -71,7 +91,8 @@ class BatchNormalization:
 
     def __init__(self, num_dims: int, decay: float, epsilon: float, global_stats: bool = False,
                  allreduce: Optional[Callable[[List[torch.Tensor]], None]] = None,
-                 stream: Optional[torch.cuda.Stream] = None, fuse_local: bool = True):
+                 stream: Optional[torch.cuda.Stream] = None, fuse_local: bool = True,
+                 clear_output_halo: bool = False):
         if num_dims not in (4, 5):
             raise ValueError("4-D (NCHW) or 5-D (NCDHW) tensors only")  # batchnorm.cu:259-270
         self.num_dims, self.decay, self.epsilon = num_dims, float(decay), float(epsilon)
@@ -80,6 +101,12 @@ class BatchNormalization:
         # stages run as two launches each (h2x_bn_forward_local / _backward_local);
         # the staged methods always use the staged entry points
         self.fuse_local = fuse_local
+        # Haloed tensors of one geometry: normalise and the input gradient also clear
+        # the halo of their output (what Convolution::forward does to its input before
+        # every exchange, convolution.hpp:400-411), in one pass over the real tensors
+        # (h2x_bn_batch_normalization_clearing / h2x_bn_backprop2_clearing).  Off by
+        # default: the reference's kernels leave halo cells alone.
+        self.clear_output_halo = clear_output_halo
         self.num_current_samples = 0
         self._lib = capi.load()
         self._workspace: Optional[torch.Tensor] = None
@@ -141,7 +168,13 @@ class BatchNormalization:
         n, c, s, sr = _channel_geometry(input)
         _, _, so, sro = _channel_geometry(output)
         ns = self.num_current_samples
-        if _is_dense(input) and _is_dense(output):
+        if self.clear_output_halo and ns == n and _share_a_haloed_geometry(input, output):
+            g = _haloed_geometry(output)
+            capi.check(self._lib.h2x_bn_batch_normalization_clearing(
+                input.h2x_dtype, ctypes.byref(g), _ptr(input.get_buffer()), _ptr(mean), _ptr(var), _ptr(scale),
+                _ptr(bias), _ptr(output.get_buffer()), self.epsilon, _stream_handle(self.stream)),
+                "batch_normalization (clearing)")
+        elif _is_dense(input) and _is_dense(output):
             capi.check(self._lib.h2x_bn_batch_normalization(
                 input.h2x_dtype, ns, c, s, sr, sro, _ptr(input.get_base_ptr()), _ptr(mean), _ptr(var),
                 _ptr(scale), _ptr(bias), _ptr(output.get_base_ptr()), self.epsilon,
@@ -167,7 +200,8 @@ class BatchNormalization:
         """No all-reduce between the stages, dense tensors, a rank that owns elements."""
         t0 = tensors[0]
         return (self.fuse_local and not (self.global_stats and self.allreduce is not None)
-                and all(_is_dense(t) for t in tensors) and t0.is_split_root() and t0.get_local_size() > 0)
+                and all(_is_dense(t) for t in tensors) and t0.is_split_root() and t0.get_local_size() > 0
+                and not (self.clear_output_halo and any(any(t.overlap) for t in tensors)))
 
     def forward(self, input, mean, var, running_mean, running_var, scale, bias, output,
                 is_training: bool = True) -> int:
@@ -227,8 +261,15 @@ class BatchNormalization:
         tail = (_ptr(input.get_base_ptr()), _ptr(d_output.get_base_ptr()), _ptr(mean), _ptr(var),
                 _ptr(scale), _ptr(mean_gradient), _ptr(var_gradient), _ptr(d_input.get_base_ptr()),
                 self.epsilon, _stream_handle(self.stream))
+        if self.clear_output_halo and ns == n and _share_a_haloed_geometry(input, d_output, d_input):
+            g = _haloed_geometry(d_input)
+            capi.check(self._lib.h2x_bn_backprop2_clearing(
+                input.h2x_dtype, self._num_per_sum(input), ctypes.byref(g), _ptr(input.get_buffer()),
+                _ptr(d_output.get_buffer()), _ptr(mean), _ptr(var), _ptr(scale), _ptr(mean_gradient),
+                _ptr(var_gradient), _ptr(d_input.get_buffer()), self.epsilon, _stream_handle(self.stream)),
+                "backprop2 (clearing)")
         # the reference takes its fast path only for halo-free tensors (batchnorm.cu:1503-1506)
-        if _is_dense(input) and _is_dense(d_output) and _is_dense(d_input):
+        elif _is_dense(input) and _is_dense(d_output) and _is_dense(d_input):
             capi.check(self._lib.h2x_bn_backprop2(
                 input.h2x_dtype, ns, c, s, sr, sro, sri, self._num_per_sum(input), *tail), "backprop2")
         else:

@@ -249,11 +249,64 @@ static int test_bn_haloed()
     return errors;
 }
 
+// set_clear_output_halo: the outputs of normalise and of the input gradient equal, in every cell
+// of the real tensors, what the plain calls followed by clear_halo on every dimension leave.
+static int test_bn_clearing()
+{
+    const Shape shape({20, 12, 10, 3, 2});
+    const Shape locale({2, 2, 2, 1, 1});
+    const Distribution dh = Distribution::make_overlapped_distribution(locale, IntVector({1, 2, 1, 0, 0}));
+    Shape pshape({1, 1, 1, 3, 1});
+    const Distribution dl = Distribution::make_localized_distribution(5);
+    int errors = 0;
+    for (int r : {0, 5})
+    {
+        const LocaleVirtual loc(r, 8), one(0, 1);
+        std::vector<std::vector<float>> outs[2];
+        for (int clearing = 0; clearing < 2; ++clearing)
+        {
+            DevTensor<float> x(shape, loc, dh), y(shape, loc, dh), dy(shape, loc, dh), dx(shape, loc, dh);
+            std::vector<DevTensor<float>> pv;
+            for (int i = 0; i < 10; ++i)
+            {
+                pv.emplace_back(pshape, one, dl);
+                pv.back().allocate();
+            }
+            for (auto* t : {&x, &y, &dy, &dx})
+                t->allocate();
+            to_device(x, randn(x.get_local_real_size(), 300 + r));   // halo cells hold values too
+            to_device(dy, randn(x.get_local_real_size(), 400 + r));
+            to_device(y, std::vector<float>(x.get_local_real_size(), NAN));
+            to_device(dx, std::vector<float>(x.get_local_real_size(), NAN));
+            to_device(pv[4], randn(3, 3, 0.25f, 1.0f));
+            to_device(pv[5], randn(3, 4, 0.1f));
+            to_device(pv[3], std::vector<float>(3, 1.0f));
+            BackendMI355X backend;
+            BatchNormalization<BackendMI355X, float> bn(backend, 5, 0.9f, 1e-5f, false);
+            bn.set_clear_output_halo(clearing == 1);
+            bn.forward(x, pv[0], pv[1], pv[2], pv[3], pv[4], pv[5], y, true);
+            bn.backward(x, dy, pv[0], pv[1], pv[4], pv[6], pv[7], pv[8], pv[9], dx);
+            if (!clearing)
+                for (int d = 0; d < 3; ++d)
+                {
+                    y.clear_halo(d, nullptr);
+                    dx.clear_halo(d, nullptr);
+                }
+            outs[clearing] = {to_host(y), to_host(dx), to_host(pv[0]), to_host(pv[1]), to_host(pv[6]),
+                              to_host(pv[7]), to_host(pv[8]), to_host(pv[9])};
+        }
+        for (size_t k = 0; k < outs[0].size(); ++k)
+            errors += std::memcmp(outs[0][k].data(), outs[1][k].data(), outs[0][k].size() * sizeof(float)) != 0;
+    }
+    return errors;
+}
+
 int main()
 {
     std::setvbuf(stdout, nullptr, _IONBF, 0); // what was printed survives a crash
     int errors = 0;
     errors += test_bn_haloed();
+    errors += test_bn_clearing();
     {
         // util::Clock brackets work on a stream, as the reference's benchmark does
         // (legacy/benchmarks/distconv_benchmark_bn.cpp:254-295); sync_stream orders two streams

@@ -421,6 +421,98 @@ def test_haloed_tensors_match_oracle(case, oracle_mod):
             assert int(torch.isnan(t.real_view()).sum()) == t.get_local_real_size() - t.get_local_size()
 
 
+CLEARING_CASES = HALO_CASES + [
+    ((16, 8, 6, 2), (1, 2, 1, 1), (0, 3, 0, 0)),          # halo on the outermost spatial dimension only
+    ((10, 6, 6, 3, 2), (2, 1, 2, 1, 1), (1, 0, 2, 0, 0)),  # real segment of 7 x 6 x 7 elements: no whole vectors
+    ((128, 128, 8, 2), (2, 2, 1, 1), (1, 1, 0, 0)),        # 66 x 66 real: rows 8 bytes off every other time
+]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float64"])
+@pytest.mark.parametrize("case", CLEARING_CASES)
+def test_clearing_variants_equal_the_strided_calls_followed_by_clear_halo(case, dtype):
+    """clear_output_halo: normalise and the input gradient leave the halo of their output
+    cleared.  Bit for bit what the reference's sequence leaves: the kernel on the interior,
+    then Tensor::clear_halo on every spatial dimension of the output
+    (legacy/src/tensor/tensor_mpi_cuda.cu:14-84); the halos of the inputs hold NaNs and stay."""
+    import ctypes
+    import torch
+    from dihydrogen_amd import capi
+    from dihydrogen_amd.layers import BatchNormalization
+    from dihydrogen_amd.tensor import Distribution, LocaleVirtual, Tensor
+    lib = capi.load()
+    gshape, locale, overlap = case
+    nd = len(gshape)
+    nranks = int(np.prod(locale))
+    tdt = getattr(torch, dtype)
+    dist = Distribution.make_overlapped_distribution(locale, overlap)
+    c = gshape[nd - 2]
+    g = torch.Generator(device="cuda").manual_seed(31)
+    scale = torch.empty(c, dtype=tdt, device="cuda").uniform_(0.5, 1.5, generator=g)
+    bias = torch.empty(c, dtype=tdt, device="cuda").normal_(0, 0.1, generator=g)
+    for r in range(nranks):
+        loc = LocaleVirtual(r, nranks)
+        results = []
+        xi = di = None
+        for clearing in (False, True):
+            x, y, dy, dx = (Tensor(gshape, loc, dist, tdt).allocate() for _ in range(4))
+            for t in (x, y, dy, dx):
+                t.real_view().fill_(float("nan"))
+            if xi is None:
+                xi = torch.empty_like(x.interior_view()).normal_(0, 1, generator=g)
+                di = torch.empty_like(x.interior_view()).normal_(0, 1, generator=g)
+            x.interior_view().copy_(xi)
+            dy.interior_view().copy_(di)
+            vec = lambda: torch.empty(c, dtype=tdt, device="cuda")
+            mean, var, rm, rv = vec(), vec(), torch.zeros(c, dtype=tdt, device="cuda"), torch.ones(c, dtype=tdt, device="cuda")
+            grads = [vec() for _ in range(4)]
+            bn = BatchNormalization(nd, 0.9, 1e-5, clear_output_halo=clearing)
+            assert bn.forward(x, mean, var, rm, rv, scale, bias, y, True) == 0
+            assert bn.backward(x, dy, mean, var, scale, *grads, dx) == 0
+            if not clearing:
+                for t in (y, dx):
+                    for d in range(nd - 2):
+                        if t.overlap[d]:
+                            capi.check(lib.h2x_halo_clear(t.h2x_dtype, ctypes.c_void_p(t.get_buffer()), nd,
+                                                          capi.i64_array(t.local_real_shape), d, t.overlap[d], None))
+            torch.cuda.synchronize()
+            results.append([t.real_view().cpu().numpy() for t in (y, dx)] + [v.cpu().numpy() for v in (mean, var, *grads)])
+            # the inputs are untouched: their halos still hold NaNs
+            for t in (x, dy):
+                assert int(torch.isnan(t.real_view()).sum()) == t.get_local_real_size() - t.get_local_size()
+        for a, b in zip(*results):
+            assert np.array_equal(a, b)
+        assert not np.isnan(results[1][0]).any() and not np.isnan(results[1][1]).any()
+
+
+def test_clearing_input_gradient_in_place():
+    """dx == x with clear_output_halo: the interior holds the gradient, the halo zeros."""
+    import torch
+    from dihydrogen_amd.layers import BatchNormalization
+    from dihydrogen_amd.tensor import Distribution, LocaleVirtual, Tensor
+    gshape, locale, overlap = (60, 12, 10, 3, 2), (2, 1, 2, 1, 1), (1, 0, 1, 0, 0)
+    dist = Distribution.make_overlapped_distribution(locale, overlap)
+    loc = LocaleVirtual(1, 4)
+    g = torch.Generator(device="cuda").manual_seed(37)
+    c = gshape[3]
+    outs = []
+    for alias in (False, True):
+        x, y, dy, dx = (Tensor(gshape, loc, dist).allocate() for _ in range(4))
+        torch.manual_seed(5)
+        for t in (x, dy):
+            t.real_view().copy_(torch.randn(t.real_view().shape, device="cuda"))
+        scale, bias = torch.ones(c, device="cuda") * 1.25, torch.zeros(c, device="cuda")
+        mean, var, rm, rv = (torch.zeros(c, device="cuda") for _ in range(4))
+        grads = [torch.empty(c, device="cuda") for _ in range(4)]
+        bn = BatchNormalization(5, 0.9, 1e-5, clear_output_halo=True)
+        bn.forward(x, mean, var, rm, rv, scale, bias, y, True)
+        target = x if alias else dx
+        bn.backward(x, dy, mean, var, scale, *grads, target)
+        torch.cuda.synchronize()
+        outs.append(target.real_view().cpu().numpy())
+    assert np.array_equal(outs[0], outs[1])
+
+
 def test_non_finite_inputs_propagate_as_in_the_oracle(oracle_mod):
     """A NaN, an infinity, values near the float32 maximum (whose squares overflow
     float32 but not the float64 accumulators) and denormals, each in a channel of
