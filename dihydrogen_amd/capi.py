@@ -160,6 +160,13 @@ SIGNATURES = {
                                          POINTER(TensorGeometry), POINTER(TensorGeometry), c_void_p,
                                          c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                          c_void_p, c_double, c_void_p]),
+    "h2x_bn_forward_local_strided": (c_int, [c_int, c_int, POINTER(TensorGeometry), POINTER(TensorGeometry), c_void_p,
+                                             c_void_p, c_void_p, c_size_t, c_double, c_double, c_void_p, c_void_p,
+                                             c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "h2x_bn_backward_local_strided": (c_int, [c_int, c_int, c_size_t, POINTER(TensorGeometry), POINTER(TensorGeometry),
+                                              POINTER(TensorGeometry), c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                              c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_double, c_void_p,
+                                              c_void_p]),
     "h2x_bn_batch_normalization_clearing": (c_int, [c_int, POINTER(HaloedGeometry), c_void_p, c_void_p, c_void_p,
                                                     c_void_p, c_void_p, c_void_p, c_double, c_void_p]),
     "h2x_bn_backprop2_clearing": (c_int, [c_int, c_size_t, POINTER(HaloedGeometry), c_void_p, c_void_p, c_void_p,

@@ -79,6 +79,7 @@ struct ScopedLaunchLog
 {
     explicit ScopedLaunchLog(LaunchLog* log) : before(t_launch_log) { t_launch_log = log; }
     ~ScopedLaunchLog() { t_launch_log = before; }
+    void restore() { t_launch_log = before; }
     ScopedLaunchLog(const ScopedLaunchLog&) = delete;
     ScopedLaunchLog& operator=(const ScopedLaunchLog&) = delete;
     LaunchLog* before;
@@ -2359,14 +2360,13 @@ int backprop2_strided(int n, size_t num_per_sum, const h2x_tensor_geometry* gx,
 // Forward pass of a rank that shares its statistics with no one: sums, then a
 // normalising kernel that finishes them itself (2 launches instead of 4).
 template <typename T>
-int forward_local(int n, int c, size_t s, size_t x_real, size_t y_real, const void* x,
+int forward_local(int n, int c, size_t s, const HostTensor& tx, const HostTensor& ty, const void* x,
                   const void* scale, const void* bias, size_t num_per_sum, double decay, double eps,
                   void* mean, void* var, void* running_mean, void* running_var, void* y, void* ws,
                   hipStream_t st)
 {
     if (c == 0)
         return H2X_SUCCESS;
-    const HostTensor tx = dense_tensor<T>(x, c, s, x_real), ty = dense_tensor<T>(y, c, s, y_real);
     if (n == 0 || s == 0 || num_per_sum == 0)
     {
         // nothing to normalise or nothing counted: the staged calls define the result
@@ -2393,6 +2393,16 @@ int forward_local(int n, int c, size_t s, size_t x_real, size_t y_real, const vo
         int err = sums_impl<T>(n, c, s, tx, x, nullptr, nullptr, ws, st, &g);
         if (!err)
             err = apply_impl<T>(n, c, s, tx, ty, x, nullptr, nullptr, scale, bias, y, eps, st, &g);
+        if (err == H2X_ERR_UNSUPPORTED)
+        {
+            // the two tensors take different families of kernels (one of them with halos inside
+            // short segments, say): the staged calls
+            scope.restore();
+            err = sums_impl<T>(n, c, s, tx, x, mean, var, ws, st);
+            if (!err)
+                err = statistics_impl<T>(c, num_per_sum, decay, mean, var, running_mean, running_var, st);
+            return err ? err : apply_impl<T>(n, c, s, tx, ty, x, mean, var, scale, bias, y, eps, st);
+        }
         if (err)
             return err;
     }
@@ -2403,15 +2413,13 @@ int forward_local(int n, int c, size_t s, size_t x_real, size_t y_real, const vo
 // Backward pass likewise: the four sums, then an input-gradient kernel that
 // finishes them itself (2 launches instead of 3).
 template <typename T>
-int backward_local(int n, int c, size_t s, size_t x_real, size_t dy_real, size_t dx_real,
-                   size_t num_per_sum, const void* x, const void* dy, const void* mean,
-                   const void* var, const void* scale, void* dscale, void* dbias, void* dmean,
-                   void* dvar, void* dx, double eps, void* ws, hipStream_t st)
+int backward_local(int n, int c, size_t s, const HostTensor& tx, const HostTensor& td,
+                   const HostTensor& to, size_t num_per_sum, const void* x, const void* dy,
+                   const void* mean, const void* var, const void* scale, void* dscale, void* dbias,
+                   void* dmean, void* dvar, void* dx, double eps, void* ws, hipStream_t st)
 {
     if (c == 0)
         return H2X_SUCCESS;
-    const HostTensor tx = dense_tensor<T>(x, c, s, x_real), td = dense_tensor<T>(dy, c, s, dy_real),
-                     to = dense_tensor<T>(dx, c, s, dx_real);
     if (n == 0 || s == 0)
         return backprop1_impl<T>(n, c, s, tx, td, x, dy, mean, var, scale, dscale, dbias, dmean,
                                  dvar, eps, ws, st); // zeroes the four outputs; no dx to write
@@ -2435,6 +2443,16 @@ int backward_local(int n, int c, size_t s, size_t x_real, size_t dy_real, size_t
         if (!err)
             err = backprop2_impl<T>(n, c, s, num_per_sum, tx, td, to, x, dy, mean, var, scale,
                                     nullptr, nullptr, dx, eps, st, &g);
+        if (err == H2X_ERR_UNSUPPORTED)
+        {
+            // the tensors take different families of kernels: the staged calls
+            scope.restore();
+            err = backprop1_impl<T>(n, c, s, tx, td, x, dy, mean, var, scale, dscale, dbias, dmean,
+                                    dvar, eps, ws, st);
+            return err ? err
+                       : backprop2_impl<T>(n, c, s, num_per_sum, tx, td, to, x, dy, mean, var, scale,
+                                           dmean, dvar, dx, eps, st);
+        }
         if (err)
             return err;
     }
@@ -2443,6 +2461,49 @@ int backward_local(int n, int c, size_t s, size_t x_real, size_t dy_real, size_t
     return err ? err
                : backprop2_impl<T>(n, c, s, num_per_sum, tx, td, to, x, dy, mean, var, scale,
                                    nullptr, nullptr, dx, eps, st, &f);
+}
+
+template <typename T>
+int forward_local_strided(int n, const h2x_tensor_geometry* gx, const h2x_tensor_geometry* gy,
+                          const void* x, const void* scale, const void* bias, size_t num_per_sum,
+                          double decay, double eps, void* mean, void* var, void* running_mean,
+                          void* running_var, void* y, void* ws, hipStream_t st)
+{
+    HostTensor tx, ty;
+    int c, c2;
+    size_t s, s2;
+    int err = strided_tensor<T>(gx, x, n, &tx, &c, &s);
+    if (!err)
+        err = strided_tensor<T>(gy, y, n, &ty, &c2, &s2);
+    if (!err && (c != c2 || s != s2 || !same_local_shape(gx, gy)))
+        err = H2X_ERR_INVALID_ARGUMENT;
+    return err ? err
+               : forward_local<T>(n, c, s, tx, ty, x, scale, bias, num_per_sum, decay, eps, mean, var,
+                                  running_mean, running_var, y, ws, st);
+}
+
+template <typename T>
+int backward_local_strided(int n, size_t num_per_sum, const h2x_tensor_geometry* gx,
+                           const h2x_tensor_geometry* gd, const h2x_tensor_geometry* go,
+                           const void* x, const void* dy, const void* mean, const void* var,
+                           const void* scale, void* dscale, void* dbias, void* dmean, void* dvar,
+                           void* dx, double eps, void* ws, hipStream_t st)
+{
+    HostTensor tx, td, to;
+    int c, c2, c3;
+    size_t s, s2, s3;
+    int err = strided_tensor<T>(gx, x, n, &tx, &c, &s);
+    if (!err)
+        err = strided_tensor<T>(gd, dy, n, &td, &c2, &s2);
+    if (!err)
+        err = strided_tensor<T>(go, dx, n, &to, &c3, &s3);
+    if (!err
+        && (c != c2 || s != s2 || c != c3 || s != s3 || !same_local_shape(gx, gd)
+            || !same_local_shape(gx, go)))
+        err = H2X_ERR_INVALID_ARGUMENT;
+    return err ? err
+               : backward_local<T>(n, c, s, tx, td, to, num_per_sum, x, dy, mean, var, scale, dscale,
+                                   dbias, dmean, dvar, dx, eps, ws, st);
 }
 
 } // namespace
@@ -2733,14 +2794,38 @@ extern "C" int h2x_bn_forward_local(h2x_dtype dtype, int num_samples, int num_ch
     if ((!x || !y) && static_cast<size_t>(num_samples) * num_channels * spatial_size > 0)
         return H2X_ERR_INVALID_ARGUMENT;
     H2X_BY_DTYPE(dtype,
-                 forward_local<float>(num_samples, num_channels, spatial_size, x_spatial_real_size,
-                                      y_spatial_real_size, x, scale, bias, num_per_sum, decay,
-                                      epsilon, mean, var, running_mean, running_var, y, workspace,
-                                      as_stream(stream)),
-                 forward_local<double>(num_samples, num_channels, spatial_size, x_spatial_real_size,
-                                       y_spatial_real_size, x, scale, bias, num_per_sum, decay,
-                                       epsilon, mean, var, running_mean, running_var, y, workspace,
-                                       as_stream(stream)));
+                 forward_local<float>(
+                     num_samples, num_channels, spatial_size,
+                     dense_tensor<float>(x, num_channels, spatial_size, x_spatial_real_size),
+                     dense_tensor<float>(y, num_channels, spatial_size, y_spatial_real_size), x, scale,
+                     bias, num_per_sum, decay, epsilon, mean, var, running_mean, running_var, y,
+                     workspace, as_stream(stream)),
+                 forward_local<double>(
+                     num_samples, num_channels, spatial_size,
+                     dense_tensor<double>(x, num_channels, spatial_size, x_spatial_real_size),
+                     dense_tensor<double>(y, num_channels, spatial_size, y_spatial_real_size), x, scale,
+                     bias, num_per_sum, decay, epsilon, mean, var, running_mean, running_var, y,
+                     workspace, as_stream(stream)));
+}
+
+extern "C" int h2x_bn_forward_local_strided(h2x_dtype dtype, int num_samples,
+                                            const h2x_tensor_geometry* x_geometry,
+                                            const h2x_tensor_geometry* y_geometry, const void* x,
+                                            const void* scale, const void* bias, size_t num_per_sum,
+                                            double decay, double epsilon, void* mean, void* var,
+                                            void* running_mean, void* running_var, void* y,
+                                            void* workspace, h2x_stream_t stream)
+{
+    if (num_samples < 0 || !x_geometry || !y_geometry || !scale || !bias || !mean || !var
+        || !running_mean || !running_var || !workspace)
+        return H2X_ERR_INVALID_ARGUMENT;
+    H2X_BY_DTYPE(dtype,
+                 forward_local_strided<float>(num_samples, x_geometry, y_geometry, x, scale, bias,
+                                              num_per_sum, decay, epsilon, mean, var, running_mean,
+                                              running_var, y, workspace, as_stream(stream)),
+                 forward_local_strided<double>(num_samples, x_geometry, y_geometry, x, scale, bias,
+                                               num_per_sum, decay, epsilon, mean, var, running_mean,
+                                               running_var, y, workspace, as_stream(stream)));
 }
 
 extern "C" int h2x_bn_backward_local(h2x_dtype dtype, int num_samples, int num_channels,
@@ -2758,13 +2843,40 @@ extern "C" int h2x_bn_backward_local(h2x_dtype dtype, int num_samples, int num_c
     if ((!x || !dy || !dx) && static_cast<size_t>(num_samples) * num_channels * spatial_size > 0)
         return H2X_ERR_INVALID_ARGUMENT;
     H2X_BY_DTYPE(dtype,
-                 backward_local<float>(num_samples, num_channels, spatial_size, x_spatial_real_size,
-                                       dy_spatial_real_size, dx_spatial_real_size, num_per_sum, x,
-                                       dy, mean, var, scale, dscale, dbias, dmean, dvar, dx, epsilon,
-                                       workspace, as_stream(stream)),
-                 backward_local<double>(num_samples, num_channels, spatial_size,
-                                        x_spatial_real_size, dy_spatial_real_size,
-                                        dx_spatial_real_size, num_per_sum, x, dy, mean, var, scale,
-                                        dscale, dbias, dmean, dvar, dx, epsilon, workspace,
-                                        as_stream(stream)));
+                 backward_local<float>(
+                     num_samples, num_channels, spatial_size,
+                     dense_tensor<float>(x, num_channels, spatial_size, x_spatial_real_size),
+                     dense_tensor<float>(dy, num_channels, spatial_size, dy_spatial_real_size),
+                     dense_tensor<float>(dx, num_channels, spatial_size, dx_spatial_real_size),
+                     num_per_sum, x, dy, mean, var, scale, dscale, dbias, dmean, dvar, dx, epsilon,
+                     workspace, as_stream(stream)),
+                 backward_local<double>(
+                     num_samples, num_channels, spatial_size,
+                     dense_tensor<double>(x, num_channels, spatial_size, x_spatial_real_size),
+                     dense_tensor<double>(dy, num_channels, spatial_size, dy_spatial_real_size),
+                     dense_tensor<double>(dx, num_channels, spatial_size, dx_spatial_real_size),
+                     num_per_sum, x, dy, mean, var, scale, dscale, dbias, dmean, dvar, dx, epsilon,
+                     workspace, as_stream(stream)));
+}
+
+extern "C" int h2x_bn_backward_local_strided(h2x_dtype dtype, int num_samples, size_t num_per_sum,
+                                             const h2x_tensor_geometry* x_geometry,
+                                             const h2x_tensor_geometry* dy_geometry,
+                                             const h2x_tensor_geometry* dx_geometry, const void* x,
+                                             const void* dy, const void* mean, const void* var,
+                                             const void* scale, void* dscale, void* dbias,
+                                             void* dmean, void* dvar, void* dx, double epsilon,
+                                             void* workspace, h2x_stream_t stream)
+{
+    if (num_samples < 0 || !x_geometry || !dy_geometry || !dx_geometry || !mean || !var || !scale
+        || !dscale || !dbias || !dmean || !dvar || !workspace)
+        return H2X_ERR_INVALID_ARGUMENT;
+    H2X_BY_DTYPE(dtype,
+                 backward_local_strided<float>(num_samples, num_per_sum, x_geometry, dy_geometry,
+                                               dx_geometry, x, dy, mean, var, scale, dscale, dbias,
+                                               dmean, dvar, dx, epsilon, workspace, as_stream(stream)),
+                 backward_local_strided<double>(num_samples, num_per_sum, x_geometry, dy_geometry,
+                                                dx_geometry, x, dy, mean, var, scale, dscale, dbias,
+                                                dmean, dvar, dx, epsilon, workspace,
+                                                as_stream(stream)));
 }

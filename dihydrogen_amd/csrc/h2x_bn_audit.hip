@@ -307,6 +307,10 @@ extern "C" int h2x_bn_audit(h2x_bn_stage stage, h2x_dtype dtype, int num_samples
         if (dense(0, &c, &s, &xr) && dense(1, &c2, &s2, &yr) && c == c2 && s == s2)
             err = h2x_bn_forward_local(dtype, num_samples, c, s, xr, yr, ptr(0), param, param, 2, 0.9,
                                        1e-5, param, param, param, param, ptr(1), param, nullptr);
+        else
+            err = h2x_bn_forward_local_strided(dtype, num_samples, geometry[0], geometry[1], ptr(0), param,
+                                               param, 2, 0.9, 1e-5, param, param, param, param, ptr(1),
+                                               param, nullptr);
         break;
     }
     case H2X_BN_STAGE_BACKWARD_LOCAL:
@@ -318,6 +322,10 @@ extern "C" int h2x_bn_audit(h2x_bn_stage stage, h2x_dtype dtype, int num_samples
             err = h2x_bn_backward_local(dtype, num_samples, c, s, xr, dr, orl, 2, ptr(0), ptr(1), param,
                                         param, param, param, param, param, param, ptr(2), 1e-5,
                                         param, nullptr);
+        else
+            err = h2x_bn_backward_local_strided(dtype, num_samples, 2, geometry[0], geometry[1], geometry[2],
+                                                ptr(0), ptr(1), param, param, param, param, param, param,
+                                                param, ptr(2), 1e-5, param, nullptr);
         break;
     }
     }

@@ -421,18 +421,32 @@ public:
     int forward(const Tensor& input, Tensor& mean, Tensor& var, Tensor& running_mean,
                 Tensor& running_var, Tensor& scale, Tensor& bias, Tensor& output, bool is_training)
     {
-        if (is_training && runs_local(input) && batchnorm::is_dense(input)
-            && batchnorm::is_dense(output) && !wants_clearing(input) && !wants_clearing(output))
+        if (is_training && runs_local(input) && !wants_clearing(input) && !wants_clearing(output))
         {
             set_num_samples(static_cast<int>(input.get_local_shape()[-1]));
             const batchnorm::ChannelGeometry<Tensor> gi(input), go(output);
-            DISTCONV_CHECK_H2X(h2x_bn_forward_local(
-                Tensor::h2x_type(), m_num_current_samples, gi.num_channels, gi.spatial,
-                gi.spatial_real, go.spatial_real, input.get_const_base_ptr(),
-                scale.get_const_base_ptr(), bias.get_const_base_ptr(), num_per_sum(input), m_decay,
-                m_epsilon, mean.get_base_ptr(), var.get_base_ptr(), running_mean.get_base_ptr(),
-                running_var.get_base_ptr(), output.get_base_ptr(), m_ws.get(gi.num_channels),
-                m_stream));
+            if (batchnorm::is_dense(input) && batchnorm::is_dense(output))
+            {
+                DISTCONV_CHECK_H2X(h2x_bn_forward_local(
+                    Tensor::h2x_type(), m_num_current_samples, gi.num_channels, gi.spatial,
+                    gi.spatial_real, go.spatial_real, input.get_const_base_ptr(),
+                    scale.get_const_base_ptr(), bias.get_const_base_ptr(), num_per_sum(input),
+                    m_decay, m_epsilon, mean.get_base_ptr(), var.get_base_ptr(),
+                    running_mean.get_base_ptr(), running_var.get_base_ptr(), output.get_base_ptr(),
+                    m_ws.get(gi.num_channels), m_stream));
+            }
+            else
+            {
+                // tensors with halos on inner dimensions: the same two launches through the strides
+                const h2x_tensor_geometry gx = batchnorm::tensor_geometry(input, m_num_current_samples),
+                                          gy = batchnorm::tensor_geometry(output, m_num_current_samples);
+                DISTCONV_CHECK_H2X(h2x_bn_forward_local_strided(
+                    Tensor::h2x_type(), m_num_current_samples, &gx, &gy, input.get_const_base_ptr(),
+                    scale.get_const_base_ptr(), bias.get_const_base_ptr(), num_per_sum(input),
+                    m_decay, m_epsilon, mean.get_base_ptr(), var.get_base_ptr(),
+                    running_mean.get_base_ptr(), running_var.get_base_ptr(), output.get_base_ptr(),
+                    m_ws.get(gi.num_channels), m_stream));
+            }
             return 0;
         }
         forward_stage1(input, mean, var, is_training);
@@ -490,19 +504,36 @@ public:
                  const Tensor& scale, Tensor& scale_gradient, Tensor& bias_gradient,
                  Tensor& mean_gradient, Tensor& var_gradient, Tensor& d_input)
     {
-        if (runs_local(input) && batchnorm::is_dense(input) && batchnorm::is_dense(d_output)
-            && batchnorm::is_dense(d_input) && !wants_clearing(input) && !wants_clearing(d_input))
+        if (runs_local(input) && !wants_clearing(input) && !wants_clearing(d_input))
         {
             set_num_samples(static_cast<int>(input.get_local_shape()[-1]));
             const batchnorm::ChannelGeometry<Tensor> gi(input), go(d_output), gd(d_input);
-            DISTCONV_CHECK_H2X(h2x_bn_backward_local(
-                Tensor::h2x_type(), m_num_current_samples, gi.num_channels, gi.spatial,
-                gi.spatial_real, go.spatial_real, gd.spatial_real, num_per_sum(input),
-                input.get_const_base_ptr(), d_output.get_const_base_ptr(),
-                mean.get_const_base_ptr(), var.get_const_base_ptr(), scale.get_const_base_ptr(),
-                scale_gradient.get_base_ptr(), bias_gradient.get_base_ptr(),
-                mean_gradient.get_base_ptr(), var_gradient.get_base_ptr(), d_input.get_base_ptr(),
-                m_epsilon, m_ws.get(gi.num_channels), m_stream));
+            if (batchnorm::is_dense(input) && batchnorm::is_dense(d_output)
+                && batchnorm::is_dense(d_input))
+            {
+                DISTCONV_CHECK_H2X(h2x_bn_backward_local(
+                    Tensor::h2x_type(), m_num_current_samples, gi.num_channels, gi.spatial,
+                    gi.spatial_real, go.spatial_real, gd.spatial_real, num_per_sum(input),
+                    input.get_const_base_ptr(), d_output.get_const_base_ptr(),
+                    mean.get_const_base_ptr(), var.get_const_base_ptr(), scale.get_const_base_ptr(),
+                    scale_gradient.get_base_ptr(), bias_gradient.get_base_ptr(),
+                    mean_gradient.get_base_ptr(), var_gradient.get_base_ptr(),
+                    d_input.get_base_ptr(), m_epsilon, m_ws.get(gi.num_channels), m_stream));
+            }
+            else
+            {
+                const int ns = m_num_current_samples;
+                const h2x_tensor_geometry gx = batchnorm::tensor_geometry(input, ns),
+                                          gy = batchnorm::tensor_geometry(d_output, ns),
+                                          gz = batchnorm::tensor_geometry(d_input, ns);
+                DISTCONV_CHECK_H2X(h2x_bn_backward_local_strided(
+                    Tensor::h2x_type(), ns, num_per_sum(input), &gx, &gy, &gz,
+                    input.get_const_base_ptr(), d_output.get_const_base_ptr(),
+                    mean.get_const_base_ptr(), var.get_const_base_ptr(), scale.get_const_base_ptr(),
+                    scale_gradient.get_base_ptr(), bias_gradient.get_base_ptr(),
+                    mean_gradient.get_base_ptr(), var_gradient.get_base_ptr(),
+                    d_input.get_base_ptr(), m_epsilon, m_ws.get(gi.num_channels), m_stream));
+            }
             return 0;
         }
         backward_stage1(input, d_output, mean, var, scale, scale_gradient, bias_gradient,

@@ -197,10 +197,10 @@ class BatchNormalization:
         return 0
 
     def _runs_local(self, *tensors: Tensor) -> bool:
-        """No all-reduce between the stages, dense tensors, a rank that owns elements."""
+        """No all-reduce between the stages, a rank that owns elements (and no halo to clear)."""
         t0 = tensors[0]
         return (self.fuse_local and not (self.global_stats and self.allreduce is not None)
-                and all(_is_dense(t) for t in tensors) and t0.is_split_root() and t0.get_local_size() > 0
+                and t0.is_split_root() and t0.get_local_size() > 0
                 and not (self.clear_output_halo and any(any(t.overlap) for t in tensors)))
 
     def forward(self, input, mean, var, running_mean, running_var, scale, bias, output,
@@ -209,11 +209,20 @@ class BatchNormalization:
             self.set_num_samples(input.local_shape[-1])
             n, c, s, sr = _channel_geometry(input)
             _, _, _, sro = _channel_geometry(output)
-            capi.check(self._lib.h2x_bn_forward_local(
-                input.h2x_dtype, self.num_current_samples, c, s, sr, sro, _ptr(input.get_base_ptr()),
-                _ptr(scale), _ptr(bias), self._num_per_sum(input), self.decay, self.epsilon, _ptr(mean),
-                _ptr(var), _ptr(running_mean), _ptr(running_var), _ptr(output.get_base_ptr()),
-                _ptr(self._ws(c)), _stream_handle(self.stream)), "bn forward (local)")
+            if _is_dense(input) and _is_dense(output):
+                capi.check(self._lib.h2x_bn_forward_local(
+                    input.h2x_dtype, self.num_current_samples, c, s, sr, sro, _ptr(input.get_base_ptr()),
+                    _ptr(scale), _ptr(bias), self._num_per_sum(input), self.decay, self.epsilon, _ptr(mean),
+                    _ptr(var), _ptr(running_mean), _ptr(running_var), _ptr(output.get_base_ptr()),
+                    _ptr(self._ws(c)), _stream_handle(self.stream)), "bn forward (local)")
+            else:
+                ns = self.num_current_samples
+                gx, gy = _tensor_geometry(input, ns), _tensor_geometry(output, ns)
+                capi.check(self._lib.h2x_bn_forward_local_strided(
+                    input.h2x_dtype, ns, ctypes.byref(gx), ctypes.byref(gy), _ptr(input.get_base_ptr()),
+                    _ptr(scale), _ptr(bias), self._num_per_sum(input), self.decay, self.epsilon, _ptr(mean),
+                    _ptr(var), _ptr(running_mean), _ptr(running_var), _ptr(output.get_base_ptr()),
+                    _ptr(self._ws(c)), _stream_handle(self.stream)), "bn forward (local, strided)")
             return 0
         self.forward_stage1(input, mean, var, is_training)
         self.forward_allreduce(mean, var, is_training)
@@ -286,12 +295,20 @@ class BatchNormalization:
             n, c, s, sr = _channel_geometry(input)
             _, _, _, sro = _channel_geometry(d_output)
             _, _, _, sri = _channel_geometry(d_input)
-            capi.check(self._lib.h2x_bn_backward_local(
-                input.h2x_dtype, self.num_current_samples, c, s, sr, sro, sri, self._num_per_sum(input),
-                _ptr(input.get_base_ptr()), _ptr(d_output.get_base_ptr()), _ptr(mean), _ptr(var),
-                _ptr(scale), _ptr(scale_gradient), _ptr(bias_gradient), _ptr(mean_gradient),
-                _ptr(var_gradient), _ptr(d_input.get_base_ptr()), self.epsilon, _ptr(self._ws(c)),
-                _stream_handle(self.stream)), "bn backward (local)")
+            tail = (_ptr(input.get_base_ptr()), _ptr(d_output.get_base_ptr()), _ptr(mean), _ptr(var),
+                    _ptr(scale), _ptr(scale_gradient), _ptr(bias_gradient), _ptr(mean_gradient),
+                    _ptr(var_gradient), _ptr(d_input.get_base_ptr()), self.epsilon, _ptr(self._ws(c)),
+                    _stream_handle(self.stream))
+            if _is_dense(input) and _is_dense(d_output) and _is_dense(d_input):
+                capi.check(self._lib.h2x_bn_backward_local(
+                    input.h2x_dtype, self.num_current_samples, c, s, sr, sro, sri, self._num_per_sum(input),
+                    *tail), "bn backward (local)")
+            else:
+                ns = self.num_current_samples
+                gx, gd, gi = (_tensor_geometry(t, ns) for t in (input, d_output, d_input))
+                capi.check(self._lib.h2x_bn_backward_local_strided(
+                    input.h2x_dtype, ns, self._num_per_sum(input), ctypes.byref(gx), ctypes.byref(gd),
+                    ctypes.byref(gi), *tail), "bn backward (local, strided)")
             return 0
         self.backward_stage1(input, d_output, mean, var, scale, scale_gradient, bias_gradient,
                              mean_gradient, var_gradient)

@@ -377,6 +377,50 @@ int h2x_bn_backprop2_strided(h2x_dtype dtype,
                              h2x_stream_t stream);
 
 /**
+ * h2x_bn_forward_local and h2x_bn_backward_local for tensors given by shape
+ * and strides (haloed shards): the same two launches, the same bits as the
+ * staged _strided calls.  Where the tensors of a call take different families
+ * of kernels (a haloed tensor with short segments beside a dense one), the
+ * staged calls run instead, with the same results.
+ */
+int h2x_bn_forward_local_strided(h2x_dtype dtype,
+                                 int num_samples,
+                                 const h2x_tensor_geometry* x_geometry,
+                                 const h2x_tensor_geometry* y_geometry,
+                                 const void* x,
+                                 const void* scale,
+                                 const void* bias,
+                                 size_t num_per_sum,
+                                 double decay,
+                                 double epsilon,
+                                 void* mean,
+                                 void* var,
+                                 void* running_mean,
+                                 void* running_var,
+                                 void* y,
+                                 void* workspace,
+                                 h2x_stream_t stream);
+int h2x_bn_backward_local_strided(h2x_dtype dtype,
+                                  int num_samples,
+                                  size_t num_per_sum,
+                                  const h2x_tensor_geometry* x_geometry,
+                                  const h2x_tensor_geometry* dy_geometry,
+                                  const h2x_tensor_geometry* dx_geometry,
+                                  const void* x,
+                                  const void* dy,
+                                  const void* mean,
+                                  const void* var,
+                                  const void* scale,
+                                  void* dscale,
+                                  void* dbias,
+                                  void* dmean,
+                                  void* dvar,
+                                  void* dx,
+                                  double epsilon,
+                                  void* workspace,
+                                  h2x_stream_t stream);
+
+/**
  * The local part of a haloed tensor as it lies in memory: the real (allocated)
  * extents and where the interior starts in them.  Innermost first; the last
  * two dimensions are channel and sample and carry no halo; num_dims is 3, 4
@@ -451,9 +495,9 @@ int h2x_bn_backprop2_clearing(h2x_dtype dtype,
  * 0; a reduction would add them twice).  Owning an element means adding it
  * into a sum or storing its result; elements that two overlapping vectors
  * share are loaded, and where allowed stored, by both but owned by one.
- * The two-launch stages take dense tensors only: geometries of three
- * dimensions {spatial, channels, samples} with strides {1, real, real *
- * channels}.  Returns what the entry point returns; H2X_ERR_TOO_LARGE if it
+ * The two-launch stages go through h2x_bn_forward_local / _backward_local for
+ * geometries of three dimensions {spatial, channels, samples} with strides
+ * {1, real, real * channels}, through their _strided twins otherwise.  Returns what the entry point returns; H2X_ERR_TOO_LARGE if it
  * plans more than H2X_BN_AUDIT_MAX_LAUNCHES launches.  Cost: proportional to
  * the elements of the tensors; meant for tests.
  */
@@ -463,8 +507,8 @@ typedef enum h2x_bn_stage
     H2X_BN_STAGE_NORMALIZE = 1,     /* h2x_bn_batch_normalization_strided */
     H2X_BN_STAGE_BACKPROP1 = 2,     /* h2x_bn_backprop1_strided */
     H2X_BN_STAGE_BACKPROP2 = 3,     /* h2x_bn_backprop2_strided */
-    H2X_BN_STAGE_FORWARD_LOCAL = 4, /* h2x_bn_forward_local */
-    H2X_BN_STAGE_BACKWARD_LOCAL = 5 /* h2x_bn_backward_local */
+    H2X_BN_STAGE_FORWARD_LOCAL = 4, /* h2x_bn_forward_local(_strided) */
+    H2X_BN_STAGE_BACKWARD_LOCAL = 5 /* h2x_bn_backward_local(_strided) */
 } h2x_bn_stage;
 
 #define H2X_BN_AUDIT_MAX_LAUNCHES 8

@@ -513,6 +513,49 @@ def test_clearing_input_gradient_in_place():
     assert np.array_equal(outs[0], outs[1])
 
 
+@pytest.mark.parametrize("case", HALO_CASES)
+def test_two_launch_calls_on_haloed_tensors_equal_the_staged_calls(case):
+    """forward()/backward() on tensors with halos on inner dimensions take
+    h2x_bn_forward_local_strided / _backward_local_strided (two launches each): every
+    output equals the staged calls' bit for bit, halo cells stay untouched."""
+    import torch
+    from dihydrogen_amd.layers import BatchNormalization
+    from dihydrogen_amd.tensor import Distribution, LocaleVirtual, Tensor
+    gshape, locale, overlap = case
+    nd = len(gshape)
+    nranks = int(np.prod(locale))
+    dist = Distribution.make_overlapped_distribution(locale, overlap)
+    dist_dy = Distribution.make_distribution(locale)
+    c = gshape[nd - 2]
+    g = torch.Generator(device="cuda").manual_seed(41)
+    scale = torch.empty(c, device="cuda").uniform_(0.5, 1.5, generator=g)
+    bias = torch.empty(c, device="cuda").normal_(0, 0.1, generator=g)
+    for r in range(nranks):
+        loc = LocaleVirtual(r, nranks)
+        xi = di = None
+        results = []
+        for fuse in (True, False):
+            x, y, dx = (Tensor(gshape, loc, dist).allocate() for _ in range(3))
+            dy = Tensor(gshape, loc, dist_dy).allocate()
+            for t in (x, y, dx):
+                t.real_view().fill_(float("nan"))
+            if xi is None:
+                xi = torch.empty_like(x.interior_view()).normal_(0, 1, generator=g)
+                di = torch.empty_like(dy.interior_view()).normal_(0, 1, generator=g)
+            x.interior_view().copy_(xi)
+            dy.interior_view().copy_(di)
+            vec = lambda v: torch.full((c,), v, device="cuda")
+            mean, var, rm, rv = vec(float("nan")), vec(float("nan")), vec(0.25), vec(0.75)
+            grads = [vec(float("nan")) for _ in range(4)]
+            bn = BatchNormalization(nd, 0.9, 1e-5, fuse_local=fuse)
+            assert bn.forward(x, mean, var, rm, rv, scale, bias, y, True) == 0
+            assert bn.backward(x, dy, mean, var, scale, *grads, dx) == 0
+            torch.cuda.synchronize()
+            results.append([t.cpu().numpy() for t in (mean, var, rm, rv, y.real_view(), *grads, dx.real_view())])
+        for a, b in zip(*results):
+            assert np.array_equal(a, b, equal_nan=True)
+
+
 def test_non_finite_inputs_propagate_as_in_the_oracle(oracle_mod):
     """A NaN, an infinity, values near the float32 maximum (whose squares overflow
     float32 but not the float64 accumulators) and denormals, each in a channel of
