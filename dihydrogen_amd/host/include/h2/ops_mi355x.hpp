@@ -225,6 +225,66 @@ void batchnorm_backprop2_impl(GPUDev_t, const Tensor<T>& x, const Tensor<T>& dy,
                   "batchnorm_backprop2");
 }
 
+// The local forward pass in two launches: sums of x and of x^2, then a kernel
+// that turns them into mean / unbiased variance / running statistics and
+// normalises.  Same bits as channel_sums + statistics + normalize, one
+// statistics launch and two reads of the partial sums fewer
+// (what BatchNormalization::forward does between its allreduces when there is
+// one process, legacy/include/distconv/dnn_backend/batchnorm.hpp:294-334).
+template <typename T>
+void batchnorm_forward_impl(GPUDev_t, const Tensor<T>& x, const Tensor<T>& scale,
+                            const Tensor<T>& bias, Tensor<T>& mean, Tensor<T>& var,
+                            Tensor<T>& running_mean, Tensor<T>& running_var, Tensor<T>& y,
+                            std::size_t num_per_sum, double decay, double epsilon)
+{
+    mi355x::require_same(x, y, "batchnorm_forward");
+    const h2x_tensor_geometry gx = mi355x::channel_geometry(x, "batchnorm_forward");
+    const h2x_tensor_geometry gy = mi355x::channel_geometry(y, "batchnorm_forward");
+    const DimType c = static_cast<DimType>(gx.local_shape[gx.num_dims - 2]);
+    for (const BaseTensor* t :
+         {static_cast<const BaseTensor*>(&scale), static_cast<const BaseTensor*>(&bias),
+          static_cast<const BaseTensor*>(&mean), static_cast<const BaseTensor*>(&var),
+          static_cast<const BaseTensor*>(&running_mean), static_cast<const BaseTensor*>(&running_var)})
+        mi355x::require_channel_vector(*t, c, "batchnorm_forward");
+    hipStream_t s = mi355x::gpu_stream(x);
+    mi355x::check(h2x_bn_forward_local_strided(
+                      mi355x::dtype_of<T>(), static_cast<int>(gx.local_shape[gx.num_dims - 1]), &gx,
+                      &gy, x.const_data(), scale.const_data(), bias.const_data(), num_per_sum, decay,
+                      epsilon, mean.data(), var.data(), running_mean.data(), running_var.data(),
+                      y.data(), mi355x::bn_workspace(s, c), s),
+                  "batchnorm_forward");
+}
+
+// The local backward pass in two launches: the four sums, then a kernel that
+// adds them and writes dx.  Same bits as backprop1 + backprop2; dx may be x
+// (legacy/include/distconv/dnn_backend/batchnorm.hpp:433-470 with one process).
+template <typename T>
+void batchnorm_backward_impl(GPUDev_t, const Tensor<T>& x, const Tensor<T>& dy,
+                             const Tensor<T>& mean, const Tensor<T>& var, const Tensor<T>& scale,
+                             Tensor<T>& dscale, Tensor<T>& dbias, Tensor<T>& dmean, Tensor<T>& dvar,
+                             Tensor<T>& dx, std::size_t num_per_sum, double epsilon)
+{
+    mi355x::require_same(x, dy, "batchnorm_backward");
+    mi355x::require_same(x, dx, "batchnorm_backward");
+    const h2x_tensor_geometry gx = mi355x::channel_geometry(x, "batchnorm_backward");
+    const h2x_tensor_geometry gd = mi355x::channel_geometry(dy, "batchnorm_backward");
+    const h2x_tensor_geometry go = mi355x::channel_geometry(dx, "batchnorm_backward");
+    const DimType c = static_cast<DimType>(gx.local_shape[gx.num_dims - 2]);
+    for (const BaseTensor* t :
+         {static_cast<const BaseTensor*>(&mean), static_cast<const BaseTensor*>(&var),
+          static_cast<const BaseTensor*>(&scale), static_cast<const BaseTensor*>(&dscale),
+          static_cast<const BaseTensor*>(&dbias), static_cast<const BaseTensor*>(&dmean),
+          static_cast<const BaseTensor*>(&dvar)})
+        mi355x::require_channel_vector(*t, c, "batchnorm_backward");
+    hipStream_t s = mi355x::gpu_stream(x);
+    mi355x::check(h2x_bn_backward_local_strided(
+                      mi355x::dtype_of<T>(), static_cast<int>(gx.local_shape[gx.num_dims - 1]),
+                      num_per_sum, &gx, &gd, &go, x.const_data(), dy.const_data(), mean.const_data(),
+                      var.const_data(), scale.const_data(), dscale.data(), dbias.data(), dmean.data(),
+                      dvar.data(), dx.data(), epsilon, mi355x::bn_workspace(s, c), s),
+                  "batchnorm_backward");
+}
+
 // softmax over the Channel dimension (legacy/src/dnn_backend/softmax.cu:538-619)
 template <typename T>
 void softmax_channel_forward_impl(GPUDev_t, const Tensor<T>& x, Tensor<T>& y)
@@ -342,6 +402,26 @@ void batchnorm_backprop2(const Tensor<T>& x, const Tensor<T>& dy, const Tensor<T
                                                    dmean, dvar, dx, num_per_sum, epsilon));
 }
 template <typename T>
+void batchnorm_forward(const Tensor<T>& x, const Tensor<T>& scale, const Tensor<T>& bias,
+                       Tensor<T>& mean, Tensor<T>& var, Tensor<T>& running_mean,
+                       Tensor<T>& running_var, Tensor<T>& y, std::size_t num_per_sum, double decay,
+                       double epsilon)
+{
+    H2X_GPU_ONLY(x, impl::batchnorm_forward_impl(DeviceT_v<Device::GPU>, x, scale, bias, mean, var,
+                                                 running_mean, running_var, y, num_per_sum, decay,
+                                                 epsilon));
+}
+template <typename T>
+void batchnorm_backward(const Tensor<T>& x, const Tensor<T>& dy, const Tensor<T>& mean,
+                        const Tensor<T>& var, const Tensor<T>& scale, Tensor<T>& dscale,
+                        Tensor<T>& dbias, Tensor<T>& dmean, Tensor<T>& dvar, Tensor<T>& dx,
+                        std::size_t num_per_sum, double epsilon)
+{
+    H2X_GPU_ONLY(x, impl::batchnorm_backward_impl(DeviceT_v<Device::GPU>, x, dy, mean, var, scale,
+                                                  dscale, dbias, dmean, dvar, dx, num_per_sum,
+                                                  epsilon));
+}
+template <typename T>
 void softmax_channel_forward(const Tensor<T>& x, Tensor<T>& y)
 {
     H2X_GPU_ONLY(x, impl::softmax_channel_forward_impl(DeviceT_v<Device::GPU>, x, y));
@@ -428,6 +508,21 @@ struct Erased
         batchnorm_backprop2(as<T>(x), as<T>(dy), as<T>(mean), as<T>(var), as<T>(scale), as<T>(dmean),
                             as<T>(dvar), as<T>(dx), num_per_sum, epsilon);
     }
+    static void forward(const BaseTensor& x, const BaseTensor& scale, const BaseTensor& bias,
+                        BaseTensor& mean, BaseTensor& var, BaseTensor& rm, BaseTensor& rv,
+                        BaseTensor& y, std::size_t num_per_sum, double decay, double epsilon)
+    {
+        batchnorm_forward(as<T>(x), as<T>(scale), as<T>(bias), as<T>(mean), as<T>(var), as<T>(rm),
+                          as<T>(rv), as<T>(y), num_per_sum, decay, epsilon);
+    }
+    static void backward(const BaseTensor& x, const BaseTensor& dy, const BaseTensor& mean,
+                         const BaseTensor& var, const BaseTensor& scale, BaseTensor& dscale,
+                         BaseTensor& dbias, BaseTensor& dmean, BaseTensor& dvar, BaseTensor& dx,
+                         std::size_t num_per_sum, double epsilon)
+    {
+        batchnorm_backward(as<T>(x), as<T>(dy), as<T>(mean), as<T>(var), as<T>(scale), as<T>(dscale),
+                           as<T>(dbias), as<T>(dmean), as<T>(dvar), as<T>(dx), num_per_sum, epsilon);
+    }
     static void softmax_forward(const BaseTensor& x, BaseTensor& y)
     {
         softmax_channel_forward(as<T>(x), as<T>(y));
@@ -486,6 +581,8 @@ void register_type()
     dispatch_register("batchnorm_normalize_gpu", key, &Erased<T>::normalize);
     dispatch_register("batchnorm_backprop1_gpu", key, &Erased<T>::backprop1);
     dispatch_register("batchnorm_backprop2_gpu", key, &Erased<T>::backprop2);
+    dispatch_register("batchnorm_forward_gpu", key, &Erased<T>::forward);
+    dispatch_register("batchnorm_backward_gpu", key, &Erased<T>::backward);
     dispatch_register("softmax_channel_forward_gpu", key, &Erased<T>::softmax_forward);
     dispatch_register("softmax_channel_backward_gpu", key, &Erased<T>::softmax_backward);
     dispatch_register("halo_pack_or_unpack_gpu", key, &Erased<T>::halo);
@@ -552,6 +649,22 @@ inline void batchnorm_backprop2(const BaseTensor& x, const BaseTensor& dy, const
 {
     mi355x::dispatch("batchnorm_backprop2_gpu", x, x, dy, mean, var, scale, dmean, dvar, dx,
                      num_per_sum, epsilon);
+}
+inline void batchnorm_forward(const BaseTensor& x, const BaseTensor& scale, const BaseTensor& bias,
+                              BaseTensor& mean, BaseTensor& var, BaseTensor& running_mean,
+                              BaseTensor& running_var, BaseTensor& y, std::size_t num_per_sum,
+                              double decay, double epsilon)
+{
+    mi355x::dispatch("batchnorm_forward_gpu", x, x, scale, bias, mean, var, running_mean, running_var,
+                     y, num_per_sum, decay, epsilon);
+}
+inline void batchnorm_backward(const BaseTensor& x, const BaseTensor& dy, const BaseTensor& mean,
+                               const BaseTensor& var, const BaseTensor& scale, BaseTensor& dscale,
+                               BaseTensor& dbias, BaseTensor& dmean, BaseTensor& dvar, BaseTensor& dx,
+                               std::size_t num_per_sum, double epsilon)
+{
+    mi355x::dispatch("batchnorm_backward_gpu", x, x, dy, mean, var, scale, dscale, dbias, dmean, dvar,
+                     dx, num_per_sum, epsilon);
 }
 inline void softmax_channel_forward(const BaseTensor& x, BaseTensor& y)
 {

@@ -193,6 +193,28 @@ static void test_batchnorm(const ShapeTuple& shape)
     Tensor<float> y2(Device::GPU, shape, types, stream);
     batchnorm_normalize(x, mean, var, scale, bias, y2, 1e-5);
     CHECK(download(y2) == download(y));
+
+    // the two-launch operators give the bits of the staged ones, dx in place included
+    Tensor<float> mean2 = cvec(), var2 = cvec(), rm2 = cvec(), rv2 = cvec(), dscale2 = cvec(),
+                  dbias2 = cvec(), dmean2 = cvec(), dvar2 = cvec();
+    Tensor<float> y3(Device::GPU, shape, types, stream), xc(Device::GPU, shape, types, stream);
+    upload(rm2, std::vector<float>(C, 0.0f));
+    upload(rv2, std::vector<float>(C, 1.0f));
+    upload(xc, hx);
+    BaseTensor &bmean2 = mean2, &bvar2 = var2, &brm2 = rm2, &brv2 = rv2, &by3 = y3, &bxc = xc,
+               &bdscale2 = dscale2, &bdbias2 = dbias2, &bdmean2 = dmean2, &bdvar2 = dvar2;
+    batchnorm_forward(bx, bscale, bbias, bmean2, bvar2, brm2, brv2, by3, n, 0.9, 1e-5);
+    CHECK(download(mean2) == download(mean));
+    CHECK(download(var2) == download(var));
+    CHECK(download(rm2) == download(rm));
+    CHECK(download(rv2) == download(rv));
+    CHECK(download(y3) == download(y));
+    batchnorm_backward(bxc, bdy, bmean, bvar, bscale, bdscale2, bdbias2, bdmean2, bdvar2, bxc, n, 1e-5);
+    CHECK(download(dscale2) == download(dscale));
+    CHECK(download(dbias2) == download(dbias));
+    CHECK(download(dmean2) == download(dmean));
+    CHECK(download(dvar2) == download(dvar));
+    CHECK(download(xc) == download(dx));
 }
 
 // A view with padded rows (stride of dimension 1 larger than the extent of
@@ -227,6 +249,27 @@ static void test_strided_view()
     batchnorm_channel_sums(view, s2, q2);
     CHECK(max_rel(download(s1), download(s2)) <= 1e-6);
     CHECK(max_rel(download(q1), download(q2)) <= 1e-6);
+
+    // the two-launch forward reads the view and leaves the bits of the staged operators
+    Tensor<float> scale(Device::GPU, cshape, ctypes, stream), bias(Device::GPU, cshape, ctypes, stream),
+        rm(Device::GPU, cshape, ctypes, stream), rv(Device::GPU, cshape, ctypes, stream),
+        rm2(Device::GPU, cshape, ctypes, stream), rv2(Device::GPU, cshape, ctypes, stream),
+        m2(Device::GPU, cshape, ctypes, stream), v2(Device::GPU, cshape, ctypes, stream);
+    Tensor<float> y1(Device::GPU, shape, types, stream), y2(Device::GPU, shape, types, stream);
+    upload(scale, std::vector<float>(C, 1.5f));
+    upload(bias, std::vector<float>(C, -0.25f));
+    for (Tensor<float>* t : {&rm, &rm2})
+        upload(*t, std::vector<float>(C, 0.0f));
+    for (Tensor<float>* t : {&rv, &rv2})
+        upload(*t, std::vector<float>(C, 1.0f));
+    const size_t n = (size_t) W * H * N;
+    batchnorm_statistics(s2, q2, rm, rv, n, 0.9);
+    batchnorm_normalize(view, s2, q2, scale, bias, y1, 1e-5);
+    batchnorm_forward(view, scale, bias, m2, v2, rm2, rv2, y2, n, 0.9, 1e-5);
+    CHECK(download(m2) == download(s2));
+    CHECK(download(v2) == download(q2));
+    CHECK(download(rm2) == download(rm));
+    CHECK(download(y2) == download(y1));
     check_hip(hipDeviceSynchronize(), "sync");
     check_hip(hipFree(raw), "hipFree");
 }
