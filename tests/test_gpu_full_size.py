@@ -59,6 +59,60 @@ def test_config3_bn3d(oracle_mod):
     _bn_full((4, 64, 64, 64, 64), 1237, oracle_mod)
 
 
+@pytest.mark.parametrize("clearing", [False, True])
+def test_config3_bn3d_on_a_haloed_shard(oracle_mod, clearing):
+    """Config 3's local size with a halo of one cell on every spatial dimension (the shard of
+    a 2 x 2 x 2 decomposition): the interior equals the oracle on the interior alone; the halo
+    cells of y and dx keep what they held, or are zero with clear_output_halo."""
+    import torch
+    from dihydrogen_amd.layers import BatchNormalization
+    from dihydrogen_amd.tensor import Distribution, LocaleVirtual, Tensor
+    shape = (4, 64, 64, 64, 64)
+    rng = np.random.default_rng(1239)
+    c = shape[1]
+    x = rng.standard_normal(shape, dtype=np.float32)
+    dy = rng.standard_normal(shape, dtype=np.float32)
+    scale = rng.uniform(0.5, 1.5, c).astype(np.float32)
+    bias = (0.1 * rng.standard_normal(c)).astype(np.float32)
+    dist = Distribution.make_overlapped_distribution([2, 2, 2, 1, 1], [1, 1, 1, 0, 0])
+    mk = lambda: Tensor([128, 128, 128, c, shape[0]], LocaleVirtual(0, 8), dist).allocate()
+    xt, yt, dyt, dxt = mk(), mk(), mk(), mk()
+    sentinel = 7.25
+    for t in (xt, dyt):
+        t.real_view().fill_(1e30)  # the halo of an input is never read
+    for t in (yt, dxt):
+        t.real_view().fill_(sentinel)
+    xt.interior_view().copy_(torch.from_numpy(x))
+    dyt.interior_view().copy_(torch.from_numpy(dy))
+    dev = lambda a: torch.from_numpy(a.copy()).cuda()
+    mean, var = torch.empty(c, device="cuda"), torch.empty(c, device="cuda")
+    rm, rv = torch.zeros(c, device="cuda"), torch.ones(c, device="cuda")
+    grads = [torch.empty(c, device="cuda") for _ in range(4)]
+    bn = BatchNormalization(len(shape), 0.9, 1e-5, clear_output_halo=clearing)
+    bn.forward(xt, mean, var, rm, rv, dev(scale), dev(bias), yt, True)
+    bn.backward(xt, dyt, mean, var, dev(scale), *grads, dxt)
+    torch.cuda.synchronize()
+    rm_o, rv_o = np.zeros(c, np.float32), np.ones(c, np.float32)
+    y_o, mean_o, var_o = oracle_mod.bn_forward(x, scale, bias, rm_o, rv_o)
+    assert max_rel(mean.cpu().numpy(), mean_o) <= TOL
+    assert max_rel(var.cpu().numpy(), var_o) <= TOL
+    assert max_rel(rm.cpu().numpy(), rm_o) <= TOL and max_rel(rv.cpu().numpy(), rv_o) <= TOL
+    assert max_rel(yt.interior_view().cpu().numpy(), y_o) <= TOL
+    del y_o
+    dx_o, dscale_o, dbias_o, dmean_o, dvar_o = oracle_mod.bn_backward(x, dy, mean_o, var_o, scale)
+    for got, want in zip(grads, (dscale_o, dbias_o, dmean_o, dvar_o)):
+        assert max_rel(got.cpu().numpy(), want) <= TOL
+    assert max_rel(dxt.interior_view().cpu().numpy(), dx_o) <= TOL
+    del dx_o
+    # the halo: what is left of the whole allocation once the interior is taken out
+    expect = 0.0 if clearing else sentinel
+    for t in (yt, dxt):
+        whole = t.real_view()
+        halo_cells = whole.numel() - t.interior_view().numel()
+        t.interior_view().fill_(expect)
+        assert int((whole == expect).sum().item()) == whole.numel() and halo_cells > 0
+
+
 def test_config4_softmax(oracle_mod):
     import torch
     from dihydrogen_amd.layers import Softmax, SoftmaxMode
