@@ -48,6 +48,20 @@ def _bn_shapes(count=36, seed=20240607, max_elems=400_000):
     return shapes
 
 
+def _bn_long_shapes(count=12, seed=20240613, max_elems=6_000_000):
+    """Segments of 6 000 to 1.5 million elements: the chunking of the long-segment kernels
+    (chunks of whole tiles, last chunks, odd lengths that end in an overlapping vector)."""
+    rng = np.random.default_rng(seed)
+    shapes = []
+    while len(shapes) < count:
+        sp = _spatial(rng, 6000, 1_500_000, int(rng.integers(2, 4)))
+        s = int(np.prod(sp))
+        c = int(np.exp(rng.uniform(0, np.log(max(1, min(40, max_elems // s))))))
+        n = int(np.exp(rng.uniform(0, np.log(max(1, min(8, max_elems // (s * c)))))))
+        shapes.append((n, c) + sp)
+    return shapes
+
+
 def _softmax_shapes(count=30, seed=20240608, max_elems=300_000):
     rng = np.random.default_rng(seed)
     shapes = []
@@ -78,6 +92,11 @@ def test_batch_norm(shape, oracle_mod):
         bn_tests.test_backward_matches_oracle(shape, oracle_mod)
     for dtype in ("float32", "float64"):
         bn_tests.test_two_launch_forward_and_backward_equal_the_staged_calls(shape, dtype)
+
+
+@pytest.mark.parametrize("shape", _bn_long_shapes())
+def test_batch_norm_on_long_segments(shape, oracle_mod):
+    test_batch_norm(shape, oracle_mod)
 
 
 @pytest.mark.parametrize("shape", _softmax_shapes())
