@@ -1,6 +1,8 @@
 """Shared helpers of the test-suite (not collected by pytest)."""
 from __future__ import annotations
 
+import contextlib
+
 import numpy as np
 
 
@@ -149,3 +151,44 @@ def oracle_halo_exchange(oracle, geoms, fields, periodic=False, widths=None, is_
                     continue
                 oracle.halo_pack_or_unpack(fields[r], d, side, w, recv[(r, side)], False,
                                            is_reverse, op)
+
+
+GUARD_ELEMS = 1024   # on either side of a tensor; keeps the tensor's 16-byte alignment
+GUARD_BYTE = 0xA5
+
+
+@contextlib.contextmanager
+def guarded_allocations():
+    """While active, Tensor.allocate puts every tensor between two guard zones of GUARD_BYTE and
+    records the allocation in the list this yields (for check_guards)."""
+    import torch
+    from dihydrogen_amd import tensor as tensor_mod
+    allocated = []
+
+    def allocate(self):
+        n = max(self.get_local_real_size(), 1)
+        whole = torch.zeros(n + 2 * GUARD_ELEMS, dtype=self.dtype, device=self.device)
+        raw = whole.view(torch.uint8)
+        guard_bytes = GUARD_ELEMS * whole.element_size()
+        raw[:guard_bytes] = GUARD_BYTE
+        raw[-guard_bytes:] = GUARD_BYTE
+        self.data = whole[GUARD_ELEMS:GUARD_ELEMS + n]
+        allocated.append((raw, guard_bytes, tuple(self.local_real_shape)))
+        return self
+
+    original = tensor_mod.Tensor.allocate
+    tensor_mod.Tensor.allocate = allocate
+    try:
+        yield allocated
+    finally:
+        tensor_mod.Tensor.allocate = original
+
+
+def check_guards(allocated):
+    import torch
+    torch.cuda.synchronize()
+    for raw, guard_bytes, shape in allocated:
+        front = int((raw[:guard_bytes] != GUARD_BYTE).sum())
+        back = int((raw[-guard_bytes:] != GUARD_BYTE).sum())
+        assert front == 0 and back == 0, \
+            f"a kernel wrote outside a tensor of real shape {shape}: {front} bytes in front, {back} behind"

@@ -191,3 +191,25 @@ def test_zero_sized_calls_are_noops_or_zero_fill():
     torch.cuda.synchronize()
     for o in out:
         assert (o == 0).all()
+
+
+def test_guard_zones_of_the_test_tensors_detect_a_stray_store(guarded_tensor_allocations):
+    """The guard zones every GPU test's tensors lie between: a store one element in front of or
+    behind the allocation is reported, a store inside it (halo cells included) is not."""
+    import helpers
+    from dihydrogen_amd.tensor import Distribution, LocaleVirtual, Tensor
+    dist = Distribution.make_overlapped_distribution([2, 2, 1, 1], [1, 1, 0, 0])
+    t = Tensor([12, 10, 3, 2], LocaleVirtual(0, 4), dist).allocate()
+    mine = [a for a in guarded_tensor_allocations if a[2] == tuple(t.local_real_shape)]
+    assert len(mine) == 1 and t.data.data_ptr() % 16 == 0
+    raw, guard_bytes, _ = mine[0]
+    t.real_view().fill_(1.0)   # the whole allocation, halo included
+    helpers.check_guards(mine)
+    elem = t.data.element_size()
+    for at in (guard_bytes - elem, raw.numel() - guard_bytes):   # last element in front, first behind
+        saved = raw[at:at + elem].clone()
+        raw[at:at + elem] = 0
+        with pytest.raises(AssertionError, match="wrote outside a tensor"):
+            helpers.check_guards(mine)
+        raw[at:at + elem] = saved
+    helpers.check_guards(mine)
