@@ -16,6 +16,13 @@ from . import capi
 from .tensor import Tensor, _prod
 
 
+def _device_buffer(count: int, dtype, device="cuda", zero: bool = False) -> torch.Tensor:
+    """Every device buffer the layers own (workspaces, receive buffers, the shuffler's arena)
+    comes from here, so that a test can put guard zones around them."""
+    return (torch.zeros if zero else torch.empty)(count, dtype=dtype, device=device)
+
+
+
 def _stream_handle(stream: Optional[torch.cuda.Stream]) -> ctypes.c_void_p:
     s = torch.cuda.current_stream() if stream is None else stream
     return ctypes.c_void_p(s.cuda_stream)
@@ -119,7 +126,7 @@ class BatchNormalization:
     def _ws(self, num_channels: int) -> torch.Tensor:
         if self._workspace is None or self._workspace_channels != num_channels:
             nbytes = self._lib.h2x_bn_workspace_bytes(num_channels)
-            self._workspace = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+            self._workspace = _device_buffer(nbytes, torch.uint8)
             self._workspace_channels = num_channels
         return self._workspace
 
@@ -366,7 +373,7 @@ def reduce_sum(src: Tensor, dst: Tensor, square: bool = False, region: Optional[
     key = torch.cuda.current_stream().cuda_stream if stream is None else stream.cuda_stream
     ws = _reduce_workspaces.get(key)
     if ws is None or ws.numel() < need:
-        ws = _reduce_workspaces[key] = torch.empty(max(need, 256), dtype=torch.uint8, device="cuda")
+        ws = _reduce_workspaces[key] = _device_buffer(max(need, 256), torch.uint8)
     capi.check(lib.h2x_tensor_reduce_sum(src.h2x_dtype, ctypes.byref(gs), ctypes.c_void_p(src.get_base_ptr()),
                                          ctypes.byref(gd), ctypes.c_void_p(dst.get_base_ptr()), int(square),
                                          ctypes.c_void_p(ws.data_ptr()), _stream_handle(stream)), "tensor reduce_sum")
@@ -406,7 +413,7 @@ class Softmax:
     def _workspace(self, n: int) -> torch.Tensor:
         need = self._lib.h2x_softmax_instance_workspace_bytes(n)
         if self._ws is None or self._ws.numel() < need:
-            self._ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+            self._ws = _device_buffer(need, torch.uint8)
         return self._ws
 
     def forward(self, x: Tensor, y: Tensor) -> int:
@@ -555,7 +562,7 @@ class HaloExchangeVirtual:
         if key not in self._recv:
             t = self.tensors[rank]
             n = self.get_halo_size(rank, dim, t.overlap[dim])  # sized for the full halo (:285-303)
-            self._recv[key] = torch.zeros(max(n, 1), dtype=t.dtype, device=t.device)
+            self._recv[key] = _device_buffer(max(n, 1), t.dtype, t.device, zero=True)
         return self._recv[key]
 
     def make_face(self, rank, dim, side, width, buf, is_pack, is_reverse, op) -> capi.HaloFace:
@@ -847,7 +854,7 @@ class TensorShufflerVirtual:
         recv_displs = [[sum(recv_counts[r][:p]) for p in range(n)] for r in range(n)]
         recv_sizes = [sum(recv_counts[r]) for r in range(n)]
         arena_offsets = [sum(recv_sizes[:r]) for r in range(n)]
-        arena = torch.zeros(max(sum(recv_sizes), 1), dtype=src[0].dtype, device=src[0].device)
+        arena = _device_buffer(max(sum(recv_sizes), 1), src[0].dtype, src[0].device, zero=True)
         if sum(recv_sizes) >= 2 ** 31:
             raise ValueError("arena exceeds the 32-bit displacements of the shuffler tables")
         pack_plans, unpack_plans = [], []

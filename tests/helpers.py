@@ -159,8 +159,9 @@ GUARD_BYTE = 0xA5
 
 @contextlib.contextmanager
 def guarded_allocations():
-    """While active, Tensor.allocate puts every tensor between two guard zones of GUARD_BYTE and
-    records the allocation in the list this yields (for check_guards)."""
+    """While active, Tensor.allocate and the buffers the layers own (workspaces, receive buffers,
+    the shuffler's arena) lie between two guard zones of GUARD_BYTE each; the allocations are
+    recorded in the list this yields (for check_guards)."""
     import torch
     from dihydrogen_amd import tensor as tensor_mod
     allocated = []
@@ -176,12 +177,22 @@ def guarded_allocations():
         allocated.append((raw, guard_bytes, tuple(self.local_real_shape)))
         return self
 
-    original = tensor_mod.Tensor.allocate
-    tensor_mod.Tensor.allocate = allocate
+    def device_buffer(count, dtype, device="cuda", zero=False):
+        whole = torch.zeros(count + 2 * GUARD_ELEMS, dtype=dtype, device=device)
+        raw = whole.view(torch.uint8)
+        guard_bytes = GUARD_ELEMS * whole.element_size()
+        raw[:guard_bytes] = GUARD_BYTE
+        raw[-guard_bytes:] = GUARD_BYTE
+        allocated.append((raw, guard_bytes, ("buffer", count)))
+        return whole[GUARD_ELEMS:GUARD_ELEMS + count]
+
+    from dihydrogen_amd import layers as layers_mod
+    original, original_buffer = tensor_mod.Tensor.allocate, layers_mod._device_buffer
+    tensor_mod.Tensor.allocate, layers_mod._device_buffer = allocate, device_buffer
     try:
         yield allocated
     finally:
-        tensor_mod.Tensor.allocate = original
+        tensor_mod.Tensor.allocate, layers_mod._device_buffer = original, original_buffer
 
 
 def check_guards(allocated):
@@ -191,4 +202,4 @@ def check_guards(allocated):
         front = int((raw[:guard_bytes] != GUARD_BYTE).sum())
         back = int((raw[-guard_bytes:] != GUARD_BYTE).sum())
         assert front == 0 and back == 0, \
-            f"a kernel wrote outside a tensor of real shape {shape}: {front} bytes in front, {back} behind"
+            f"a kernel wrote outside a tensor of real shape (or a buffer of size) {shape}: {front} bytes in front, {back} behind"
