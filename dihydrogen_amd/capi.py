@@ -173,6 +173,8 @@ SIGNATURES = {
                                           c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_double, c_void_p]),
     "h2x_bn_audit": (c_int, [c_int, c_int, c_int, POINTER(POINTER(TensorGeometry)), POINTER(c_uint64),
                              POINTER(BnAuditReport)]),
+    "h2x_bn_audit_clearing": (c_int, [c_int, c_int, POINTER(HaloedGeometry), POINTER(c_uint64),
+                                      POINTER(BnAuditReport)]),
     "h2x_tensor_transform": (c_int, [c_int, c_int, c_int, POINTER(POINTER(TensorGeometry)), POINTER(c_void_p),
                                      POINTER(c_double), c_void_p]),
     "h2x_tensor_reduce_sum_workspace_bytes": (c_size_t, [POINTER(TensorGeometry), POINTER(TensorGeometry)]),

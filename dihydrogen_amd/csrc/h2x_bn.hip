@@ -761,36 +761,6 @@ __global__ __launch_bounds__(kBlockSize) void bn_backprop2_kernel(
 // legacy/include/distconv/dnn_backend/convolution.hpp:400-411), in one pass and
 // without the partly written sectors that the gaps between interior rows cost
 // the kernels above.  Halo cells of the inputs are loaded and ignored.
-struct RealBox
-{
-    FastDiv wr, hr;        // real extents of spatial dimensions 0 and 1
-    uint32_t lo[3], hi[3]; // interior: lo <= index < hi, per spatial dimension (real coordinates)
-};
-
-// Whether the elements i ... i + VEC - 1 of a real segment are interior ones.
-template <int VEC>
-__device__ __forceinline__ void interior_mask(const RealBox& b, uint32_t i, bool (&inside)[VEC])
-{
-    uint32_t t = fastdiv(i, b.wr);
-    uint32_t x = i - t * b.wr.divisor;
-    uint32_t z = fastdiv(t, b.hr);
-    uint32_t y = t - z * b.hr.divisor;
-#pragma unroll
-    for (int j = 0; j < VEC; ++j)
-    {
-        inside[j] = x >= b.lo[0] && x < b.hi[0] && y >= b.lo[1] && y < b.hi[1] && z >= b.lo[2] && z < b.hi[2];
-        if (++x == b.wr.divisor)
-        {
-            x = 0;
-            if (++y == b.hr.divisor)
-            {
-                y = 0;
-                ++z;
-            }
-        }
-    }
-}
-
 // BACKWARD: the input gradient (x, dy -> dx); else normalise (x -> y).  Segments
 // are `real` elements long and follow one another (channel stride = real).
 template <typename T, int VEC, bool BACKWARD>
@@ -2238,6 +2208,24 @@ int clearing_impl(bool backward, size_t num_per_sum, const h2x_haloed_geometry* 
     if (!grid_ok(workgroups))
         return H2X_ERR_TOO_LARGE;
     const unsigned int grid = static_cast<unsigned int>(workgroups);
+    {
+        LaunchRecord rec;
+        rec.kernel = kKernelClearing;
+        rec.family = kFamilyDense;
+        rec.vec = vw;
+        rec.grid_x = grid;
+        rec.num_samples = static_cast<int>(g->local_shape[nd - 1]);
+        rec.num_channels = num_channels;
+        rec.spatial = real;
+        rec.real = real;
+        rec.chunk = ch.chunk;
+        rec.chunks_per_seg = ch.chunks_per_seg;
+        rec.num_tensors = backward ? 3 : 2;
+        rec.last_is_output = true;
+        rec.box = box;
+        if (logged(rec))
+            return H2X_SUCCESS;
+    }
 #define H2X_LAUNCH_CLEARING(VEC, BACKWARD)                                                         \
     bn_clearing_kernel<T, VEC, BACKWARD><<<grid, kBlockSize, 0, stream>>>(                         \
         static_cast<const T*>(x), static_cast<const T*>(dy), static_cast<const T*>(mean),          \

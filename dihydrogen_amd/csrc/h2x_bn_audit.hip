@@ -16,10 +16,13 @@
 //     workgroup b = (segment, chunk), segment = (sample, channel), same vectors.
 //   short family: lane = short_lane(thread, window); reductions walk samples
 //     first + row, + rows, ...; elementwise kernels every sample of the range.
+//   halo-clearing kernel (bn_clearing_kernel): workgroup b = (segment, chunk)
+//     over the real tensor, vectors as above, interior_mask per vector.
 #include "h2x_bn_plan.hpp"
 
 #include <algorithm>
 #include <cstring>
+#include <type_traits>
 #include <vector>
 
 namespace h2x
@@ -369,6 +372,106 @@ extern "C" int h2x_bn_audit(h2x_bn_stage stage, h2x_dtype dtype, int num_samples
             walk<2>(r, count.data());
         for (int t = 0; t < r.num_tensors; ++t)
             count[t].finish(&out.tensor[t]);
+    }
+    return H2X_SUCCESS;
+}
+
+extern "C" int h2x_bn_audit_clearing(int backward, h2x_dtype dtype, const h2x_haloed_geometry* geometry,
+                                     const uint64_t* address, h2x_bn_audit_report* report)
+{
+    if (!geometry || !address || !report || (dtype != H2X_F32 && dtype != H2X_F64))
+        return H2X_ERR_INVALID_ARGUMENT;
+    std::memset(report, 0, sizeof(*report));
+    void* const param = reinterpret_cast<void*>(static_cast<uintptr_t>(4096));
+    const auto ptr = [&](int t) { return reinterpret_cast<void*>(static_cast<uintptr_t>(address[t])); };
+    LaunchLog log;
+    LaunchLog* before = install_launch_log(&log);
+    const int err = backward ? h2x_bn_backprop2_clearing(dtype, 2, geometry, ptr(0), ptr(1), param, param, param,
+                                                         param, param, ptr(2), 1e-5, nullptr)
+                             : h2x_bn_batch_normalization_clearing(dtype, geometry, ptr(0), param, param, param,
+                                                                   param, ptr(1), 1e-5, nullptr);
+    install_launch_log(before);
+    if (err)
+        return err;
+    report->num_launches = static_cast<int32_t>(log.records.size());
+    if (log.records.size() > H2X_BN_AUDIT_MAX_LAUNCHES)
+        return H2X_ERR_TOO_LARGE;
+    for (size_t l = 0; l < log.records.size(); ++l)
+    {
+        const LaunchRecord& r = log.records[l];
+        h2x_bn_audit_launch& out = report->launch[l];
+        out.kernel = r.kernel;
+        out.family = r.family;
+        out.vector_width = r.vec;
+        out.grid_x = r.grid_x;
+        out.grid_y = r.grid_y;
+        out.num_tensors = r.num_tensors;
+        if (r.kernel != kKernelClearing)
+            return H2X_ERR_UNSUPPORTED;
+        // the interior of one real segment, from the local shape and the halo widths alone
+        const int ns = geometry->num_dims - 2;
+        int64_t real_extent[3] = {1, 1, 1}, lo[3] = {0, 0, 0}, len[3] = {1, 1, 1};
+        for (int d = 0; d < ns; ++d)
+        {
+            real_extent[d] = geometry->real_shape[d];
+            lo[d] = geometry->lower_halo[d];
+            len[d] = geometry->local_shape[d];
+        }
+        std::vector<uint8_t> interior(r.real, 0);
+        for (int64_t z = 0; z < len[2]; ++z)
+            for (int64_t y = 0; y < len[1]; ++y)
+                for (int64_t x = 0; x < len[0]; ++x)
+                    interior[static_cast<size_t>(((z + lo[2]) * real_extent[1] + (y + lo[1])) * real_extent[0]
+                                                 + (x + lo[0]))] = 1;
+        const size_t segments = static_cast<size_t>(r.num_samples) * r.num_channels;
+        const size_t cells = segments * r.real;
+        std::vector<uint8_t> stored(cells, 0);
+        h2x_bn_audit_tensor* t = out.tensor;
+        const int last = r.num_tensors - 1;
+        const auto play = [&](auto vec_tag) {
+            constexpr int VEC = decltype(vec_tag)::value;
+            for (unsigned int b = 0; b < r.grid_x; ++b)
+            {
+                const size_t seg = b / r.chunks_per_seg;
+                const size_t begin = static_cast<size_t>(b % r.chunks_per_seg) * r.chunk;
+                const size_t end = std::min(begin + r.chunk, r.real);
+                for (size_t i = begin; i + VEC <= end; i += VEC)
+                {
+                    bool inside[VEC];
+                    interior_mask<VEC>(r.box, static_cast<uint32_t>(i), inside);
+                    for (int j = 0; j < VEC; ++j)
+                    {
+                        const size_t at = seg * r.real + i + j;
+                        const bool beyond = seg >= segments || i + j >= r.real;
+                        for (int k = 0; k < last; ++k) // x (and dy): halo cells are loaded and ignored
+                        {
+                            ++t[k].loads;
+                            t[k].outside += beyond;
+                        }
+                        ++t[last].stores;
+                        if (beyond)
+                        {
+                            ++t[last].outside;
+                            continue;
+                        }
+                        t[last].outside += inside[j] != (interior[i + j] != 0);
+                        if (stored[at] < 255)
+                            ++stored[at];
+                    }
+                }
+            }
+        };
+        if (r.vec == 4)
+            play(std::integral_constant<int, 4>());
+        else if (r.vec == 2)
+            play(std::integral_constant<int, 2>());
+        else
+            play(std::integral_constant<int, 1>());
+        for (size_t i = 0; i < cells; ++i)
+        {
+            t[last].missed += stored[i] == 0;
+            t[last].owned_twice += stored[i] > 1;
+        }
     }
     return H2X_SUCCESS;
 }

@@ -176,5 +176,37 @@ __host__ __device__ __forceinline__ int slot_offset(const ShortLane& l, const Sh
     return static_cast<int>(l.first + y * t.sy + z * t.sz);
 }
 
+// The real (allocated) local tensor of the halo-clearing kernels: they walk
+// every cell of a (sample, channel) segment, interior and halo alike.
+struct RealBox
+{
+    FastDiv wr, hr;        // real extents of spatial dimensions 0 and 1
+    uint32_t lo[3], hi[3]; // interior: lo <= index < hi, per spatial dimension (real coordinates)
+};
+
+// Whether the elements i ... i + VEC - 1 of a real segment are interior ones.
+template <int VEC>
+__host__ __device__ __forceinline__ void interior_mask(const RealBox& b, uint32_t i, bool (&inside)[VEC])
+{
+    uint32_t t = fastdiv(i, b.wr);
+    uint32_t x = i - t * b.wr.divisor;
+    uint32_t z = fastdiv(t, b.hr);
+    uint32_t y = t - z * b.hr.divisor;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j)
+    {
+        inside[j] = x >= b.lo[0] && x < b.hi[0] && y >= b.lo[1] && y < b.hi[1] && z >= b.lo[2] && z < b.hi[2];
+        if (++x == b.wr.divisor)
+        {
+            x = 0;
+            if (++y == b.hr.divisor)
+            {
+                y = 0;
+                ++z;
+            }
+        }
+    }
+}
+
 } // namespace bn
 } // namespace h2x

@@ -23,7 +23,8 @@ enum Kernel : int
     kKernelBackprop2 = 3,
     kKernelFinish = 4,      // adds the partial sums of a reduction
     kKernelStatistics = 5,  // sums -> mean / variance / running statistics
-    kKernelFill = 6         // zeroes per-channel outputs (empty tensors)
+    kKernelFill = 6,        // zeroes per-channel outputs (empty tensors)
+    kKernelClearing = 7     // normalise / input gradient over the real tensor, halo of the output zeroed
 };
 
 enum Family : int
@@ -59,6 +60,8 @@ struct LaunchRecord
     TensorMap map[kMaxLaunchTensors];     // dense and strided families
     ShortTensor tensor[kMaxLaunchTensors]; // short family
     ShortGeometry geometry;                // short family
+    RealBox box;                           // halo-clearing kernel: real extents and interior
+    size_t real = 0;                       // halo-clearing kernel: cells of a real segment
 };
 
 struct LaunchLog

@@ -521,7 +521,7 @@ typedef struct h2x_bn_audit_tensor
 
 typedef struct h2x_bn_audit_launch
 {
-    int32_t kernel; /* 0 sums, 1 normalise, 2 backprop1, 3 backprop2, 4 finish, 5 statistics, 6 fill */
+    int32_t kernel; /* 0 sums, 1 normalise, 2 backprop1, 3 backprop2, 4 finish, 5 statistics, 6 fill, 7 halo-clearing */
     int32_t family; /* 0 dense, 1 strided (padded rows, folded samples), 2 short segments */
     int32_t vector_width; /* elements per access */
     int32_t tail;         /* short family: 0 whole vectors, 1 overlapping last vector, 2 element by element */
@@ -549,6 +549,23 @@ int h2x_bn_audit(h2x_bn_stage stage,
                  const h2x_tensor_geometry* const* geometry,
                  const uint64_t* address,
                  h2x_bn_audit_report* report);
+
+/**
+ * The same audit for h2x_bn_batch_normalization_clearing (`backward` 0: tensors
+ * x, y) and h2x_bn_backprop2_clearing (`backward` 1: x, dy, dx), which walk the
+ * real local tensor.  Addresses are the allocation starts.  Per tensor:
+ * `outside` counts accesses beyond the real tensor and, for the output, cells
+ * the kernel's interior test places on the wrong side (a halo cell computed or
+ * an interior cell zeroed; the interior is enumerated independently from the
+ * local shape and the halo widths); `missed` / `owned_twice` count real cells
+ * of the output that are stored never / more than once.  All must be 0.  The
+ * launch is reported with kernel 7.
+ */
+int h2x_bn_audit_clearing(int backward,
+                          h2x_dtype dtype,
+                          const h2x_haloed_geometry* geometry,
+                          const uint64_t* address,
+                          h2x_bn_audit_report* report);
 
 /* ------------------------------------------------------------------------ */
 /* Elementwise transforms and sums over dimensions                           */

@@ -424,7 +424,10 @@ def test_haloed_tensors_match_oracle(case, oracle_mod):
 CLEARING_CASES = HALO_CASES + [
     ((16, 8, 6, 2), (1, 2, 1, 1), (0, 3, 0, 0)),          # halo on the outermost spatial dimension only
     ((10, 6, 6, 3, 2), (2, 1, 2, 1, 1), (1, 0, 2, 0, 0)),  # real segment of 7 x 6 x 7 elements: no whole vectors
-    ((128, 128, 8, 2), (2, 2, 1, 1), (1, 1, 0, 0)),        # 66 x 66 real: rows 8 bytes off every other time
+    ((128, 128, 8, 2), (2, 2, 1, 1), (1, 1, 0, 0)),        # 66 x 66 real: rows 8 bytes off every other time    # real planes of 18 and 15 cells with no halo on dimension 1: vectors that begin in the last row of a
+    # plane and end in the first, interior, row of the next
+    ((8, 3, 4, 3, 2), (2, 1, 2, 1, 1), (1, 0, 1, 0, 0)),
+    ((6, 3, 4, 3, 2), (2, 1, 2, 1, 1), (1, 0, 1, 0, 0)),
 ]
 
 

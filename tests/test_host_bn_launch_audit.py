@@ -209,3 +209,76 @@ def test_rejected_and_empty_calls():
     err, _ = audit(capi.BN_STAGE_NORMALIZE, capi.F32, 2,
                    [haloed_geometry((8, 4), 3, 2, (1, 1)), haloed_geometry((4, 8), 3, 2, (1, 1))], [1 << 20, 1 << 30])
     assert err == -1
+
+
+def clearing_geometry(spatial, c, n, lower, upper):
+    g = capi.HaloedGeometry()
+    shape = list(spatial) + [c, n]
+    g.num_dims = len(shape)
+    for i, e in enumerate(shape):
+        lo = lower[i] if i < len(spatial) else 0
+        hi = upper[i] if i < len(spatial) else 0
+        g.local_shape[i], g.real_shape[i], g.lower_halo[i] = e, e + lo + hi, lo
+    return g
+
+
+def audit_clearing(backward, dtype, geometry, addresses):
+    lib = capi.load()
+    adr = (ctypes.c_uint64 * 3)(*(list(addresses) + [0] * (3 - len(addresses))))
+    rep = capi.BnAuditReport()
+    err = lib.h2x_bn_audit_clearing(int(backward), dtype, ctypes.byref(geometry), adr, ctypes.byref(rep))
+    return err, rep
+
+
+CLEARING = [((64, 64, 64), (1, 1, 1), (1, 1, 1)), ((14, 14), (1, 1), (1, 1)), ((7, 7), (1, 1), (1, 1)),
+            ((30, 6, 5), (1, 0, 1), (1, 0, 1)), ((8, 8, 8), (2, 1, 0), (0, 1, 2)), ((33, 9), (3, 2), (0, 1)),
+            ((5, 51), (0, 1), (0, 1)), ((1, 300), (1, 1), (1, 1)), ((130, 3), (1, 1), (2, 2)), ((6, 6, 40), (0, 1, 1), (0, 1, 1)),
+            ((12, 3, 4), (0, 0, 0), (0, 0, 0)),
+            # real planes of 15 and 18 cells, no halo on dimension 1: vectors that begin in the last row
+            # of one plane and end in the first, interior, row of the next
+            ((4, 3, 2), (1, 0, 1), (0, 0, 1)), ((5, 3, 2), (1, 0, 1), (0, 0, 1))]
+
+
+@pytest.mark.parametrize("dtype", (capi.F32, capi.F64))
+@pytest.mark.parametrize("backward", (False, True))
+def test_halo_clearing_kernels_store_every_real_cell_once_and_zero_exactly_the_halo(backward, dtype):
+    elem = 4 if dtype == capi.F32 else 8
+    vec = 16 // elem
+    for (spatial, lower, upper), (n, c), shift in itertools.product(CLEARING, ((1, 2), (3, 5)), (0, 1)):
+        if spatial[0] == 64 and (n, c) != (1, 2):
+            continue  # the large box once: enough to cross several chunks
+        g = clearing_geometry(spatial, c, n, lower, upper)
+        real = 1
+        for e, lo, hi in zip(spatial, lower, upper):
+            real *= e + lo + hi
+        k = 3 if backward else 2
+        x = (1 << 20) + shift * elem
+        # out of place, and in place (the output is x itself)
+        for out in (x + (2 << 30), x):
+            addresses = [x, x + (1 << 30), out][:k - 1] + [out]
+            err, rep = audit_clearing(backward, dtype, g, addresses)
+            what = f"backward {backward} dtype {dtype} spatial {spatial} halo {lower}/{upper} N {n} C {c} shift {shift}"
+            assert err == 0 and rep.num_launches == 1, what
+            l = rep.launch[0]
+            assert l.kernel == 7 and l.num_tensors == k and 1 <= l.grid_x <= 0x7FFFFFFF, what
+            assert l.vector_width == (vec if real % vec == 0 and shift == 0 else 1), what
+            for t in range(k):
+                c_ = l.tensor[t]
+                assert (c_.outside, c_.missed, c_.owned_twice) == (0, 0, 0), (what, t, c_.outside, c_.missed, c_.owned_twice)
+            assert l.tensor[k - 1].stores == n * c * real, what
+            assert all(l.tensor[t].loads == n * c * real for t in range(k - 1)), what
+
+
+def test_halo_clearing_audit_rejects_what_the_entry_points_reject():
+    g = clearing_geometry((8, 8), 3, 2, (1, 1), (1, 1))
+    g.lower_halo[2] = 1          # a halo on the channel dimension
+    g.real_shape[2] += 1
+    err, _ = audit_clearing(False, capi.F32, g, [1 << 20, 1 << 30])
+    assert err == -2
+    g = clearing_geometry((8, 8), 3, 2, (1, 1), (1, 1))
+    g.real_shape[0] = 8          # real extent smaller than halo + local
+    err, _ = audit_clearing(False, capi.F32, g, [1 << 20, 1 << 30])
+    assert err == -1
+    # nothing to do: no launch is planned
+    err, rep = audit_clearing(True, capi.F32, clearing_geometry((8, 8), 0, 2, (1, 1), (1, 1)), [1 << 20, 1 << 30, 1 << 31])
+    assert err == 0 and rep.num_launches == 0
