@@ -566,23 +566,23 @@ def cpu_baseline(repeats: int = 5):
 # label -> (bytes read, bytes written) per launch
 PMC_TRAFFIC = {
     "bn_sums": (268455424, 131072),
-    "bn_apply": (268462080, 268486656),
-    "bn_backprop1": (536912896, 131072),
+    "bn_apply": (268462080, 268477824),
+    "bn_backprop1": (536912896, 131104),
     "bn_backprop2": (536906240, 268435456),
-    "halo_dim0_pack": (149778336, 8652800),    # 4 faces (2 ranks) a launch, four launches a step
-    "halo_dim0_unpack": (9218400, 43264000),
-    "halo_dim1_pack": (42624704, 34611200),
-    "halo_dim1_unpack": (34637696, 36217120),
+    "halo_dim0_pack": (149798208, 8652800),    # 4 faces (2 ranks) a launch, four launches a step
+    "halo_dim0_unpack": (9218944, 43264000),
+    "halo_dim1_pack": (42624768, 34611200),
+    "halo_dim1_unpack": (34637632, 36215936),
     "halo_dim2_pack": (34694400, 34611200),
-    "halo_dim2_unpack": (34637568, 34619392),
+    "halo_dim2_unpack": (34637568, 34619488),
 }
 # steps of the timed region whose dominant-kernel launches are bracketed by events: every EVENT_EVERY-th
 EVENT_EVERY = 4
 
 # sha256 (first 16 hex digits) of the kernel sources the table was measured with, see
 # kernel_sources_sha(); with other sources the traffic fields are omitted
-PMC_SOURCES_SHA = "5b4d37e541964a13"
-PMC_COMMIT = "dfa9f1c"
+PMC_SOURCES_SHA = "aff7bdece482e508"
+PMC_COMMIT = "ab39e8e"
 
 KERNEL_OF = {
     "bn_sums": "bn_sums_kernel<float,4> (+bn_finish_kernel<float,2>)",
