@@ -106,22 +106,22 @@ struct Words
 struct OpId
 {
     template <typename T>
-    __device__ __forceinline__ T operator()(T, T b) const { return b; }
+    __host__ __device__ __forceinline__ T operator()(T, T b) const { return b; }
 };
 struct OpSum
 {
     template <typename T>
-    __device__ __forceinline__ T operator()(T a, T b) const { return a + b; }
+    __host__ __device__ __forceinline__ T operator()(T a, T b) const { return a + b; }
 };
 struct OpMax
 {
     template <typename T>
-    __device__ __forceinline__ T operator()(T a, T b) const { return a > b ? a : b; }
+    __host__ __device__ __forceinline__ T operator()(T a, T b) const { return a > b ? a : b; }
 };
 struct OpMin
 {
     template <typename T>
-    __device__ __forceinline__ T operator()(T a, T b) const { return a < b ? a : b; }
+    __host__ __device__ __forceinline__ T operator()(T a, T b) const { return a < b ? a : b; }
 };
 
 #ifdef __HIPCC__
@@ -129,7 +129,7 @@ struct OpMin
 // Offset of packed element g of a box in its tensor (and, for transfers, in
 // the source tensor); `first` receives the index along the first dimension.
 template <bool TRANSFER>
-__device__ __forceinline__ void box_offsets(const Box& box, uint32_t g, int64_t* toff, int64_t* soff,
+__host__ __device__ __forceinline__ void box_offsets(const Box& box, uint32_t g, int64_t* toff, int64_t* soff,
                                             uint32_t* first)
 {
     uint32_t rem = g;
@@ -165,54 +165,97 @@ __device__ __forceinline__ void box_offsets(const Box& box, uint32_t g, int64_t*
     *soff = src;
 }
 
+// How the kernel body below reaches memory: VEC elements at an element
+// pointer, aligned to the whole vector or to one element.  The kernel uses
+// DeviceMem; the launch audit plays the same body on the CPU with an accessor
+// that records addresses instead of following them (h2x_copy_audit.hip).
+// (The accessor takes element pointers and names the vector types itself: an
+// under-aligned vector type passed as a deduced template argument would lose
+// its alignment.)
+struct DeviceMem
+{
+    template <int VEC, bool ALIGNED, typename T>
+    __device__ __forceinline__ typename Words<T, VEC>::unaligned_t load(const T* p) const
+    {
+        if constexpr (ALIGNED)
+            return *reinterpret_cast<const typename Words<T, VEC>::aligned_t*>(p);
+        else
+            return *reinterpret_cast<const typename Words<T, VEC>::unaligned_t*>(p);
+    }
+    // a load whose data is not needed again (nontemporal)
+    template <int VEC, bool ALIGNED, typename T>
+    __device__ __forceinline__ typename Words<T, VEC>::unaligned_t load_last_use(const T* p) const
+    {
+        if constexpr (ALIGNED)
+            return __builtin_nontemporal_load(reinterpret_cast<const typename Words<T, VEC>::aligned_t*>(p));
+        else
+            return __builtin_nontemporal_load(reinterpret_cast<const typename Words<T, VEC>::unaligned_t*>(p));
+    }
+    template <int VEC, bool ALIGNED, typename T>
+    __device__ __forceinline__ void store(T* p, typename Words<T, VEC>::unaligned_t v) const
+    {
+        if constexpr (ALIGNED)
+            *reinterpret_cast<typename Words<T, VEC>::aligned_t*>(p) = v;
+        else
+            *reinterpret_cast<typename Words<T, VEC>::unaligned_t*>(p) = v;
+    }
+    template <typename T>
+    __device__ __forceinline__ T load1(const T* p) const { return *p; }
+    template <typename T>
+    __device__ __forceinline__ T load1_last_use(const T* p) const { return __builtin_nontemporal_load(p); }
+    template <typename T>
+    __device__ __forceinline__ void store1(T* p, T v) const { *p = v; }
+};
+
 // Stores (identity) or folds (any other op) the vectors `va` / `vb` into the
 // tensor at `pa` / `pb` (`pb` null: a single box).  When the two boxes of a
 // pair share no element (`disjoint`), both tensor vectors are loaded before
 // either is stored: one trip to memory instead of two in a row (reverse SUM
 // exchange of the innermost dimension, 2 ranks a launch: 73 us -> 45 us).
-template <typename T, int VEC, typename WU, typename Op, bool IDENTITY>
-__device__ __forceinline__ void accumulate_pair(T* pa, T* pb, WU va, WU vb, bool disjoint, Op op)
+template <typename T, int VEC, typename WU, typename Op, bool IDENTITY, typename Mem>
+__host__ __device__ __forceinline__ void accumulate_pair(T* pa, T* pb, WU va, WU vb, bool disjoint, Op op,
+                                                         const Mem& mem)
 {
     if constexpr (IDENTITY)
     {
-        *reinterpret_cast<WU*>(pa) = va;
+        mem.template store<VEC, false>(pa, va);
         if (pb != nullptr)
-            *reinterpret_cast<WU*>(pb) = vb;
+            mem.template store<VEC, false>(pb, vb);
     }
     else if (pb == nullptr)
     {
-        WU ta = *reinterpret_cast<const WU*>(pa);
+        WU ta = mem.template load<VEC, false>(pa);
 #pragma unroll
         for (int j = 0; j < VEC; ++j)
             ta[j] = op(ta[j], va[j]);
-        *reinterpret_cast<WU*>(pa) = ta;
+        mem.template store<VEC, false>(pa, ta);
     }
     else if (disjoint)
     {
-        WU ta = *reinterpret_cast<const WU*>(pa);
-        WU tb = *reinterpret_cast<const WU*>(pb);
+        WU ta = mem.template load<VEC, false>(pa);
+        WU tb = mem.template load<VEC, false>(pb);
 #pragma unroll
         for (int j = 0; j < VEC; ++j)
         {
             ta[j] = op(ta[j], va[j]);
             tb[j] = op(tb[j], vb[j]);
         }
-        *reinterpret_cast<WU*>(pa) = ta;
-        *reinterpret_cast<WU*>(pb) = tb;
+        mem.template store<VEC, false>(pa, ta);
+        mem.template store<VEC, false>(pb, tb);
     }
     else
     {
         // the boxes may share elements: the second fold sees the first one's result
-        WU ta = *reinterpret_cast<const WU*>(pa);
+        WU ta = mem.template load<VEC, false>(pa);
 #pragma unroll
         for (int j = 0; j < VEC; ++j)
             ta[j] = op(ta[j], va[j]);
-        *reinterpret_cast<WU*>(pa) = ta;
-        WU tb = *reinterpret_cast<const WU*>(pb);
+        mem.template store<VEC, false>(pa, ta);
+        WU tb = mem.template load<VEC, false>(pb);
 #pragma unroll
         for (int j = 0; j < VEC; ++j)
             tb[j] = op(tb[j], vb[j]);
-        *reinterpret_cast<WU*>(pb) = tb;
+        mem.template store<VEC, false>(pb, tb);
     }
 }
 
@@ -238,9 +281,10 @@ __device__ __forceinline__ void accumulate_pair(T* pa, T* pb, WU va, WU vb, bool
 // often still cached from the kernel that produced them, and use plain loads
 // (a 69 MB launch: 16 us -> 12 us when the strips are cached, no difference
 // when they are not).
-template <typename T, int VEC, typename Op, bool SPARSE, int MODE, bool TABLE>
-__global__ __launch_bounds__(kCopyBlock, 8) void box_copy_kernel(
-    const typename std::conditional<TABLE, TableBatch, BoxBatch>::type batch, Op op)
+template <typename T, int VEC, typename Op, bool SPARSE, int MODE, bool TABLE, typename Mem>
+__host__ __device__ __forceinline__ void box_copy_body(
+    const typename std::conditional<TABLE, TableBatch, BoxBatch>::type& batch, Op op, const uint32_t block,
+    const uint32_t thread, const Mem& mem)
 {
     using WA = typename Words<T, VEC>::aligned_t;
     using WU = typename Words<T, VEC>::unaligned_t;
@@ -260,8 +304,8 @@ __global__ __launch_bounds__(kCopyBlock, 8) void box_copy_kernel(
     char* buffer_base = nullptr;
     if constexpr (TABLE)
     {
-        const uint32_t gb = blockIdx.x % batch.num_boxes;
-        local_block = blockIdx.x / batch.num_boxes;
+        const uint32_t gb = block % batch.num_boxes;
+        local_block = block / batch.num_boxes;
         int p = 0;
 #pragma unroll 1
         for (int i = 1; i < batch.num_plans; ++i)
@@ -276,16 +320,16 @@ __global__ __launch_bounds__(kCopyBlock, 8) void box_copy_kernel(
         int b = 0;
         if (batch.blocks_per_box != 0)
         {
-            b = blockIdx.x % batch.num_boxes;
-            local_block = blockIdx.x / batch.num_boxes;
+            b = block % batch.num_boxes;
+            local_block = block / batch.num_boxes;
         }
         else
         {
 #pragma unroll 1
             for (int i = 1; i < batch.num_boxes; ++i)
-                if (blockIdx.x >= batch.box[i].first_block)
+                if (block >= batch.box[i].first_block)
                     b = i;
-            local_block = blockIdx.x - batch.box[b].first_block;
+            local_block = block - batch.box[b].first_block;
         }
         entry = &batch.box[b];
     }
@@ -306,7 +350,7 @@ __global__ __launch_bounds__(kCopyBlock, 8) void box_copy_kernel(
 #pragma unroll
     for (int u = 0; u < kCopyUnroll; ++u)
     {
-        g[u] = block_base + u * kStride + threadIdx.x * VEC;
+        g[u] = block_base + u * kStride + thread * VEC;
         uint32_t first = 0;
         box_offsets<kTransferMode>(box, g[u], &toff[u], &soff[u], &first);
         head[u] = VEC;
@@ -342,9 +386,9 @@ __global__ __launch_bounds__(kCopyBlock, 8) void box_copy_kernel(
                     const int64_t at = MODE == kPack ? toff[u] : soff[u];
                     const T* const from_a = MODE == kPack ? tensor_a : buffer_a;
                     const T* const from_b = MODE == kPack ? tensor_b : buffer_b;
-                    va[u] = *reinterpret_cast<const WU*>(from_a + at);
+                    va[u] = mem.template load<VEC, false>(from_a + at);
                     if (tensor_b != nullptr)
-                        vb[u] = *reinterpret_cast<const WU*>(from_b + at);
+                        vb[u] = mem.template load<VEC, false>(from_b + at);
                 }
 #pragma unroll
             for (int u = 0; u < kCopyUnroll; ++u)
@@ -352,14 +396,14 @@ __global__ __launch_bounds__(kCopyBlock, 8) void box_copy_kernel(
                 {
                     if constexpr (MODE == kPack)
                     {
-                        *reinterpret_cast<WA*>(buffer_a + g[u]) = static_cast<WA>(va[u]);
+                        mem.template store<VEC, true>(buffer_a + g[u], va[u]);
                         if (tensor_b != nullptr)
-                            *reinterpret_cast<WA*>(buffer_b + g[u]) = static_cast<WA>(vb[u]);
+                            mem.template store<VEC, true>(buffer_b + g[u], vb[u]);
                     }
                     else
                     {
-                        accumulate_pair<T, VEC, WU, Op, kIdentity>(tensor_a + toff[u], tensor_b != nullptr ? tensor_b + toff[u] : nullptr,
-                                                                   va[u], vb[u], box.disjoint, op);
+                        accumulate_pair<T, VEC, WU, Op, kIdentity, Mem>(tensor_a + toff[u], tensor_b != nullptr ? tensor_b + toff[u] : nullptr,
+                                                                   va[u], vb[u], box.disjoint, op, mem);
                     }
                 }
         }
@@ -375,9 +419,9 @@ __global__ __launch_bounds__(kCopyBlock, 8) void box_copy_kernel(
                 for (int u = 0; u < kCopyUnroll; ++u)
                     if (g[u] < count)
                     {
-                        hi[u] = __builtin_nontemporal_load(buffer_b + g[u]);
+                        hi[u] = mem.load1_last_use(buffer_b + g[u]);
                         if (g[u] + 1 < count)
-                            lo[u] = __builtin_nontemporal_load(buffer_a + g[u] + 1);
+                            lo[u] = mem.load1_last_use(buffer_a + g[u] + 1);
                     }
 #pragma unroll
                 for (int u = 0; u < kCopyUnroll; ++u)
@@ -394,21 +438,21 @@ __global__ __launch_bounds__(kCopyBlock, 8) void box_copy_kernel(
                             }
                             else
                             {
-                                t = *reinterpret_cast<const Seam*>(p);
+                                t = mem.template load<2, false>(p);
                                 t[0] = op(t[0], hi[u]);
                                 t[1] = op(t[1], lo[u]);
                             }
-                            *reinterpret_cast<Seam*>(p) = t;
+                            mem.template store<2, false>(p, t);
                         }
                         else
                         {
-                            *p = kIdentity ? hi[u] : op(*p, hi[u]);
+                            mem.store1(p, kIdentity ? hi[u] : op(mem.load1(p), hi[u]));
                         }
                     }
-                if (block_base == 0 && threadIdx.x == 0) // element 0 of the first box has no partner
+                if (block_base == 0 && thread == 0) // element 0 of the first box has no partner
                 {
-                    const T v = buffer_a[0];
-                    tensor_a[0] = kIdentity ? v : op(tensor_a[0], v);
+                    const T v = mem.load1(buffer_a);
+                    mem.store1(tensor_a, kIdentity ? v : op(mem.load1(tensor_a), v));
                 }
             }
             else
@@ -418,18 +462,16 @@ __global__ __launch_bounds__(kCopyBlock, 8) void box_copy_kernel(
                 for (int u = 0; u < kCopyUnroll; ++u)
                     if (g[u] < count)
                     {
-                        va[u] = __builtin_nontemporal_load(
-                            reinterpret_cast<const WA*>(buffer_a + g[u])); // last use of the image
+                        va[u] = mem.template load_last_use<VEC, true>(buffer_a + g[u]); // last use of the image
                         if (tensor_b != nullptr)
-                            vb[u] = __builtin_nontemporal_load(
-                                reinterpret_cast<const WA*>(buffer_b + g[u]));
+                            vb[u] = mem.template load_last_use<VEC, true>(buffer_b + g[u]);
                     }
 #pragma unroll
                 for (int u = 0; u < kCopyUnroll; ++u)
                     if (g[u] < count)
                     {
-                        accumulate_pair<T, VEC, WU, Op, kIdentity>(tensor_a + toff[u], tensor_b != nullptr ? tensor_b + toff[u] : nullptr,
-                                                                   static_cast<WU>(va[u]), static_cast<WU>(vb[u]), box.disjoint, op);
+                        accumulate_pair<T, VEC, WU, Op, kIdentity, Mem>(tensor_a + toff[u], tensor_b != nullptr ? tensor_b + toff[u] : nullptr,
+                                                                   static_cast<WU>(va[u]), static_cast<WU>(vb[u]), box.disjoint, op, mem);
                     }
             }
         }
@@ -443,9 +485,9 @@ __global__ __launch_bounds__(kCopyBlock, 8) void box_copy_kernel(
 #pragma unroll
                     for (int j = 0; j < VEC; ++j)
                         z[j] = T(0);
-                    *reinterpret_cast<WU*>(tensor_a + toff[u]) = z;
+                    mem.template store<VEC, false>(tensor_a + toff[u], z);
                     if (tensor_b != nullptr)
-                        *reinterpret_cast<WU*>(tensor_b + toff[u]) = z;
+                        mem.template store<VEC, false>(tensor_b + toff[u], z);
                 }
         }
     }
@@ -476,9 +518,9 @@ __global__ __launch_bounds__(kCopyBlock, 8) void box_copy_kernel(
                     if (head[u] == VEC)
                     {
                         if constexpr (TABLE)
-                            v[u] = __builtin_nontemporal_load(reinterpret_cast<const WU*>(from + at));
+                            v[u] = mem.template load_last_use<VEC, false>(from + at);
                         else
-                            v[u] = *reinterpret_cast<const WU*>(from + at);
+                            v[u] = mem.template load<VEC, false>(from + at);
                     }
                     else
                     {
@@ -488,7 +530,7 @@ __global__ __launch_bounds__(kCopyBlock, 8) void box_copy_kernel(
 #pragma unroll
                         for (int j = 0; j < VEC; ++j)
                             if (g[u] + j < count)
-                                v[u][j] = from[j < static_cast<int>(head[u]) ? at + j : next + j];
+                                v[u][j] = mem.load1(from + (j < static_cast<int>(head[u]) ? at + j : next + j));
                     }
                 }
         }
@@ -500,15 +542,14 @@ __global__ __launch_bounds__(kCopyBlock, 8) void box_copy_kernel(
                 {
                     if (g[u] + VEC <= count)
                     {
-                        v[u] = static_cast<WU>(__builtin_nontemporal_load(
-                            reinterpret_cast<const WA*>(buffer + g[u]))); // last use of the image
+                        v[u] = mem.template load_last_use<VEC, true>(buffer + g[u]); // last use of the image
                     }
                     else
                     {
 #pragma unroll
                         for (int j = 0; j < VEC; ++j)
                             if (g[u] + j < count)
-                                v[u][j] = buffer[g[u] + j];
+                                v[u][j] = mem.load1(buffer + g[u] + j);
                     }
                 }
         }
@@ -529,14 +570,14 @@ __global__ __launch_bounds__(kCopyBlock, 8) void box_copy_kernel(
                 {
                     if (g[u] + VEC <= count)
                     {
-                        *reinterpret_cast<WA*>(buffer + g[u]) = static_cast<WA>(v[u]);
+                        mem.template store<VEC, true>(buffer + g[u], v[u]);
                     }
                     else
                     {
 #pragma unroll
                         for (int j = 0; j < VEC; ++j)
                             if (g[u] + j < count)
-                                buffer[g[u] + j] = v[u][j];
+                                mem.store1(buffer + g[u] + j, static_cast<T>(v[u][j]));
                     }
                 }
         }
@@ -552,12 +593,12 @@ __global__ __launch_bounds__(kCopyBlock, 8) void box_copy_kernel(
                         WU t = v[u];
                         if constexpr (kCombine)
                         {
-                            t = *reinterpret_cast<const WU*>(tensor + toff[u]);
+                            t = mem.template load<VEC, false>(tensor + toff[u]);
 #pragma unroll
                             for (int j = 0; j < VEC; ++j)
                                 t[j] = op(t[j], v[u][j]);
                         }
-                        *reinterpret_cast<WU*>(tensor + toff[u]) = t;
+                        mem.template store<VEC, false>(tensor + toff[u], t);
                     }
                     else
                     {
@@ -571,13 +612,21 @@ __global__ __launch_bounds__(kCopyBlock, 8) void box_copy_kernel(
                                 T* const p = tensor + (j < static_cast<int>(head[u]) ? toff[u] + j : next + j);
                                 T e = v[u][j];
                                 if constexpr (kCombine)
-                                    e = op(*p, e);
-                                *p = e;
+                                    e = op(mem.load1(p), e);
+                                mem.store1(p, e);
                             }
                     }
                 }
         }
     }
+}
+
+
+template <typename T, int VEC, typename Op, bool SPARSE, int MODE, bool TABLE>
+__global__ __launch_bounds__(kCopyBlock, 8) void box_copy_kernel(
+    const typename std::conditional<TABLE, TableBatch, BoxBatch>::type batch, Op op)
+{
+    box_copy_body<T, VEC, Op, SPARSE, MODE, TABLE, DeviceMem>(batch, op, blockIdx.x, threadIdx.x, DeviceMem());
 }
 
 #endif // __HIPCC__
