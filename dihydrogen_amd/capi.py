@@ -120,6 +120,27 @@ class ShuffleGeometry(ctypes.Structure):
     ]
 
 
+class CopyAuditRegion(ctypes.Structure):
+    """struct h2x_copy_audit_region"""
+    _fields_ = [
+        ("base", c_uint64),
+        ("bytes", c_uint64),
+        ("loads", POINTER(ctypes.c_uint8)),
+        ("stores", POINTER(ctypes.c_uint8)),
+    ]
+
+
+class CopyAuditReport(ctypes.Structure):
+    """struct h2x_copy_audit_report"""
+    _fields_ = [
+        ("launches", c_uint64),
+        ("workgroups", c_uint64),
+        ("outside_loads", c_uint64),
+        ("outside_stores", c_uint64),
+        ("misaligned", c_uint64),
+    ]
+
+
 # name -> (restype, argtypes); every symbol include/h2x.h declares.
 SIGNATURES = {
     "h2x_abi_version": (c_int, []),
@@ -173,6 +194,9 @@ SIGNATURES = {
                                           c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_double, c_void_p]),
     "h2x_bn_audit": (c_int, [c_int, c_int, c_int, POINTER(POINTER(TensorGeometry)), POINTER(c_uint64),
                              POINTER(BnAuditReport)]),
+    "h2x_copy_audit_begin": (c_int, []),
+    "h2x_copy_audit_add_region": (c_int, [POINTER(CopyAuditRegion)]),
+    "h2x_copy_audit_end": (c_int, [POINTER(CopyAuditReport)]),
     "h2x_bn_audit_clearing": (c_int, [c_int, c_int, POINTER(HaloedGeometry), POINTER(c_uint64),
                                       POINTER(BnAuditReport)]),
     "h2x_tensor_transform": (c_int, [c_int, c_int, c_int, POINTER(POINTER(TensorGeometry)), POINTER(c_void_p),

@@ -44,24 +44,14 @@ namespace
 template <typename T, int VEC, bool SPARSE>
 int launch_mode(const LaunchShape& s, const BoxBatch& batch)
 {
-    const dim3 grid(s.grid);
     switch (s.mode)
     {
-    case kPack:
-        box_copy_kernel<T, VEC, OpId, SPARSE, kPack, false><<<grid, kCopyBlock, 0, s.stream>>>(batch, OpId());
-        break;
-    case kUnpack:
-        box_copy_kernel<T, VEC, OpId, SPARSE, kUnpack, false><<<grid, kCopyBlock, 0, s.stream>>>(batch, OpId());
-        break;
-    case kClear:
-        box_copy_kernel<T, VEC, OpId, SPARSE, kClear, false><<<grid, kCopyBlock, 0, s.stream>>>(batch, OpId());
-        break;
-    case kTransfer:
-        box_copy_kernel<T, VEC, OpId, SPARSE, kTransfer, false><<<grid, kCopyBlock, 0, s.stream>>>(batch, OpId());
-        break;
+    case kPack: return run_box_copy<T, VEC, OpId, SPARSE, kPack, false>(s.grid, s.stream, batch, OpId());
+    case kUnpack: return run_box_copy<T, VEC, OpId, SPARSE, kUnpack, false>(s.grid, s.stream, batch, OpId());
+    case kClear: return run_box_copy<T, VEC, OpId, SPARSE, kClear, false>(s.grid, s.stream, batch, OpId());
+    case kTransfer: return run_box_copy<T, VEC, OpId, SPARSE, kTransfer, false>(s.grid, s.stream, batch, OpId());
     default: return H2X_ERR_UNSUPPORTED;
     }
-    return launch_status();
 }
 
 template <typename T, int VEC>
@@ -73,17 +63,22 @@ int launch_sparse(const LaunchShape& s, const BoxBatch& batch)
 template <typename T, int VEC>
 int launch_table_mode(const LaunchShape& s, const TableBatch& batch)
 {
-    const dim3 grid(s.grid);
     if (s.mode == kPack)
-        box_copy_kernel<T, VEC, OpId, false, kPack, true><<<grid, kCopyBlock, 0, s.stream>>>(batch, OpId());
-    else if (s.mode == kUnpack)
-        box_copy_kernel<T, VEC, OpId, false, kUnpack, true><<<grid, kCopyBlock, 0, s.stream>>>(batch, OpId());
-    else
-        return H2X_ERR_UNSUPPORTED;
-    return launch_status();
+        return run_box_copy<T, VEC, OpId, false, kPack, true>(s.grid, s.stream, batch, OpId());
+    if (s.mode == kUnpack)
+        return run_box_copy<T, VEC, OpId, false, kUnpack, true>(s.grid, s.stream, batch, OpId());
+    return H2X_ERR_UNSUPPORTED;
 }
 
+// The audit the calling thread has opened with h2x_copy_audit_begin.
+thread_local Audit* t_audit = nullptr;
+
 } // namespace
+
+Audit* current_audit()
+{
+    return t_audit;
+}
 
 int launch_identity(const LaunchShape& s, const BoxBatch& batch)
 {
@@ -705,6 +700,9 @@ struct h2x_shuffle_plan
     // hold byte offsets where a launch from kernel arguments holds addresses.
     Box* table = nullptr;
     int table_device = -1;
+    // A plan made while a launch audit is open keeps the table on the host
+    // instead (no GPU call is made); it serves audited launches only.
+    std::vector<Box> host_table;
     int table_vec = 0;         // vector width the table's `ragged` flags were made for
     uint32_t most_blocks = 0;  // workgroups of the largest box at table_vec
     uint64_t total_blocks = 0; // over all boxes
@@ -739,6 +737,12 @@ int make_table(h2x_shuffle_plan* p)
         const uint64_t blocks = box_blocks(h.count, vec);
         p->most_blocks = std::max<uint64_t>(p->most_blocks, blocks);
         p->total_blocks += blocks;
+    }
+    if (current_audit())
+    {
+        p->host_table = host;
+        p->table_vec = vec;
+        return H2X_SUCCESS;
     }
     hipError_t err = hipGetDevice(&p->table_device);
     if (err == hipSuccess)
@@ -850,8 +854,9 @@ static bool shuffle_through_tables(const h2x_shuffle_plan* const* plans, void* c
                                    void* const* buffers, int num_plans, int mode,
                                    h2x_stream_t stream, int* status)
 {
+    const bool audited = current_audit() != nullptr;
     int device = -1;
-    if (hipGetDevice(&device) != hipSuccess)
+    if (!audited && hipGetDevice(&device) != hipSuccess)
         return false;
     const h2x_shuffle_plan* first = nullptr;
     uint32_t most = 0;
@@ -861,8 +866,8 @@ static bool shuffle_through_tables(const h2x_shuffle_plan* const* plans, void* c
         const h2x_shuffle_plan* p = plans[i];
         if (p->boxes.empty())
             continue;
-        if (!p->table || p->table_device != device
-            || reinterpret_cast<uintptr_t>(buffers[i]) % 16 != 0)
+        const bool has_table = audited ? !p->host_table.empty() : (p->table && p->table_device == device);
+        if (!has_table || reinterpret_cast<uintptr_t>(buffers[i]) % 16 != 0)
             return false;
         if (!first)
             first = p;
@@ -891,7 +896,7 @@ static bool shuffle_through_tables(const h2x_shuffle_plan* const* plans, void* c
             if (p->boxes.empty())
                 continue;
             PlanRef& ref = batch.plan[batch.num_plans++];
-            ref.table = p->table;
+            ref.table = audited ? p->host_table.data() : p->table;
             ref.tensor = static_cast<char*>(tensors[i]);
             ref.buffer = static_cast<char*>(buffers[i]);
             ref.first_box = batch.num_boxes;
@@ -979,4 +984,39 @@ extern "C" int h2x_shuffle_unpack_batched(const h2x_shuffle_plan* const* plans,
                                           int num_plans, h2x_stream_t stream)
 {
     return shuffle_batched(plans, tensors, const_cast<void* const*>(buffers), num_plans, kUnpack, stream);
+}
+
+// ---- launch audit ------------------------------------------------------------------
+
+extern "C" int h2x_copy_audit_begin(void)
+{
+    if (t_audit)
+        return H2X_ERR_INVALID_ARGUMENT;
+    t_audit = new (std::nothrow) Audit;
+    return t_audit ? static_cast<int>(H2X_SUCCESS) : static_cast<int>(hipErrorOutOfMemory);
+}
+
+extern "C" int h2x_copy_audit_add_region(const h2x_copy_audit_region* region)
+{
+    if (!t_audit || !region)
+        return H2X_ERR_INVALID_ARGUMENT;
+    t_audit->regions.push_back(AuditRegion{region->base, region->bytes, region->loads, region->stores});
+    return H2X_SUCCESS;
+}
+
+extern "C" int h2x_copy_audit_end(h2x_copy_audit_report* report)
+{
+    if (!t_audit)
+        return H2X_ERR_INVALID_ARGUMENT;
+    if (report)
+    {
+        report->launches = t_audit->launches;
+        report->workgroups = t_audit->workgroups;
+        report->outside_loads = t_audit->outside_loads;
+        report->outside_stores = t_audit->outside_stores;
+        report->misaligned = t_audit->misaligned;
+    }
+    delete t_audit;
+    t_audit = nullptr;
+    return H2X_SUCCESS;
 }

@@ -13,26 +13,13 @@ namespace
 template <typename T, int VEC, typename Op>
 int launch_op(const LaunchShape& s, const BoxBatch& batch)
 {
-    const dim3 grid(s.grid);
     if (s.mode == kUnpack)
-    {
-        if (s.sparse)
-            box_copy_kernel<T, VEC, Op, true, kUnpack, false><<<grid, kCopyBlock, 0, s.stream>>>(batch, Op());
-        else
-            box_copy_kernel<T, VEC, Op, false, kUnpack, false><<<grid, kCopyBlock, 0, s.stream>>>(batch, Op());
-    }
-    else if (s.mode == kTransfer)
-    {
-        if (s.sparse)
-            box_copy_kernel<T, VEC, Op, true, kTransfer, false><<<grid, kCopyBlock, 0, s.stream>>>(batch, Op());
-        else
-            box_copy_kernel<T, VEC, Op, false, kTransfer, false><<<grid, kCopyBlock, 0, s.stream>>>(batch, Op());
-    }
-    else
-    {
-        return H2X_ERR_UNSUPPORTED;
-    }
-    return launch_status();
+        return s.sparse ? run_box_copy<T, VEC, Op, true, kUnpack, false>(s.grid, s.stream, batch, Op())
+                        : run_box_copy<T, VEC, Op, false, kUnpack, false>(s.grid, s.stream, batch, Op());
+    if (s.mode == kTransfer)
+        return s.sparse ? run_box_copy<T, VEC, Op, true, kTransfer, false>(s.grid, s.stream, batch, Op())
+                        : run_box_copy<T, VEC, Op, false, kTransfer, false>(s.grid, s.stream, batch, Op());
+    return H2X_ERR_UNSUPPORTED;
 }
 
 template <typename T, int VEC>

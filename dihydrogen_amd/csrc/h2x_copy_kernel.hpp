@@ -19,6 +19,7 @@
 #include "h2x_device.hpp"
 
 #include <type_traits>
+#include <vector>
 
 namespace h2x
 {
@@ -627,6 +628,113 @@ __global__ __launch_bounds__(kCopyBlock, 8) void box_copy_kernel(
     const typename std::conditional<TABLE, TableBatch, BoxBatch>::type batch, Op op)
 {
     box_copy_body<T, VEC, Op, SPARSE, MODE, TABLE, DeviceMem>(batch, op, blockIdx.x, threadIdx.x, DeviceMem());
+}
+
+// ---- launch audit: the kernel body played on the CPU -----------------------------
+// While an audit is open on the calling thread (h2x_copy_audit_begin), the copy
+// entry points plan their launches as usual, and every launch is played on the
+// host instead of being issued: each workgroup and lane runs the body above with
+// an accessor that follows no pointer but counts, byte by byte, what would be
+// loaded and stored in the address ranges the caller registered, and what falls
+// outside them.  No GPU call is made.
+struct AuditRegion
+{
+    uint64_t base, bytes;
+    uint8_t* loads;  // per byte, saturating; may be null
+    uint8_t* stores;
+};
+
+struct Audit
+{
+    std::vector<AuditRegion> regions;
+    uint64_t launches = 0, workgroups = 0;
+    uint64_t outside_loads = 0, outside_stores = 0; // bytes outside every region
+    uint64_t misaligned = 0;                        // accesses not aligned as their instruction needs
+
+    void touch(const void* p, size_t bytes, size_t align, bool store)
+    {
+        const uint64_t at = reinterpret_cast<uintptr_t>(p);
+        if (at % align != 0)
+            ++misaligned;
+        for (const AuditRegion& r : regions)
+        {
+            if (at >= r.base && at + bytes <= r.base + r.bytes)
+            {
+                uint8_t* const count = store ? r.stores : r.loads;
+                if (count)
+                    for (size_t i = 0; i < bytes; ++i)
+                    {
+                        uint8_t& c = count[at - r.base + i];
+                        if (c < 255)
+                            ++c;
+                    }
+                return;
+            }
+        }
+        (store ? outside_stores : outside_loads) += bytes;
+    }
+};
+
+// The audit open on the calling thread, or null (h2x_copy.hip).
+Audit* current_audit();
+
+struct TraceMem
+{
+    Audit* audit;
+    template <int VEC, bool ALIGNED, typename T>
+    typename Words<T, VEC>::unaligned_t load(const T* p) const
+    {
+        audit->touch(p, sizeof(T) * VEC, ALIGNED ? sizeof(T) * VEC : sizeof(T), false);
+        typename Words<T, VEC>::unaligned_t v;
+        for (int j = 0; j < VEC; ++j)
+            v[j] = T(0);
+        return v;
+    }
+    template <int VEC, bool ALIGNED, typename T>
+    typename Words<T, VEC>::unaligned_t load_last_use(const T* p) const
+    {
+        return load<VEC, ALIGNED>(p);
+    }
+    template <int VEC, bool ALIGNED, typename T>
+    void store(T* p, typename Words<T, VEC>::unaligned_t) const
+    {
+        audit->touch(p, sizeof(T) * VEC, ALIGNED ? sizeof(T) * VEC : sizeof(T), true);
+    }
+    template <typename T>
+    T load1(const T* p) const
+    {
+        audit->touch(p, sizeof(T), sizeof(T), false);
+        return T(0);
+    }
+    template <typename T>
+    T load1_last_use(const T* p) const
+    {
+        return load1(p);
+    }
+    template <typename T>
+    void store1(T* p, T) const
+    {
+        audit->touch(p, sizeof(T), sizeof(T), true);
+    }
+};
+
+// Issues one launch of the kernel - or plays it for the audit.
+template <typename T, int VEC, typename Op, bool SPARSE, int MODE, bool TABLE>
+int run_box_copy(uint32_t grid, hipStream_t stream,
+                 const typename std::conditional<TABLE, TableBatch, BoxBatch>::type& batch, Op op)
+{
+    if (Audit* const audit = current_audit())
+    {
+        const TraceMem mem{audit};
+        for (uint32_t block = 0; block < grid; ++block)
+            for (uint32_t thread = 0; thread < kCopyBlock; ++thread)
+                box_copy_body<T, VEC, Op, SPARSE, MODE, TABLE, TraceMem>(batch, op, block, thread, mem);
+        ++audit->launches;
+        audit->workgroups += grid;
+        return H2X_SUCCESS;
+    }
+    box_copy_kernel<T, VEC, Op, SPARSE, MODE, TABLE><<<dim3(grid), kCopyBlock, 0, stream>>>(batch, op);
+    return launch_status();
 }
 
 #endif // __HIPCC__

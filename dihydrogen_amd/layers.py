@@ -24,6 +24,10 @@ def _device_buffer(count: int, dtype, device="cuda", zero: bool = False) -> torc
 
 
 def _stream_handle(stream: Optional[torch.cuda.Stream]) -> ctypes.c_void_p:
+    if stream is None and not torch.cuda.is_available():
+        # no GPU: the null stream; every launch then fails with HIP's own error.  (Launch audits,
+        # which play the kernels' indexing on the CPU, ignore the stream.)
+        return ctypes.c_void_p(0)
     s = torch.cuda.current_stream() if stream is None else stream
     return ctypes.c_void_p(s.cuda_stream)
 

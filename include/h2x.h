@@ -567,6 +567,47 @@ int h2x_bn_audit_clearing(int backward,
                           const uint64_t* address,
                           h2x_bn_audit_report* report);
 
+/**
+ * Launch audit of the copy entry points (halo pack / unpack / clear / fused
+ * exchange, shuffle plans, pack and unpack), on the host: no GPU call is made
+ * and no pointer is followed.  No counterpart in the reference.  Between
+ * h2x_copy_audit_begin and h2x_copy_audit_end the calling thread's calls to
+ * those entry points plan their launches as usual, and every launch is played
+ * on the CPU, workgroup by workgroup and lane by lane, through the code of the
+ * kernel itself with memory accesses counted instead of made.  The caller
+ * registers the address ranges of its tensors and buffers (any addresses: real
+ * host allocations serve as well as imaginary ones) and, per
+ * range, two arrays of one counter per byte: `loads[i]` / `stores[i]` say how
+ * often byte base + i would be loaded / stored (saturating at 255; either may
+ * be null).  What falls outside every range is counted in the report
+ * (`outside_loads`, `outside_stores`, in bytes: must be 0), as are accesses not
+ * aligned as their instruction needs (`misaligned`: must be 0).  A shuffle plan
+ * made while an audit is open serves audited launches only; destroy it as any
+ * other.  Cost: proportional to the elements moved; meant for tests on machines
+ * without a GPU.  The stream argument of the audited calls is ignored.
+ */
+typedef struct h2x_copy_audit_region
+{
+    uint64_t base;
+    uint64_t bytes;
+    uint8_t* loads;
+    uint8_t* stores;
+} h2x_copy_audit_region;
+
+typedef struct h2x_copy_audit_report
+{
+    uint64_t launches;
+    uint64_t workgroups;
+    uint64_t outside_loads, outside_stores; /* bytes */
+    uint64_t misaligned;                    /* accesses */
+} h2x_copy_audit_report;
+
+int h2x_copy_audit_begin(void);
+/** Registers one address range with the open audit (the counter arrays must outlive it). */
+int h2x_copy_audit_add_region(const h2x_copy_audit_region* region);
+/** Closes the audit of the calling thread and reports (report may be null). */
+int h2x_copy_audit_end(h2x_copy_audit_report* report);
+
 /* ------------------------------------------------------------------------ */
 /* Elementwise transforms and sums over dimensions                           */
 /* ------------------------------------------------------------------------ */

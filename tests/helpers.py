@@ -203,3 +203,63 @@ def check_guards(allocated):
         back = int((raw[-guard_bytes:] != GUARD_BYTE).sum())
         assert front == 0 and back == 0, \
             f"a kernel wrote outside a tensor of real shape (or a buffer of size) {shape}: {front} bytes in front, {back} behind"
+
+
+class CopyAudit:
+    """A launch audit of the copy entry points (h2x_copy_audit_begin ... _end) around host-layer
+    code that runs on CPU tensors: every tensor registered here, and every buffer the layers
+    allocate while the audit is open, gets one load and one store counter per byte."""
+
+    def __init__(self):
+        self.entries = []     # (torch tensor, loads, stores, region struct): kept alive until the end
+        self.report = None
+
+    def __enter__(self):
+        from dihydrogen_amd import capi, layers
+        self._lib = capi.load()
+        capi.check(self._lib.h2x_copy_audit_begin(), "audit begin")
+        self._layers, self._original = layers, layers._device_buffer
+
+        def device_buffer(count, dtype, device="cuda", zero=False):
+            import torch
+            t = torch.zeros(count, dtype=dtype, device="cpu")
+            self.register(t)
+            self.buffers.append(t)
+            return t
+
+        self.buffers = []
+        layers._device_buffer = device_buffer
+        return self
+
+    def register(self, t):
+        import ctypes
+        from dihydrogen_amd import capi
+        nbytes = t.numel() * t.element_size()
+        loads, stores = np.zeros(nbytes, np.uint8), np.zeros(nbytes, np.uint8)
+        region = capi.CopyAuditRegion()
+        region.base, region.bytes = t.data_ptr(), nbytes
+        region.loads = loads.ctypes.data_as(ctypes.POINTER(ctypes.c_uint8))
+        region.stores = stores.ctypes.data_as(ctypes.POINTER(ctypes.c_uint8))
+        capi.check(self._lib.h2x_copy_audit_add_region(ctypes.byref(region)), "audit region")
+        self.entries.append((t, loads, stores, region))
+
+    def counts(self, t):
+        """(loads, stores) per element of a registered tensor; all bytes of an element move together."""
+        for u, loads, stores, _ in self.entries:
+            if u.data_ptr() == t.data_ptr():
+                e = u.element_size()
+                out = []
+                for c in (loads, stores):
+                    per = c.reshape(-1, e)
+                    assert (per == per[:, :1]).all(), "bytes of one element were moved separately"
+                    out.append(per[:, 0].astype(np.int64))
+                return out
+        raise KeyError("tensor not registered")
+
+    def __exit__(self, *exc):
+        import ctypes
+        from dihydrogen_amd import capi
+        self._layers._device_buffer = self._original
+        self.report = capi.CopyAuditReport()
+        capi.check(self._lib.h2x_copy_audit_end(ctypes.byref(self.report)), "audit end")
+        return False
