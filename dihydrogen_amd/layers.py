@@ -23,13 +23,20 @@ def _device_buffer(count: int, dtype, device="cuda", zero: bool = False) -> torc
 
 
 
+_has_gpu: Optional[bool] = None
+
+
 def _stream_handle(stream: Optional[torch.cuda.Stream]) -> ctypes.c_void_p:
-    if stream is None and not torch.cuda.is_available():
-        # no GPU: the null stream; every launch then fails with HIP's own error.  (Launch audits,
-        # which play the kernels' indexing on the CPU, ignore the stream.)
-        return ctypes.c_void_p(0)
-    s = torch.cuda.current_stream() if stream is None else stream
-    return ctypes.c_void_p(s.cuda_stream)
+    global _has_gpu
+    if stream is None:
+        if _has_gpu is None:
+            _has_gpu = torch.cuda.is_available()  # asked once: the answer does not change
+        if not _has_gpu:
+            # no GPU: the null stream; every launch then fails with HIP's own error.  (Launch
+            # audits, which play the kernels' indexing on the CPU, ignore the stream.)
+            return ctypes.c_void_p(0)
+        stream = torch.cuda.current_stream()
+    return ctypes.c_void_p(stream.cuda_stream)
 
 
 def _ptr(t) -> ctypes.c_void_p:
