@@ -249,3 +249,45 @@ def test_an_access_outside_the_registered_ranges_is_reported():
     assert audit.report.outside_stores > 0 and audit.report.outside_loads == 0
     # calls outside an audit are not affected: without a GPU they fail with HIP's error, with one they run
     assert lib.h2x_copy_audit_end(None) == -1
+
+
+def test_random_halo_and_shuffle_geometries():
+    """Seeded random decompositions (the generators of the GPU suite, other seeds): forward and reverse
+    exchanges and shuffles in both directions touch what their definition says, and nothing else."""
+    import torch
+    import test_gpu_random_shapes as shapes
+    from dihydrogen_amd.layers import HaloExchangeAccumOp, HaloExchangeVirtual, TensorShufflerVirtual
+    from dihydrogen_amd.tensor import Distribution, LocaleVirtual, Tensor
+    for (shape, locale, overlap, periodic, fused), reverse in itertools.product(shapes._halo_cases(60, 731), (False, True)):
+        with CopyAudit() as audit:
+            ts = _tensors(shape, locale, overlap, torch.float32, audit)
+            xch = HaloExchangeVirtual(ts, periodic=periodic)
+            xch.exchange(is_reverse=reverse, op=HaloExchangeAccumOp.SUM if reverse else HaloExchangeAccumOp.ID,
+                         fused=fused)
+            packed, unpacked = _expected_exchange(xch, reverse=reverse)
+        what = (shape, locale, overlap, periodic, fused, reverse)
+        assert (audit.report.outside_loads, audit.report.outside_stores, audit.report.misaligned) == (0, 0, 0), what
+        for t, p, u in zip(ts, packed, unpacked):
+            loads, stores = audit.counts(t.data)
+            assert np.array_equal(loads, p + u if reverse else p) and np.array_equal(stores, u), what
+    for (shape, (sl, ss, so), (dl, ds, do)), forward in itertools.product(shapes._shuffle_cases(40, 732), (True, False)):
+        if ss is not None or ds is not None:
+            continue
+        n = int(np.prod(sl))
+        with CopyAudit() as audit:
+            src = [Tensor(shape, LocaleVirtual(r, n), Distribution(sl, ss, so), device="cpu").allocate() for r in range(n)]
+            dst = [Tensor(shape, LocaleVirtual(r, n), Distribution(dl, ds, do), device="cpu").allocate() for r in range(n)]
+            for t in src + dst:
+                audit.register(t.data)
+            sh = TensorShufflerVirtual(src, dst)
+            (sh.shuffle_forward if forward else sh.shuffle_backward)()
+            del sh
+        what = (shape, sl, so, dl, do, forward)
+        assert (audit.report.outside_loads, audit.report.outside_stores, audit.report.misaligned) == (0, 0, 0), what
+        read = src if forward else dst
+        for t in src + dst:
+            interior = np.zeros(t.local_real_shape[::-1], np.int64)
+            interior[tuple(slice(o, o + l) for o, l in zip(reversed(t.overlap), reversed(t.local_shape)))] = 1
+            loads, stores = audit.counts(t.data)
+            moved, other = (loads, stores) if any(t is r for r in read) else (stores, loads)
+            assert not other.any() and (np.array_equal(moved, interior.ravel()) if interior.size else not moved.any()), what
