@@ -291,3 +291,42 @@ def test_random_halo_and_shuffle_geometries():
             loads, stores = audit.counts(t.data)
             moved, other = (loads, stores) if any(t is r for r in read) else (stores, loads)
             assert not other.any() and (np.array_equal(moved, interior.ravel()) if interior.size else not moved.any()), what
+
+
+def test_strips_of_a_tensor_beyond_2_to_the_32_elements():
+    """Offsets that need 64 bits: the far strips of an (imaginary) tensor of 4.85 billion elements.  The
+    outermost strip is contiguous, so its own byte range is registered with counters and everything else
+    counts as outside; the strided strip of dimension 1 is checked against the bounds of the tensor."""
+    import ctypes
+    import torch
+    from dihydrogen_amd import capi
+    lib = capi.load()
+    real = (2100, 2100, 1100, 1, 1)
+    total = int(np.prod(real))
+    assert total > 2 ** 32
+    base = 1 << 44                     # never followed
+    for dim, is_pack in itertools.product((2, 1), (1, 0)):
+        n = lib.h2x_halo_size(5, capi.i64_array(real), dim, 1)
+        buffer = torch.zeros(n, dtype=torch.float32)
+        with CopyAudit() as audit:
+            audit.register(buffer)
+            region = capi.CopyAuditRegion()
+            if dim == 2:
+                # RHS strip, inner when packing: plane 1098 (1099 is the halo), outer when unpacking: plane 1099
+                plane = 1098 if is_pack else 1099
+                loads = np.zeros(n * 4, np.uint8)
+                stores = np.zeros(n * 4, np.uint8)
+                region.base, region.bytes = base + plane * 2100 * 2100 * 4, n * 4
+                region.loads = loads.ctypes.data_as(ctypes.POINTER(ctypes.c_uint8))
+                region.stores = stores.ctypes.data_as(ctypes.POINTER(ctypes.c_uint8))
+            else:
+                region.base, region.bytes = base, total * 4      # bounds only
+            capi.check(lib.h2x_copy_audit_add_region(ctypes.byref(region)), "region")
+            capi.check(lib.h2x_halo_pack_or_unpack(capi.F32, ctypes.c_void_p(base), 5, capi.i64_array(real), dim, 1, 1,
+                                                   ctypes.c_void_p(buffer.data_ptr()), is_pack, 0, 0,
+                                                   ctypes.c_void_p(0)), "pack_or_unpack")
+        _clean(audit.report)
+        b_loads, b_stores = audit.counts(buffer)
+        assert ((b_stores if is_pack else b_loads) == 1).all() and not (b_loads if is_pack else b_stores).any()
+        if dim == 2:
+            assert ((loads if is_pack else stores) == 1).all() and not (stores if is_pack else loads).any()
