@@ -114,10 +114,22 @@ int static_scratch(void** out)
 }
 
 constexpr int kUnroll = 4;
-// Workgroups a reduction aims at over all channels (bounds the workspace) and
-// workgroups an elementwise pass aims at; both from a sweep on MI355X.
+// Workgroups a reduction aims at over all channels (bounds the workspace); from
+// a sweep on MI355X.
 constexpr int kTargetGroups = 4096;
+// Elementwise passes aim at 16384 workgroups (from a sweep on MI355X at the
+// headline shapes) - except on haloed tensors and on tensors beyond the
+// memory-side cache, where a workgroup gets two passes of its 256 lanes (8 KB
+// of fp32 per tensor) however large the tensor is.  Measured against the
+// budget of 16384: normalise on the haloed C3 shard 158 -> 145 us, input
+// gradient 240 -> 222 us; dense tensors of 1 GB 571 -> 529 us and 896 -> 836
+// us, of 537 MB 279 -> 267 us and 443 -> 423 us.  Dense tensors that the cache
+// holds lose with the small chunks (268 MB: input gradient 191 -> 194 us, the
+// benchmark step 676 -> 680 us; N 64 x 256 x 56 x 56: 150 -> 161 us) and keep
+// the budget.
 constexpr int kElementwiseBlocks = 16384;
+constexpr int kUnboundedBlocks = 1 << 30;
+constexpr size_t kBeyondCacheBytes = size_t(384) << 20;
 constexpr int kMinGroupsPerChannel = 8;
 constexpr int kMaxGroupsPerChannel = 2048;
 constexpr int kMaxSums = 4;
@@ -1880,11 +1892,12 @@ int statistics_impl(int num_channels, size_t num_per_sum, double decay, void* me
 
 // Chunking of an elementwise pass over N*C segments: at least one full vector
 // per thread, about kElementwiseBlocks workgroups.
-Chunking elementwise_chunking(size_t spatial, size_t segments, int vw, int unroll)
+Chunking elementwise_chunking(size_t spatial, size_t segments, int vw, int unroll,
+                              int budget = kElementwiseBlocks)
 {
     const size_t tile = static_cast<size_t>(kBlockSize) * vw * unroll;
     const size_t one_pass = static_cast<size_t>(kBlockSize) * vw;
-    Chunking c = make_chunking(spatial, segments, kElementwiseBlocks, one_pass,
+    Chunking c = make_chunking(spatial, segments, budget, one_pass,
                                one_pass * 2 > tile ? one_pass : one_pass * 2);
     // A chunk of more than a tile is cut down to whole tiles: the passes beyond the
     // last whole tile run with one load in flight per lane instead of `unroll`
@@ -1945,7 +1958,9 @@ int apply_impl(int num_samples, int num_channels, size_t spatial, const HostTens
         spatial = pad_rows<T>({&tx, &ty}, spatial);
     if (spatial >= (1ull << 31) && strided)
         return H2X_ERR_TOO_LARGE;
-    const Chunking ch = elementwise_chunking(spatial, segments, vw, kUnroll);
+    const bool beyond_cache = segments * spatial * sizeof(T) > kBeyondCacheBytes;
+    const Chunking ch = elementwise_chunking(spatial, segments, vw, kUnroll,
+                                             strided || beyond_cache ? kUnboundedBlocks : kElementwiseBlocks);
     const size_t workgroups = segments * ch.chunks_per_seg;
     if (!grid_ok(workgroups))
         return H2X_ERR_TOO_LARGE;
@@ -2127,7 +2142,9 @@ int backprop2_impl(int num_samples, int num_channels, size_t spatial, size_t num
         spatial = pad_rows<T>({&tx, &td, &to}, spatial);
     if (spatial >= (1ull << 31) && strided)
         return H2X_ERR_TOO_LARGE;
-    const Chunking ch = elementwise_chunking(spatial, segments, vw, kUnroll / 2);
+    const bool beyond_cache = segments * spatial * sizeof(T) > kBeyondCacheBytes;
+    const Chunking ch = elementwise_chunking(spatial, segments, vw, kUnroll / 2,
+                                             strided || beyond_cache ? kUnboundedBlocks : kElementwiseBlocks);
     const size_t workgroups = segments * ch.chunks_per_seg;
     if (!grid_ok(workgroups))
         return H2X_ERR_TOO_LARGE;
