@@ -566,23 +566,23 @@ def cpu_baseline(repeats: int = 5):
 # label -> (bytes read, bytes written) per launch
 PMC_TRAFFIC = {
     "bn_sums": (268455424, 131072),
-    "bn_apply": (268462080, 268474368),
-    "bn_backprop1": (536913280, 131072),
+    "bn_apply": (268462080, 268488832),
+    "bn_backprop1": (536912896, 131072),
     "bn_backprop2": (536906240, 268435456),
-    "halo_dim0_pack": (151162432, 8652800),    # 4 faces (2 ranks) a launch, four launches a step
-    "halo_dim0_unpack": (9218080, 43264000),
-    "halo_dim1_pack": (42624832, 34611200),
-    "halo_dim1_unpack": (34630528, 36217152),
+    "halo_dim0_pack": (150761152, 8652800),    # 4 faces (2 ranks) a launch, four launches a step
+    "halo_dim0_unpack": (9218192, 43264000),
+    "halo_dim1_pack": (42624640, 34611200),
+    "halo_dim1_unpack": (34630400, 36218784),
     "halo_dim2_pack": (34694400, 34611200),
-    "halo_dim2_unpack": (34630400, 34619520),
+    "halo_dim2_unpack": (34630400, 34619392),
 }
 # steps of the timed region whose dominant-kernel launches are bracketed by events: every EVENT_EVERY-th
 EVENT_EVERY = 4
 
 # sha256 (first 16 hex digits) of the kernel sources the table was measured with, see
 # kernel_sources_sha(); with other sources the traffic fields are omitted
-PMC_SOURCES_SHA = "5d42d3729f694129"
-PMC_COMMIT = "b96dc97"
+PMC_SOURCES_SHA = "5a239d5c230b60a7"
+PMC_COMMIT = "19208a7"
 
 KERNEL_OF = {
     "bn_sums": "bn_sums_kernel<float,4> (+bn_finish_kernel<float,2>)",
