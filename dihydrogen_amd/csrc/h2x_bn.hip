@@ -114,9 +114,13 @@ int static_scratch(void** out)
 }
 
 constexpr int kUnroll = 4;
-// Workgroups a reduction aims at over all channels (bounds the workspace); from
-// a sweep on MI355X.
-constexpr int kTargetGroups = 4096;
+// Workgroups a reduction aims at over all channels, from sweeps on MI355X: 4096
+// on dense tensors, 16384 on haloed ones (the haloed C3 shard: two-launch
+// forward 141 -> 134 us, backward 217 -> 211 us; dense shapes are the same or
+// up to 4 % slower with more).  The workspace holds partial sums for the larger
+// number.
+constexpr int kTargetGroups = 16384;
+constexpr int kDenseTargetGroups = 4096;
 // Elementwise passes aim at 16384 workgroups (from a sweep on MI355X at the
 // headline shapes) - except on haloed tensors and on tensors beyond the
 // memory-side cache, where a workgroup gets two passes of its 256 lanes (8 KB
@@ -134,10 +138,24 @@ constexpr int kMinGroupsPerChannel = 8;
 constexpr int kMaxGroupsPerChannel = 2048;
 constexpr int kMaxSums = 4;
 
+int groups_per_channel(int num_channels, int target)
+{
+    const int g = (target + num_channels - 1) / std::max(num_channels, 1);
+    return std::min(std::max(g, kMinGroupsPerChannel), kMaxGroupsPerChannel);
+}
+
+// Partial sums the workspace holds per channel and sum: the stride of the
+// partials of a channel, and the most groups any launch uses.
 int max_groups_per_channel(int num_channels)
 {
-    const int g = (kTargetGroups + num_channels - 1) / std::max(num_channels, 1);
-    return std::min(std::max(g, kMinGroupsPerChannel), kMaxGroupsPerChannel);
+    return groups_per_channel(num_channels, kTargetGroups);
+}
+
+// Groups a long-segment reduction cuts a channel into.
+int reduction_groups_per_channel(int num_channels, bool strided)
+{
+    return strided ? max_groups_per_channel(num_channels)
+                   : groups_per_channel(num_channels, kDenseTargetGroups);
 }
 
 size_t partials_bytes(int num_channels)
@@ -1848,12 +1866,13 @@ int sums_impl(int num_samples, int num_channels, size_t spatial, const HostTenso
     if (spatial >= (1ull << 31) && strided)
         return H2X_ERR_TOO_LARGE;
     const int gmax = max_groups_per_channel(num_channels);
+    const int budget = reduction_groups_per_channel(num_channels, strided);
     const size_t tile = static_cast<size_t>(kBlockSize) * vw * kUnroll;
-    const Chunking ch = make_chunking(spatial, num_samples, gmax, tile, tile);
+    const Chunking ch = make_chunking(spatial, num_samples, budget, tile, tile);
     const size_t units = static_cast<size_t>(ch.chunks_per_seg) * num_samples;
     if (units > 0xffffffffull || num_channels > 65535)
         return H2X_ERR_TOO_LARGE;
-    const size_t groups = std::min<size_t>(units, gmax);
+    const size_t groups = std::min<size_t>(units, budget);
     double* partials = static_cast<double*>(workspace);
     const dim3 grid(static_cast<unsigned int>(groups), num_channels);
     LaunchRecord rec = long_record(kKernelSums, strided, vw, grid, num_samples, num_channels,
@@ -2046,12 +2065,13 @@ int backprop1_impl(int num_samples, int num_channels, size_t spatial, const Host
     if (spatial >= (1ull << 31) && strided)
         return H2X_ERR_TOO_LARGE;
     const int gmax = max_groups_per_channel(num_channels);
+    const int budget = reduction_groups_per_channel(num_channels, strided);
     const size_t tile = static_cast<size_t>(kBlockSize) * vw * (kUnroll / 2);
-    const Chunking ch = make_chunking(spatial, num_samples, gmax, tile, tile);
+    const Chunking ch = make_chunking(spatial, num_samples, budget, tile, tile);
     const size_t units = static_cast<size_t>(ch.chunks_per_seg) * num_samples;
     if (units > 0xffffffffull || num_channels > 65535)
         return H2X_ERR_TOO_LARGE;
-    const size_t groups = std::min<size_t>(units, gmax);
+    const size_t groups = std::min<size_t>(units, budget);
     double* partials = static_cast<double*>(workspace);
     const dim3 grid(static_cast<unsigned int>(groups), num_channels);
     LaunchRecord rec = long_record(kKernelBackprop1, strided, vw, grid, num_samples, num_channels,
