@@ -566,13 +566,13 @@ def cpu_baseline(repeats: int = 5):
 # label -> (bytes read, bytes written) per launch
 PMC_TRAFFIC = {
     "bn_sums": (268455424, 131072),
-    "bn_apply": (268461824, 268487936),
-    "bn_backprop1": (536913024, 131072),
+    "bn_apply": (268462080, 268468224),
+    "bn_backprop1": (536912576, 131104),
     "bn_backprop2": (536906240, 268435456),
-    "halo_dim0_pack": (150589264, 8652800),    # 4 faces (2 ranks) a launch, four launches a step
-    "halo_dim0_unpack": (9217904, 43264000),
-    "halo_dim1_pack": (42624768, 34611200),
-    "halo_dim1_unpack": (34630400, 36220544),
+    "halo_dim0_pack": (150615792, 8652800),    # 4 faces (2 ranks) a launch, four launches a step
+    "halo_dim0_unpack": (9218176, 43264000),
+    "halo_dim1_pack": (42624704, 34611200),
+    "halo_dim1_unpack": (34630400, 36218592),
     "halo_dim2_pack": (34694400, 34611200),
     "halo_dim2_unpack": (34630400, 34619392),
 }
@@ -581,8 +581,8 @@ EVENT_EVERY = 4
 
 # sha256 (first 16 hex digits) of the kernel sources the table was measured with, see
 # kernel_sources_sha(); with other sources the traffic fields are omitted
-PMC_SOURCES_SHA = "985887b976bee0d8"
-PMC_COMMIT = "2497a9b"
+PMC_SOURCES_SHA = "3bcdabae02179b5c"
+PMC_COMMIT = "3387492"
 
 KERNEL_OF = {
     "bn_sums": "bn_sums_kernel<float,4> (+bn_finish_kernel<float,2>)",

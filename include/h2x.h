@@ -447,8 +447,9 @@ typedef struct h2x_haloed_geometry
  * feeds a convolution can hand over its output with the halo already cleared.
  * The kernels walk the whole allocation in aligned vectors, so the 8-byte gaps
  * between interior rows cost no partial writes (a shard of NCDHW 4 x 64 x 64^3
- * with a halo of 1: forward + backward at 0.76-0.78 of the HBM peak against
- * 0.73-0.74 with the halo left alone).  The pointers are the starts of the allocations
+ * with a halo of 1: forward + backward at 0.76-0.78 of the HBM peak, the rate
+ * of the calls that leave the halo alone, without the clear_halo launches that
+ * would follow them).  The pointers are the starts of the allocations
  * (Tensor::get_buffer()), not of the interiors.  Halo cells of the inputs are
  * read and ignored; dx_buffer may be x_buffer.  Falls back to single elements
  * when a segment of the real tensor is no multiple of 16 bytes long or a
